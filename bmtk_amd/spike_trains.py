@@ -1,0 +1,245 @@
+"""Input spike sources for the GPU path.
+
+``PoissonSpikeGenerator`` follows the sampling scheme, random stream and units
+of bmtk/utils/reports/spike_trains/spike_trains.py:113-251 (exponential
+inter-spike intervals on NumPy's global legacy generator, optional refractory
+thinning, linear-interpolated rate thinning for time-varying rates), so a
+seeded run produces the trains bmtk would write to ``inputs/*.h5``.
+``bin_spike_times`` applies the rules NEST's ``spike_generator`` enforces when
+bmtk hands it those trains (bmtk/simulator/pointnet/pointnetwork.py:39-61) and
+turns them into the per-step event lists the kernels consume.
+"""
+import numpy as np
+
+
+def _refractory_rate_correction(abs_ref, tau_ref):
+    """Rate lost to refractoriness and the polynomial that inverts it
+    (bmtk/utils/reports/spike_trains/spike_trains.py:317-338)."""
+    before = np.logspace(0, 3, 40)
+    if tau_ref != 0:
+        after = (np.exp(-before * abs_ref)
+                 - before * np.exp(abs_ref / tau_ref) * tau_ref / (before * tau_ref + 1)
+                 * np.exp(-(before + 1 / tau_ref) * abs_ref)) * before
+    else:
+        after = np.exp(-before * abs_ref) * before
+    top = int(np.argmax(after))
+    inverse = np.poly1d(np.polyfit(after[:top], before[:top], 10))
+    return float(np.max(after)), inverse
+
+
+class PoissonSpikeGenerator(object):
+    """Homogeneous / inhomogeneous Poisson spike trains (times stored in ms)."""
+
+    def __init__(self, population=None, seed=None, output_units="ms", **kwargs):
+        self.default_population = kwargs.get("default_population", population)
+        if seed:  # a seed of 0 / 0.0 / None leaves the global stream where it is, as the reference does
+            np.random.seed(seed)
+        units = output_units.lower()
+        if units in ("ms", "millisecond", "milliseconds"):
+            self.units, self.output_conversion = "ms", 1000.0
+        elif units in ("s", "second", "seconds"):
+            self.units, self.output_conversion = "s", 1.0
+        else:
+            raise AttributeError("Unknown output_units value {}".format(output_units))
+        self._trains = {}  # population -> {node_id: [chunks of times]}
+
+    # -- container ---------------------------------------------------------
+    def add_spikes(self, node_ids, timestamps, population=None):
+        pop = population if population is not None else self.default_population
+        store = self._trains.setdefault(pop, {})
+        timestamps = np.atleast_1d(np.asarray(timestamps, np.float64))
+        if np.isscalar(node_ids):
+            store.setdefault(int(node_ids), []).append(timestamps)
+        else:
+            for nid, ts in zip(node_ids, timestamps):
+                store.setdefault(int(nid), []).append(np.atleast_1d(ts))
+
+    @property
+    def populations(self):
+        return list(self._trains.keys())
+
+    def _pop(self, population):
+        return population if population is not None else self.default_population
+
+    def node_ids(self, population=None):
+        return sorted(self._trains.get(self._pop(population), {}).keys())
+
+    def get_times(self, node_id, population=None, time_window=None):
+        chunks = self._trains.get(self._pop(population), {}).get(int(node_id), [])
+        ts = np.concatenate(chunks) if chunks else np.zeros(0)
+        if time_window is not None:
+            ts = ts[(ts >= time_window[0]) & (ts <= time_window[1])]
+        return ts
+
+    def n_spikes(self, population=None):
+        pops = [population] if population is not None else self.populations
+        return int(sum(sum(c.size for c in chunks) for p in pops for chunks in self._trains.get(p, {}).values()))
+
+    def time_range(self, population=None):
+        pops = [population] if population is not None else self.populations
+        ts = np.concatenate([self.get_times(n, p) for p in pops for n in self.node_ids(p)])
+        return float(np.min(ts)), float(np.max(ts))
+
+    def to_dataframe(self, populations=None, with_population_col=True):
+        import pandas as pd
+        pops = self.populations if populations is None else np.atleast_1d(populations).tolist()
+        rows_t, rows_p, rows_n = [], [], []
+        for p in pops:
+            for n in self.node_ids(p):
+                t = self.get_times(n, p)
+                rows_t.append(t)
+                rows_n.append(np.full(t.size, n, np.uint64))
+                rows_p.extend([p] * t.size)
+        df = pd.DataFrame({"timestamps": np.concatenate(rows_t) if rows_t else [],
+                           "population": rows_p, "node_ids": np.concatenate(rows_n) if rows_n else []})
+        return df if with_population_col else df.drop(columns="population")
+
+    # -- generators --------------------------------------------------------
+    def add(self, node_ids, firing_rate, population=None, times=(0.0, 1.0), abs_ref=0, tau_ref=0):
+        """``firing_rate`` in Hz (scalar, or an array paired with ``times``), ``times`` in seconds."""
+        if tau_ref < 0:
+            raise ValueError("Refractory period time constant (sec) cannot be negative.")
+        if abs_ref < 0:
+            raise ValueError("Absolute refractory period (sec) cannot be negative.")
+        if np.isscalar(node_ids):
+            node_ids = [node_ids]
+        if np.isscalar(firing_rate):
+            self._fixed_rate(node_ids, population, firing_rate, times, abs_ref, tau_ref)
+        elif isinstance(firing_rate, (list, np.ndarray)):
+            self._varying_rate(node_ids, population, np.asarray(firing_rate, np.float64), np.asarray(times),
+                               abs_ref, tau_ref)
+
+    def _fixed_rate(self, node_ids, population, fr, times, abs_ref, tau_ref):
+        if np.isscalar(times) and times > 0.0:
+            tstart, tstop = 0.0, times
+        else:
+            tstart, tstop = times[0], times[-1]
+            if tstart >= tstop:
+                raise ValueError("Invalid start and stop times.")
+        if fr < 0:
+            raise ValueError("Firing rates must not be negative.")
+        if abs_ref != 0 or tau_ref != 0:
+            limit, inverse = _refractory_rate_correction(abs_ref, tau_ref)
+            if fr > limit:
+                raise ValueError("Cannot achieve firing rate above {} with these absolute and relative "
+                                 "refractory properties.".format(limit))
+            fr = inverse(fr)
+            self._fixed_rate_refractory(node_ids, population, fr, tstart, tstop, abs_ref, tau_ref)
+            return
+        # No refractoriness: one uniform draw per candidate spike, the draw that
+        # crosses tstop is consumed too.  Draw in blocks for speed, then put the
+        # global stream exactly where a draw-by-draw loop would have left it.
+        state0 = np.random.get_state()
+        block = max(1024, int((tstop - tstart) * fr * 1.2) + 16)
+        buf, pos, used = np.zeros(0), 0, 0
+        for nid in node_ids:
+            c_time, pieces = tstart, []
+            while True:
+                if pos == buf.size:
+                    buf, pos = -np.log(1.0 - np.random.uniform(size=block)) / fr, 0
+                acc = np.cumsum(np.concatenate(([c_time], buf[pos:])))[1:]  # sequential adds, as a scalar loop does
+                k = int(np.searchsorted(acc, tstop, side="right"))           # first acc > tstop
+                pieces.append(acc[:k])
+                if k < acc.size:
+                    pos += k + 1
+                    used += k + 1
+                    break
+                used += acc.size
+                pos = buf.size
+                c_time = acc[-1]
+            self.add_spikes(nid, np.concatenate(pieces) * self.output_conversion, population)
+        np.random.set_state(state0)
+        if used:
+            np.random.uniform(size=used)
+
+    def _fixed_rate_refractory(self, node_ids, population, fr, tstart, tstop, abs_ref, tau_ref):
+        for nid in node_ids:
+            c_time, out = tstart, []
+            while True:
+                interval = -np.log(1.0 - np.random.uniform()) / fr
+                c_time += interval
+                if c_time > tstop:
+                    break
+                w = 1 - np.exp(-(interval - abs_ref) / tau_ref) if tau_ref != 0 else 1
+                if abs_ref != 0:
+                    w = w * (interval > abs_ref)
+                if w == 1 or np.random.uniform() < w:
+                    out.append(c_time * self.output_conversion)
+            self.add_spikes(nid, np.asarray(out), population)
+
+    def _varying_rate(self, node_ids, population, fr, times, abs_ref, tau_ref):
+        if np.min(fr) < 0:
+            raise ValueError("Firing rates must not be negative")
+        if len(fr) != len(times):
+            raise ValueError("If using a time series for firing rate, times must be an array of equal length")
+        max_fr = np.max(fr)
+        limit, inverse = _refractory_rate_correction(abs_ref, tau_ref)
+        if max_fr > limit:
+            raise ValueError("Cannot achieve firing rate above {} with these absolute and relative "
+                             "refractory properties".format(limit))
+        fr = inverse(fr)
+        tstart, tstop = times[0], times[-1]
+        for nid in node_ids:
+            c_time, idx, out = tstart, 0, []
+            while True:
+                interval = -np.log(1.0 - np.random.uniform()) / max_fr
+                c_time += interval
+                if c_time > tstop:
+                    break
+                w = 1 - np.exp(-(interval - abs_ref) / tau_ref) if tau_ref != 0 else 1
+                if abs_ref != 0:
+                    w = w * (interval > abs_ref)
+                while times[idx] <= c_time:
+                    idx += 1
+                t0, t1, f0, f1 = times[idx - 1], times[idx], fr[idx - 1], fr[idx]
+                fr_i = f0 + (f1 - f0) * (c_time - t0) / (t1 - t0)
+                if not fr_i / max_fr * w < np.random.uniform():
+                    out.append(c_time * self.output_conversion)
+            self.add_spikes(nid, np.asarray(out), population)
+
+
+def check_spike_times(st):
+    """The rule bmtk applies before ``nest.SetStatus(.., {'spike_times': ..})``
+    (bmtk/simulator/pointnet/pointnetwork.py:39-61): empty/None trains are
+    skipped, times must be strictly positive, and they are sorted."""
+    if st is None or len(st) == 0:
+        return None
+    st = np.array(st, np.float64)
+    if np.any(st <= 0.0):
+        raise ValueError("spike train {} contains negative/zero time, unable to run virtual cell".format(st))
+    st.sort()
+    return st
+
+
+def bin_spike_times(trains, dt, n_steps, batch=1, trial=0, precise_times=True):
+    """Per-source spike times (ms) -> (in_ptr int64[n_steps+1], in_events int32[]).
+
+    ``trains`` is a sequence indexed by source id (entries may be None).  A
+    spike at time t gets the stamp ``round(t/dt)`` steps (NEST ``spike_generator``
+    with on-grid delivery; ``precise_times`` only keeps the sub-step offset,
+    which ``static_synapse`` delivery ignores) and is emitted in step stamp-1.
+    An event is the element id ``source*batch + trial``; events of one step are
+    ascending.  Stamps of 0 (times below dt/2) cannot be emitted and raise, as
+    NEST does for a spike time that rounds to the current time.
+    """
+    steps, elems = [], []
+    for j, st in enumerate(trains):
+        st = check_spike_times(st)
+        if st is None:
+            continue
+        stamp = np.rint(st / dt).astype(np.int64)
+        if np.any(stamp < 1):
+            raise ValueError("spike time rounds to step 0 at resolution {}".format(dt))
+        emit = stamp - 1
+        emit = emit[emit < n_steps]
+        steps.append(emit)
+        elems.append(np.full(emit.size, j * batch + trial, np.int64))
+    if steps:
+        steps, elems = np.concatenate(steps), np.concatenate(elems)
+    else:
+        steps, elems = np.zeros(0, np.int64), np.zeros(0, np.int64)
+    order = np.lexsort((elems, steps))
+    steps, elems = steps[order], elems[order]
+    in_ptr = np.zeros(n_steps + 1, np.int64)
+    np.add.at(in_ptr, steps + 1, 1)
+    return np.cumsum(in_ptr), elems.astype(np.int32)

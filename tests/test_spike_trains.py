@@ -1,0 +1,106 @@
+"""Input spike sources: the reference's seeded Poisson vectors
+(bmtk/tests/utils/reports/spike_trains/test_spikes_core.py:8-44) and the
+spike_generator rules of bmtk/simulator/pointnet/pointnetwork.py:39-61."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from bmtk_amd.spike_trains import PoissonSpikeGenerator, bin_spike_times, check_spike_times
+
+
+@pytest.fixture(scope="module")
+def gold(golden_dir):
+    return json.load(open(os.path.join(golden_dir, "poisson_seed100.json")))
+
+
+def _fixed(gold):
+    g = gold["fixed"]
+    psg = PoissonSpikeGenerator(population="test", seed=g["seed"])
+    psg.add(node_ids=range(g["node_ids"]), firing_rate=g["firing_rate"], times=tuple(g["times"]))
+    return psg
+
+
+def test_psg_fixed_matches_reference_vectors(gold):
+    g = gold["fixed"]
+    psg = _fixed(gold)
+    assert psg.populations == ["test"]
+    assert psg.node_ids() == list(range(10))
+    assert psg.n_spikes() == g["n_spikes"] and psg.n_spikes(population="test") == g["n_spikes"]
+    np.testing.assert_allclose(psg.time_range(), g["time_range"])
+    assert psg.to_dataframe().shape == (g["n_spikes"], 3)
+    np.testing.assert_allclose(psg.get_times(node_id=0), g["node0"], atol=g["atol"])
+    np.testing.assert_allclose(psg.get_times(node_id=9, population="test"), g["node9"], atol=g["atol"])
+
+
+def test_psg_variable_continues_the_global_stream(gold):
+    """The reference's second test passes seed=0.0, which does not reseed, so
+    its expected trains depend on the stream position the first test left
+    behind; reproducing them shows the block-drawing generator consumes
+    exactly the draws a draw-by-draw loop would."""
+    _fixed(gold)
+    g = gold["variable"]
+    times = np.linspace(g["t0"], g["t1"], g["n_times"])
+    fr = np.exp(-np.power(times - 1.0, 2) / (2 * np.power(.5, 2))) * 5
+    psg = PoissonSpikeGenerator(population="test", seed=g["seed"])
+    psg.add(node_ids=range(g["node_ids"]), firing_rate=fr, times=times)
+    assert psg.n_spikes() == g["n_spikes"]
+    np.testing.assert_allclose(psg.time_range(), g["time_range"])
+    np.testing.assert_allclose(psg.get_times(node_id=0), g["node0"], atol=g["atol"])
+    np.testing.assert_allclose(psg.get_times(node_id=9), g["node9"], atol=g["atol"])
+
+
+def test_block_drawing_equals_scalar_loop():
+    np.random.seed(7)
+    want = []
+    for _ in range(25):
+        c, ts = 0.25, []
+        while True:
+            c += -np.log(1.0 - np.random.uniform()) / 40.0
+            if c > 2.0:
+                break
+            ts.append(c * 1000.0)
+        want.append(ts)
+    tail = np.random.uniform()
+    psg = PoissonSpikeGenerator(seed=7)
+    psg.add(node_ids=range(25), firing_rate=40.0, times=(0.25, 2.0))
+    for i in range(25):
+        np.testing.assert_allclose(psg.get_times(i), want[i], rtol=1e-14)
+    assert np.random.uniform() == tail
+
+
+def test_argument_errors():
+    psg = PoissonSpikeGenerator(seed=1)
+    with pytest.raises(ValueError):
+        psg.add(node_ids=[0], firing_rate=-1.0)
+    with pytest.raises(ValueError):
+        psg.add(node_ids=[0], firing_rate=5.0, times=(1.0, 0.5))
+    with pytest.raises(ValueError):
+        psg.add(node_ids=[0], firing_rate=5.0, tau_ref=-1)
+    with pytest.raises(ValueError):
+        psg.add(node_ids=[0], firing_rate=[1.0, 2.0], times=[0.0, 1.0, 2.0])
+    with pytest.raises(AttributeError):
+        PoissonSpikeGenerator(output_units="hours")
+
+
+def test_spike_time_rules():
+    # empty / None are skipped, unsorted is sorted, non-positive raises
+    assert check_spike_times(None) is None and check_spike_times([]) is None
+    np.testing.assert_array_equal(check_spike_times([3.0, 1.0, 2.0]), [1.0, 2.0, 3.0])
+    with pytest.raises(ValueError):
+        check_spike_times([1.0, 0.0])
+    with pytest.raises(ValueError):
+        check_spike_times([-0.1, 2.0])
+
+
+def test_binning_to_step_events():
+    trains = [[1.0, 3.0], None, [3.0, 2.0, 7.6]]
+    in_ptr, ev = bin_spike_times(trains, dt=1.0, n_steps=6, batch=2, trial=1)
+    # stamp s -> emitted in step s-1; event id = source*batch + trial
+    assert in_ptr.tolist() == [0, 1, 2, 4, 4, 4, 4]
+    assert ev.tolist() == [1, 5, 1, 5]
+    in_ptr, ev = bin_spike_times(trains, dt=1.0, n_steps=10)
+    assert in_ptr[-1] == 5 and ev[in_ptr[7]:in_ptr[8]].tolist() == [2]
+    with pytest.raises(ValueError):
+        bin_spike_times([[0.2]], dt=1.0, n_steps=4)
