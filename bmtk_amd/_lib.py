@@ -1,0 +1,84 @@
+"""ctypes binding of ``libbmtk_amd.so`` (declarations mirror ``include/bmtk_amd.h``).
+
+There is no fallback: if the library cannot be loaded every compute entry
+point raises.  ``load()`` compiles it once if the file is missing.
+"""
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libbmtk_amd.so")
+_lib = None
+
+c_void_p, c_int32, c_int64, c_float, c_double = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_double
+
+
+class Glif3Sim(C.Structure):
+    """``bmtk_glif3_sim`` of include/bmtk_amd.h, field for field."""
+    _fields_ = [
+        ("n_neurons", c_int64), ("batch", c_int32), ("ring_slots", c_int32), ("h", c_float), ("_pad0", c_int32),
+        ("V", c_void_p), ("asc", c_void_p), ("y1", c_void_p), ("y2", c_void_p), ("ref", c_void_p),
+        ("prop", c_void_p), ("prop_stride", c_int64), ("class_id", c_void_p), ("ring", c_void_p),
+        ("rec_indptr", c_void_p), ("rec_indices", c_void_p), ("rec_weights", c_void_p),
+        ("rec_delays", c_void_p), ("rec_receptors", c_void_p),
+        ("n_inputs", c_int64), ("in_ptr", c_void_p), ("in_events", c_void_p),
+        ("inp_indptr", c_void_p), ("inp_indices", c_void_p), ("inp_weights", c_void_p),
+        ("inp_delays", c_void_p), ("inp_receptors", c_void_p), ("i_ext", c_void_p),
+        ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
+        ("spike_step", c_void_p), ("spike_elem", c_void_p), ("spike_frac", c_void_p),
+        ("spike_cap", c_int64), ("spike_count", c_void_p),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
+SIGNATURES = {
+    "bmtk_amd_abi_version": (c_int32, []),
+    "bmtk_amd_last_error": (C.c_char_p, []),
+    "bmtk_glif3_precompute": (c_int32, [c_int64, c_void_p, c_double, c_void_p, c_void_p]),
+    "bmtk_glif3_step_fwd": (c_int32, [c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int32, c_void_p,
+                                      c_void_p, c_void_p, c_void_p, c_void_p]),
+    "bmtk_spikes_compact_workspace_bytes": (c_int64, [c_int64]),
+    "bmtk_spikes_compact": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "bmtk_spikes_compact_bits": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "bmtk_csr_propagate_scatter": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
+                                             c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
+    "bmtk_csr_propagate_gather": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
+    "bmtk_glif3_simulate_fwd": (c_int32, [C.POINTER(Glif3Sim), c_int64, c_int64, c_void_p]),
+}
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def load(build_if_missing=True):
+    """Return the loaded library, compiling it first if the file is absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        if not build_if_missing:
+            raise LibraryMissing("{} not built; run `python -m bmtk_amd.csrc.build`".format(LIB_PATH))
+        from .csrc.build import build
+        build()
+    try:
+        lib = C.CDLL(LIB_PATH)
+    except OSError as exc:
+        raise LibraryMissing("cannot load {}: {}".format(LIB_PATH, exc))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = lib
+    return lib
+
+
+class BmtkAmdError(RuntimeError):
+    pass
+
+
+def check(code):
+    if code != 0:
+        msg = load().bmtk_amd_last_error()
+        raise BmtkAmdError("libbmtk_amd error {}: {}".format(code, msg.decode() if msg else "?"))

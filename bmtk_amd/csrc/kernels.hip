@@ -1,0 +1,432 @@
+// HIP kernels and C entry points of the per-step operations: propagator
+// precompute, fused GLIF3 state update, spike compaction, event-driven scatter
+// and row-wise gather into the delay ring buffer.  gfx950 only.
+#include <math.h>
+#include <stdarg.h>
+
+#include "common.hpp"
+#include "glif3_update.hpp"
+#include "propagate.hpp"
+
+namespace bmtk {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+// ---------------------------------------------------------------------------
+// Propagators (NEST glif_psc::pre_run_hook + libnestutil/propagator_stability)
+// ---------------------------------------------------------------------------
+
+__device__ double propagator_32(double tau_syn, double tau, double C, double h)
+{
+    const double lin = 1.0 / (2.0 * C * tau * tau) * h * h * (tau_syn - tau) * exp(-h / tau);
+    const double sing = h / C * exp(-h / tau);
+    const double P32 = -tau / (C * (1.0 - tau / tau_syn)) * exp(-h / tau_syn) * expm1(h * (1.0 / tau_syn - 1.0 / tau));
+    const double dev = fabs(P32 - sing);
+    if (tau == tau_syn || (fabs(tau - tau_syn) < 0.1 && dev > 2.0 * fabs(lin))) return sing;
+    return P32;
+}
+
+__device__ double propagator_31(double tau_syn, double tau, double C, double h)
+{
+    const double lin = 1.0 / (3.0 * C * tau * tau) * h * h * h * (tau_syn - tau) * exp(-h / tau);
+    const double P31 = 1.0 / C *
+                       (exp(-h / tau_syn) * expm1(-h / tau + h / tau_syn) / (tau / tau_syn - 1.0) * tau -
+                        h * exp(-h / tau_syn)) /
+                       (-1.0 - -tau / tau_syn) * tau;
+    const double sing = h * h / 2.0 / C * exp(-h / tau);
+    const double dev = fabs(P31 - sing);
+    if (tau == tau_syn || (fabs(tau - tau_syn) < 0.1 && dev > 2.0 * fabs(lin))) return sing;
+    return P31;
+}
+
+__global__ __launch_bounds__(kBlock) void precompute_kernel(int64_t n, const double *__restrict__ par, double h,
+                                                            float *__restrict__ prop)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+#define PA(k) par[(int64_t)(k) * n + i]
+#define PO(k) prop[(int64_t)(k) * n + i]
+    const double C = PA(GLIF3_PAR_C_M), g = PA(GLIF3_PAR_G);
+    const double tau = C / g;
+    const double P33 = exp(-h / tau);
+    PO(GLIF3_P33) = (float)P33;
+    PO(GLIF3_P30) = (float)(1.0 / C * (1.0 - P33) * tau);
+    PO(GLIF3_TH) = (float)(PA(GLIF3_PAR_V_TH) - PA(GLIF3_PAR_E_L));
+    PO(GLIF3_UR) = (float)(PA(GLIF3_PAR_V_RESET) - PA(GLIF3_PAR_E_L));
+    // NEST counts the refractory period down in floating point, one resolution per step
+    const double t_ref = PA(GLIF3_PAR_T_REF);
+    double rem = t_ref;
+    int nref = 0;
+    while (rem > 0.0 && nref < (1 << 24)) {
+        rem -= h;
+        ++nref;
+    }
+    PO(GLIF3_NREF) = (float)nref;
+    for (int a = 0; a < GLIF3_NASC; ++a) {
+        const double k = PA(GLIF3_PAR_ASC_DECAY0 + a);
+        const double d = exp(-k * h);
+        PO(GLIF3_D0 + a) = (float)d;
+        PO(GLIF3_C0 + a) = (float)(((1.0 / k) / h) * (1.0 - d));
+        PO(GLIF3_R0 + a) = (float)(PA(GLIF3_PAR_ASC_R0 + a) * exp(-k * t_ref));
+        PO(GLIF3_AMP0 + a) = (float)PA(GLIF3_PAR_ASC_AMPS0 + a);
+    }
+    for (int r = 0; r < GLIF3_NREC; ++r) {
+        const double ts = PA(GLIF3_PAR_TAU_SYN0 + r);
+        PO(GLIF3_P11_0 + r) = (float)exp(-h / ts);
+        PO(GLIF3_P31_0 + r) = (float)propagator_31(ts, tau, C, h);
+        PO(GLIF3_P32_0 + r) = (float)propagator_32(ts, tau, C, h);
+        PO(GLIF3_PSC0_0 + r) = (float)(2.718281828459045235360287 / ts);
+    }
+#undef PA
+#undef PO
+}
+
+// ---------------------------------------------------------------------------
+// Fused state update: one thread per element, every array access is a
+// contiguous 256-byte row per wavefront.
+// ---------------------------------------------------------------------------
+
+struct StepArgs {
+    int64_t ne;
+    int32_t batch;
+    float *V, *asc, *y1, *y2;
+    int32_t *ref;
+    const float *prop;
+    int64_t stride;
+    const int32_t *class_id;
+    float h;
+    float *syn;
+    int32_t clear_syn;
+    const float *i_ext;
+    uint8_t *z;
+    uint64_t *zbits;
+    float *frac;
+};
+
+__global__ __launch_bounds__(kBlock) void glif3_step_kernel(StepArgs a)
+{
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    bool spike = false;
+    if (e < a.ne) {
+        const int64_t n = (a.batch == 1) ? e : (int64_t)((uint32_t)e / (uint32_t)a.batch);
+        const int64_t col = a.class_id ? (int64_t)a.class_id[n] : n;
+        Glif3Prop p;
+        p.load(a.prop, a.stride, col);
+        Glif3Elem s;
+        glif3_load(s, a.V, a.asc, a.y1, a.y2, a.ref, a.ne, e);
+        float syn[GLIF3_NREC];
+#pragma unroll
+        for (int k = 0; k < GLIF3_NREC; ++k) syn[k] = a.syn ? a.syn[k * a.ne + e] : 0.0f;
+        const float I = a.i_ext ? a.i_ext[e] : 0.0f;
+        float frac = 0.0f;
+        spike = glif3_update(s, p, a.h, syn, I, &frac);
+        glif3_store(s, a.V, a.asc, a.y1, a.y2, a.ref, a.ne, e);
+        if (a.syn && a.clear_syn) {
+#pragma unroll
+            for (int k = 0; k < GLIF3_NREC; ++k) a.syn[k * a.ne + e] = 0.0f;
+        }
+        if (a.z) a.z[e] = spike ? 1 : 0;
+        if (a.frac && spike) a.frac[e] = frac;
+    }
+    if (a.zbits) {
+        const unsigned long long m = __ballot(spike);
+        if (lane_id() == 0 && (e & ~(int64_t)(kWave - 1)) < a.ne) a.zbits[e >> 6] = m;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Compaction: flags -> bits -> per-block popcounts -> scan -> ordered ids
+// ---------------------------------------------------------------------------
+
+constexpr int kWordsPerBlock = kBlock;  // one 64-element word per thread
+
+__global__ __launch_bounds__(kBlock) void pack_bits_kernel(const uint8_t *__restrict__ z, int64_t n,
+                                                           uint64_t *__restrict__ bits)
+{
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const bool on = e < n && z[e] != 0;
+    const unsigned long long m = __ballot(on);
+    if (lane_id() == 0 && (e & ~(int64_t)(kWave - 1)) < n) bits[e >> 6] = m;
+}
+
+__device__ __forceinline__ unsigned long long load_word(const uint64_t *bits, int64_t w, int64_t n_words, int64_t n)
+{
+    if (w >= n_words) return 0ull;
+    unsigned long long v = bits[w];
+    const int tail = (int)(n & 63);
+    if (w == n_words - 1 && tail) v &= (1ull << tail) - 1ull;
+    return v;
+}
+
+__global__ __launch_bounds__(kBlock) void compact_count_kernel(const uint64_t *__restrict__ bits, int64_t n_words,
+                                                               int64_t n, uint32_t *__restrict__ block_count)
+{
+    const int64_t w = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x;
+    unsigned total;
+    block_exclusive_scan((unsigned)__popcll(load_word(bits, w, n_words, n)), &total);
+    if (threadIdx.x == 0) block_count[blockIdx.x] = total;
+}
+
+// one workgroup: exclusive scan of block_count in place, total -> *count
+__global__ __launch_bounds__(kBlock) void compact_scan_kernel(uint32_t *__restrict__ block_count, int n_blocks,
+                                                              int32_t *__restrict__ count)
+{
+    const int per = (n_blocks + kBlock - 1) / kBlock;
+    const int lo = threadIdx.x * per;
+    const int hi = min(lo + per, n_blocks);
+    unsigned sum = 0;
+    for (int i = lo; i < hi; ++i) sum += block_count[i];
+    unsigned total;
+    unsigned run = block_exclusive_scan(sum, &total);
+    for (int i = lo; i < hi; ++i) {
+        const unsigned c = block_count[i];
+        block_count[i] = run;
+        run += c;
+    }
+    if (threadIdx.x == 0) *count = (int32_t)total;
+}
+
+__global__ __launch_bounds__(kBlock) void compact_write_kernel(const uint64_t *__restrict__ bits, int64_t n_words,
+                                                               int64_t n, const uint32_t *__restrict__ block_offset,
+                                                               int32_t *__restrict__ ids)
+{
+    const int64_t w = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x;
+    unsigned long long v = load_word(bits, w, n_words, n);
+    unsigned total;
+    unsigned pos = block_offset[blockIdx.x] + block_exclusive_scan((unsigned)__popcll(v), &total);
+    const int32_t base = (int32_t)(w << 6);
+    while (v) {
+        const int b = __ffsll((long long)v) - 1;
+        v &= v - 1ull;
+        ids[pos++] = base + b;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Event-driven scatter: one wavefront per active element walks the source's
+// out-going synapses 64 at a time (coalesced table reads), fp32 atomics into
+// the ring.
+// ---------------------------------------------------------------------------
+
+__global__ __launch_bounds__(kBlock) void scatter_kernel(const int32_t *__restrict__ active,
+                                                         const int32_t *__restrict__ n_active, int batch, Table t,
+                                                         float *__restrict__ ring, int L, int64_t ne, int slot0)
+{
+    const int n_waves = gridDim.x * (kBlock / kWave);
+    const int cnt = *n_active;
+    for (int k = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; k < cnt; k += n_waves) {
+        const int e = active[k];
+        const int j = batch == 1 ? e : (int)((uint32_t)e / (uint32_t)batch);
+        deliver_row(t, j, e - j * batch, batch, ring, L, slot0, ne);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Row-wise gather: one wavefront per target row, lane = trial.  The spike
+// bits of a source over 64 trials are a native lane mask: a synapse whose
+// source fired in any trial is broadcast to the wavefront and every lane whose
+// trial fired adds the weight to its own accumulator (LDS, one column per
+// lane, one row per (slot, receptor)).  Accumulators start from the ring cell
+// on first touch and are stored back once, so every cell sees its additions
+// in stored synapse order: deterministic and equal to a scalar loop.
+// ---------------------------------------------------------------------------
+
+__device__ __forceinline__ unsigned long long source_mask(const uint64_t *__restrict__ zbits, int src, int batch,
+                                                          int tile0, int width)
+{
+    const int64_t bit = (int64_t)src * batch + tile0;
+    const int64_t w = bit >> 6;
+    const int sh = (int)(bit & 63);
+    unsigned long long m = zbits[w] >> sh;
+    if (sh + width > 64) m |= zbits[w + 1] << (64 - sh);
+    if (width < 64) m &= (1ull << width) - 1ull;
+    return m;
+}
+
+__global__ __launch_bounds__(kBlock) void gather_kernel(const uint64_t *__restrict__ zbits, int batch, Table t,
+                                                        float *__restrict__ ring, int L, int64_t n_tgt, int64_t ne,
+                                                        int slot0)
+{
+    extern __shared__ float lds[];
+    const int lane = lane_id();
+    const int wave_in_block = threadIdx.x / kWave;
+    float *acc = lds + (size_t)wave_in_block * L * GLIF3_NREC * kWave;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + wave_in_block;
+    if (row >= n_tgt) return;
+    const int tile0 = blockIdx.y * kWave;
+    const int width = min(kWave, batch - tile0);
+    const bool lane_on = lane < width;
+    const int64_t cell0 = row * batch + tile0 + lane;
+    unsigned long long touched = 0ull;  // bit (slot*4+r): accumulator row is live
+    const int p0 = t.indptr[row], p1 = t.indptr[row + 1];
+    for (int base = p0; base < p1; base += kWave) {
+        const int p = base + lane;
+        const bool valid = p < p1;
+        float w = 0.0f;
+        int dr = 0;
+        unsigned long long m = 0ull;
+        if (valid) {
+            const int src = t.indices[p];
+            w = t.weights[p];
+            int slot = slot0 + (int)t.delays[p];
+            slot = slot >= L ? slot - L : slot;
+            dr = slot * GLIF3_NREC + (int)t.receptors[p];
+            m = source_mask(zbits, src, batch, tile0, width);
+        }
+        unsigned long long act = __ballot(m != 0ull);
+        while (act) {
+            const int l = __ffsll((long long)act) - 1;
+            act &= act - 1ull;
+            const float wl = bcast_f(w, l);
+            const int drl = bcast_i(dr, l);
+            const unsigned long long ml = bcast_u64(m, l);
+            float *a = acc + drl * kWave + lane;
+            if (!((touched >> drl) & 1ull)) {
+                touched |= 1ull << drl;
+                *a = lane_on ? ring[(int64_t)drl * ne + cell0] : 0.0f;
+            }
+            if ((ml >> lane) & 1ull) *a += wl;
+        }
+    }
+    while (touched) {
+        const int drl = __ffsll((long long)touched) - 1;
+        touched &= touched - 1ull;
+        if (lane_on) ring[(int64_t)drl * ne + cell0] = acc[drl * kWave + lane];
+    }
+}
+
+}  // namespace bmtk
+
+// ===========================================================================
+// C entry points
+// ===========================================================================
+
+using namespace bmtk;
+
+extern "C" {
+
+int bmtk_amd_abi_version(void) { return 1; }
+
+const char *bmtk_amd_last_error(void) { return g_error; }
+
+int bmtk_glif3_precompute(int64_t n, const double *par, double h, float *prop, void *stream)
+{
+    BMTK_REQUIRE(n > 0 && par && prop, "glif3_precompute: n must be positive and pointers non-null");
+    BMTK_REQUIRE(h > 0.0, "glif3_precompute: resolution h must be positive");
+    const unsigned grid = (unsigned)((n + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(precompute_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, n, par, h, prop);
+    BMTK_CHECK_LAUNCH("glif3_precompute");
+    return BMTK_OK;
+}
+
+int bmtk_glif3_step_fwd(int64_t n_neurons, int32_t batch, float *V, float *asc, float *y1, float *y2, int32_t *ref,
+                        const float *prop, int64_t prop_stride, const int32_t *class_id, float h, float *syn,
+                        int32_t clear_syn, const float *i_ext, uint8_t *z, uint64_t *zbits, float *frac,
+                        void *stream)
+{
+    BMTK_REQUIRE(n_neurons > 0 && batch > 0, "glif3_step_fwd: n_neurons and batch must be positive");
+    BMTK_REQUIRE(V && asc && y1 && y2 && ref && prop, "glif3_step_fwd: state and prop pointers must be non-null");
+    BMTK_REQUIRE(class_id || prop_stride >= n_neurons, "glif3_step_fwd: prop_stride smaller than n_neurons");
+    BMTK_REQUIRE(prop_stride > 0, "glif3_step_fwd: prop_stride must be positive");
+    BMTK_REQUIRE(h > 0.0f, "glif3_step_fwd: resolution h must be positive");
+    const int64_t ne = n_neurons * (int64_t)batch;
+    BMTK_REQUIRE(ne < (1ll << 31), "glif3_step_fwd: n_neurons*batch must stay below 2^31");
+    StepArgs a{ne, batch, V, asc, y1, y2, ref, prop, prop_stride, class_id, h, syn, clear_syn, i_ext, z, zbits, frac};
+    const unsigned grid = (unsigned)((ne + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(glif3_step_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, a);
+    BMTK_CHECK_LAUNCH("glif3_step_fwd");
+    return BMTK_OK;
+}
+
+static int64_t n_words_of(int64_t n) { return (n + 63) / 64; }
+static int64_t n_blocks_of(int64_t n) { return (n_words_of(n) + kWordsPerBlock - 1) / kWordsPerBlock; }
+
+int64_t bmtk_spikes_compact_workspace_bytes(int64_t n)
+{
+    if (n <= 0) return 0;
+    // bit words (+1 padding) followed by the per-block counters
+    return 8 * (n_words_of(n) + 1) + 4 * (n_blocks_of(n) + 1);
+}
+
+static int compact_from_bits(const uint64_t *bits, int64_t n, int32_t *ids, int32_t *count, uint32_t *block_count,
+                             hipStream_t stream)
+{
+    const int64_t n_words = n_words_of(n);
+    const int n_blocks = (int)n_blocks_of(n);
+    hipLaunchKernelGGL(compact_count_kernel, dim3(n_blocks), dim3(kBlock), 0, stream, bits, n_words, n, block_count);
+    hipLaunchKernelGGL(compact_scan_kernel, dim3(1), dim3(kBlock), 0, stream, block_count, n_blocks, count);
+    hipLaunchKernelGGL(compact_write_kernel, dim3(n_blocks), dim3(kBlock), 0, stream, bits, n_words, n,
+                       (const uint32_t *)block_count, ids);
+    BMTK_CHECK_LAUNCH("spikes_compact");
+    return BMTK_OK;
+}
+
+int bmtk_spikes_compact(const uint8_t *z, int64_t n, int32_t *ids, int32_t *count, void *workspace, void *stream)
+{
+    BMTK_REQUIRE(n > 0 && n < (1ll << 31), "spikes_compact: n must lie in 1..2^31-1");
+    BMTK_REQUIRE(z && ids && count && workspace, "spikes_compact: pointers must be non-null");
+    uint64_t *bits = (uint64_t *)workspace;
+    uint32_t *block_count = (uint32_t *)(bits + n_words_of(n) + 1);
+    const unsigned grid = (unsigned)((n + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(pack_bits_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, z, n, bits);
+    return compact_from_bits(bits, n, ids, count, block_count, (hipStream_t)stream);
+}
+
+int bmtk_spikes_compact_bits(const uint64_t *zbits, int64_t n, int32_t *ids, int32_t *count, void *workspace,
+                             void *stream)
+{
+    BMTK_REQUIRE(n > 0 && n < (1ll << 31), "spikes_compact_bits: n must lie in 1..2^31-1");
+    BMTK_REQUIRE(zbits && ids && count && workspace, "spikes_compact_bits: pointers must be non-null");
+    uint32_t *block_count = (uint32_t *)((uint64_t *)workspace + n_words_of(n) + 1);
+    return compact_from_bits(zbits, n, ids, count, block_count, (hipStream_t)stream);
+}
+
+int bmtk_csr_propagate_scatter(const int32_t *active, const int32_t *n_active, int64_t max_active, int32_t batch,
+                               const int32_t *indptr, const int32_t *indices, const float *weights,
+                               const uint8_t *delays, const uint8_t *receptors, float *ring, int32_t L,
+                               int64_t n_tgt, int64_t step, void *stream)
+{
+    BMTK_REQUIRE(active && n_active && indptr && indices && weights && delays && receptors && ring,
+                 "csr_propagate_scatter: pointers must be non-null");
+    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && L > 1 && step >= 0, "csr_propagate_scatter: bad batch, n_tgt, L or step");
+    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31), "csr_propagate_scatter: n_tgt*batch must stay below 2^31");
+    if (max_active <= 0) return BMTK_OK;
+    const int64_t waves = max_active < 8192 ? max_active : 8192;
+    const unsigned grid = (unsigned)((waves + kBlock / kWave - 1) / (kBlock / kWave));
+    Table t{indptr, indices, weights, delays, receptors};
+    hipLaunchKernelGGL(scatter_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, active, n_active, batch, t,
+                       ring, L, n_tgt * (int64_t)batch, (int)(step % L));
+    BMTK_CHECK_LAUNCH("csr_propagate_scatter");
+    return BMTK_OK;
+}
+
+int bmtk_csr_propagate_gather(const uint64_t *zbits, int64_t n_src, int32_t batch, const int32_t *indptr,
+                              const int32_t *indices, const float *weights, const uint8_t *delays,
+                              const uint8_t *receptors, float *ring, int32_t L, int64_t n_tgt, int64_t step,
+                              void *stream)
+{
+    BMTK_REQUIRE(zbits && indptr && indices && weights && delays && receptors && ring,
+                 "csr_propagate_gather: pointers must be non-null");
+    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && n_src > 0 && step >= 0, "csr_propagate_gather: bad batch, sizes or step");
+    BMTK_REQUIRE(L > 1 && L <= 16, "csr_propagate_gather: ring_slots must lie in 2..16");
+    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31), "csr_propagate_gather: n_tgt*batch must stay below 2^31");
+    const unsigned rows_per_block = kBlock / kWave;
+    const dim3 grid((unsigned)((n_tgt + rows_per_block - 1) / rows_per_block), (unsigned)((batch + kWave - 1) / kWave));
+    BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_gather: batch too large");
+    const size_t lds = (size_t)rows_per_block * L * GLIF3_NREC * kWave * sizeof(float);
+    Table t{indptr, indices, weights, delays, receptors};
+    hipLaunchKernelGGL(gather_kernel, grid, dim3(kBlock), lds, (hipStream_t)stream, zbits, batch, t, ring, L, n_tgt,
+                       n_tgt * (int64_t)batch, (int)(step % L));
+    BMTK_CHECK_LAUNCH("csr_propagate_gather");
+    return BMTK_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,218 @@
+"""The per-step operations on torch device tensors (torch supplies memory and
+streams only; all arithmetic is in ``libbmtk_amd.so``).
+
+Layout: element e = neuron*batch + trial; state tensors are flat ``[ne]`` or
+``[k, ne]``; the ring buffer is ``[L, 4, ne]``; spike bits are uint64 words
+stored in int64 tensors of ``ceil(ne/64)+1`` entries.
+"""
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import _lib
+from .layout import NASC, NPARAM, NPROP, NREC
+
+
+def _dev():
+    if not torch.cuda.is_available():
+        raise RuntimeError("bmtk_amd needs a ROCm GPU; there is no CPU implementation of these operations")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t, dtype=None, numel=None, name="tensor"):
+    """Device pointer of a tensor after checking placement, dtype, contiguity and size."""
+    if t is None:
+        return None
+    if not t.is_cuda or not t.is_contiguous():
+        raise ValueError("{} must be a contiguous device tensor".format(name))
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError("{} must be {}, got {}".format(name, dtype, t.dtype))
+    if numel is not None and t.numel() < numel:
+        raise ValueError("{} holds {} entries, needs {}".format(name, t.numel(), numel))
+    return t.data_ptr()
+
+
+def n_words(ne):
+    return (ne + 63) // 64
+
+
+@dataclass
+class Glif3State:
+    """SoA fp32 state of ``ne = n_neurons*batch`` elements."""
+    V: torch.Tensor     # [ne]   membrane potential minus E_L (mV)
+    asc: torch.Tensor   # [2,ne] after-spike currents (pA)
+    y1: torch.Tensor    # [4,ne] alpha-PSC auxiliary state
+    y2: torch.Tensor    # [4,ne] post-synaptic currents (pA)
+    ref: torch.Tensor   # [ne]   int32 refractory steps left
+
+    @classmethod
+    def zeros(cls, n_neurons, batch=1, asc_init=None, u_init=None, device=None):
+        dev = device or _dev()
+        ne = n_neurons * batch
+        st = cls(torch.zeros(ne, device=dev), torch.zeros(NASC, ne, device=dev), torch.zeros(NREC, ne, device=dev),
+                 torch.zeros(NREC, ne, device=dev), torch.zeros(ne, dtype=torch.int32, device=dev))
+        if asc_init is not None:
+            a = torch.as_tensor(np.asarray(asc_init, np.float32).reshape(NASC, n_neurons), device=dev)
+            st.asc.copy_(a.repeat_interleave(batch, dim=1))
+        if u_init is not None:
+            u = torch.as_tensor(np.asarray(u_init, np.float32).reshape(n_neurons), device=dev)
+            st.V.copy_(u.repeat_interleave(batch))
+        return st
+
+    @classmethod
+    def from_numpy(cls, st, device=None):
+        dev = device or _dev()
+        return cls(*(torch.as_tensor(np.ascontiguousarray(st[k]), device=dev) for k in ("V", "asc", "y1", "y2", "ref")))
+
+    def to_numpy(self):
+        return {k: getattr(self, k).cpu().numpy() for k in ("V", "asc", "y1", "y2", "ref")}
+
+    def clone(self):
+        return Glif3State(self.V.clone(), self.asc.clone(), self.y1.clone(), self.y2.clone(), self.ref.clone())
+
+    @property
+    def ne(self):
+        return self.V.numel()
+
+
+def glif3_precompute(par, h):
+    """par: fp64 ``[NPARAM, n]`` NEST-unit parameters (host array or device tensor) ->
+    fp32 ``[NPROP, n]`` propagators (NEST ``glif_psc::pre_run_hook``)."""
+    lib = _lib.load()
+    par = torch.as_tensor(np.ascontiguousarray(par, np.float64) if not torch.is_tensor(par) else par, device=_dev())
+    if par.dim() != 2 or par.shape[0] != NPARAM:
+        raise ValueError("par must be [{}, n]".format(NPARAM))
+    par = par.contiguous()
+    n = par.shape[1]
+    prop = torch.empty(NPROP, n, dtype=torch.float32, device=par.device)
+    _lib.check(lib.bmtk_glif3_precompute(n, _p(par, torch.float64), float(h), _p(prop), _stream()))
+    return prop
+
+
+def glif3_step_fwd(state, prop, h, batch=1, class_id=None, syn=None, clear_syn=False, i_ext=None,
+                   z=None, zbits=None, frac=None):
+    """One ``glif_psc`` update step in place on ``state``."""
+    lib = _lib.load()
+    ne = state.ne
+    if ne % batch:
+        raise ValueError("state size {} is not a multiple of batch {}".format(ne, batch))
+    n = ne // batch
+    if prop.dim() != 2 or prop.shape[0] != NPROP:
+        raise ValueError("prop must be [{}, columns]".format(NPROP))
+    if class_id is not None and class_id.numel() != n:
+        raise ValueError("class_id must have one entry per neuron")
+    _lib.check(lib.bmtk_glif3_step_fwd(
+        n, batch, _p(state.V, torch.float32, ne, "V"), _p(state.asc, torch.float32, NASC * ne, "asc"),
+        _p(state.y1, torch.float32, NREC * ne, "y1"), _p(state.y2, torch.float32, NREC * ne, "y2"),
+        _p(state.ref, torch.int32, ne, "ref"), _p(prop, torch.float32), prop.shape[1],
+        _p(class_id, torch.int32, n, "class_id"), float(h), _p(syn, torch.float32, NREC * ne, "syn"),
+        1 if clear_syn else 0, _p(i_ext, torch.float32, ne, "i_ext"), _p(z, torch.uint8, ne, "z"),
+        _p(zbits, torch.int64, n_words(ne) + 1, "zbits"), _p(frac, torch.float32, ne, "frac"), _stream()))
+
+
+class SpikeCompactor:
+    """Flags or spike bits -> (ascending int32 ids, int32 count on the device).
+    Owns the workspace so repeated calls allocate nothing."""
+
+    def __init__(self, n, device=None):
+        lib = _lib.load()
+        dev = device or _dev()
+        self.n = n
+        self.workspace = torch.zeros(lib.bmtk_spikes_compact_workspace_bytes(n) // 8 + 1, dtype=torch.int64, device=dev)
+        self.ids = torch.empty(n, dtype=torch.int32, device=dev)
+        self.count = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def __call__(self, z):
+        lib = _lib.load()
+        if z.dtype == torch.uint8:
+            _lib.check(lib.bmtk_spikes_compact(_p(z, torch.uint8, self.n, "z"), self.n, _p(self.ids), _p(self.count),
+                                               _p(self.workspace), _stream()))
+        else:
+            _lib.check(lib.bmtk_spikes_compact_bits(_p(z, torch.int64, n_words(self.n), "zbits"), self.n,
+                                                    _p(self.ids), _p(self.count), _p(self.workspace), _stream()))
+        return self.ids, self.count
+
+
+def spikes_compact(z):
+    """Convenience form: returns the id list as a tensor of the exact length (synchronises)."""
+    c = SpikeCompactor(z.numel())
+    ids, count = c(z)
+    return ids[:int(count.item())].clone()
+
+
+@dataclass
+class SynapseTable:
+    """Device copy of a synapse table (see ``bmtk_amd.network``)."""
+    indptr: torch.Tensor
+    indices: torch.Tensor
+    weights: torch.Tensor
+    delays: torch.Tensor
+    receptors: torch.Tensor
+    n_rows: int
+    max_row: int
+
+    @classmethod
+    def from_numpy(cls, csr, device=None):
+        dev = device or _dev()
+        indptr, indices, w, d, r = csr
+        t = [torch.as_tensor(np.ascontiguousarray(a), device=dev) for a in (indptr, indices, w, d, r)]
+        deg = np.diff(indptr)
+        return cls(*t, n_rows=indptr.size - 1, max_row=int(deg.max()) if deg.size else 0)
+
+    @property
+    def nnz(self):
+        return self.indices.numel()
+
+    def pointers(self):
+        nnz = self.nnz
+        return (_p(self.indptr, torch.int32, self.n_rows + 1, "indptr"), _p(self.indices, torch.int32, nnz, "indices"),
+                _p(self.weights, torch.float32, nnz, "weights"), _p(self.delays, torch.uint8, nnz, "delays"),
+                _p(self.receptors, torch.uint8, nnz, "receptors"))
+
+
+def csr_propagate_scatter(active, n_active, table, ring, n_tgt, batch, step, max_active=None):
+    """Event-driven delivery of the active element list through a source-major table."""
+    lib = _lib.load()
+    L = ring.shape[0]
+    if ring.numel() != L * NREC * n_tgt * batch:
+        raise ValueError("ring must be [L, 4, n_tgt*batch]")
+    if max_active is None:
+        max_active = active.numel()
+    _lib.check(lib.bmtk_csr_propagate_scatter(
+        _p(active, torch.int32, None, "active"), _p(n_active, torch.int32, 1, "n_active"), max_active, batch,
+        *table.pointers(), _p(ring, torch.float32), L, n_tgt, int(step), _stream()))
+
+
+def csr_propagate_gather(zbits, n_src, table, ring, n_tgt, batch, step):
+    """Deterministic row-wise delivery through a target-major table from spike bits."""
+    lib = _lib.load()
+    L = ring.shape[0]
+    if ring.numel() != L * NREC * n_tgt * batch:
+        raise ValueError("ring must be [L, 4, n_tgt*batch]")
+    if table.n_rows != n_tgt:
+        raise ValueError("target-major table must have one row per target")
+    _lib.check(lib.bmtk_csr_propagate_gather(
+        _p(zbits, torch.int64, n_words(n_src * batch) + 1, "zbits"), n_src, batch, *table.pointers(),
+        _p(ring, torch.float32), L, n_tgt, int(step), _stream()))
+
+
+def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_active=None, zbits=None, n_src=None):
+    """``mode`` "scatter" (source-major table + active list) or "gather"
+    (target-major table + spike bits)."""
+    if mode == "scatter":
+        return csr_propagate_scatter(active, n_active, table, ring, n_tgt, batch, step)
+    if mode == "gather":
+        return csr_propagate_gather(zbits, n_src, table, ring, n_tgt, batch, step)
+    raise ValueError("mode must be 'scatter' or 'gather'")
+
+
+def unpack_bits(bits, ne):
+    """int64 spike-bit words ``[..., words]`` -> uint8 flags ``[..., ne]`` (host or device)."""
+    shifts = torch.arange(64, device=bits.device, dtype=torch.int64)
+    flags = ((bits.unsqueeze(-1) >> shifts) & 1).to(torch.uint8)
+    return flags.reshape(*bits.shape[:-1], -1)[..., :ne]

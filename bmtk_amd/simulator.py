@@ -1,0 +1,152 @@
+"""Forward GLIF3 simulation on one GPU: the work ``nest.Simulate`` does for a
+bmtk PointNet network (bmtk/simulator/pointnet/pointsimulator.py:159-166).
+
+``Glif3Simulator`` owns the device state, the ring buffer and the synapse
+tables, validates everything a kernel will index with on the host, and drives
+``bmtk_glif3_simulate_fwd``.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib, network as net
+from .layout import NPARAM, NPROP, NREC
+from .ops import Glif3State, SpikeCompactor, SynapseTable, _dev, _p, _stream, glif3_precompute, n_words, unpack_bits
+
+
+class Glif3Simulator:
+    """A population of GLIF3 neurons with recurrent and external synapses.
+
+    par         fp64 [NPARAM, columns] NEST-unit parameters; one column per
+                neuron, or per parameter class when ``class_id`` is given
+    rec, inp    source-major synapse tables (numpy tuples, see bmtk_amd.network):
+                recurrent (rows = neurons) and external (rows = input sources)
+    ring_slots  slots of the delay ring buffer; default = largest delay + 1
+    """
+
+    def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
+                 asc_init=None, u_init=None, i_ext=None, device=None):
+        self.lib = _lib.load()
+        self.dev = device or _dev()
+        self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
+        self.ne = self.n * self.batch
+        if self.ne >= 2 ** 31:
+            raise ValueError("n_neurons*batch must stay below 2^31")
+        par = np.ascontiguousarray(par, np.float64)
+        if par.shape[0] != NPARAM:
+            raise ValueError("par must be [{}, columns]".format(NPARAM))
+        if class_id is not None:
+            class_id = np.ascontiguousarray(class_id, np.int32)
+            if class_id.size != self.n or class_id.min() < 0 or class_id.max() >= par.shape[1]:
+                raise ValueError("class_id must map every neuron to a column of par")
+        elif par.shape[1] != self.n:
+            raise ValueError("par needs one column per neuron when class_id is not given")
+        self.prop = glif3_precompute(par, h)
+        self.class_id = None if class_id is None else torch.as_tensor(class_id, device=self.dev)
+        max_delay = 1
+        for t in (rec, inp):
+            if t is not None and t[3].size:
+                max_delay = max(max_delay, int(t[3].max()))
+        self.L = int(ring_slots) if ring_slots else max_delay + 1
+        self.rec = self._table(rec, self.n) if rec is not None else None
+        self.inp = self._table(inp, None) if inp is not None else None
+        self.n_inputs = self.inp.n_rows if self.inp is not None else 0
+        self.state = Glif3State.zeros(self.n, self.batch, asc_init=asc_init, u_init=u_init, device=self.dev)
+        self.ring = torch.zeros(self.L, NREC, self.ne, device=self.dev)
+        self.i_ext = None if i_ext is None else torch.as_tensor(np.asarray(i_ext, np.float32), device=self.dev)
+        if self.i_ext is not None and self.i_ext.numel() != self.ne:
+            raise ValueError("i_ext needs one entry per element")
+        self.in_ptr = self.in_events = None
+        self.in_steps = 0
+        self.step = 0
+        self.words = n_words(self.ne)
+
+    def _table(self, csr, n_rows):
+        rows = csr[0].size - 1 if n_rows is None else n_rows
+        net.check_csr(csr, rows, self.n, self.L)
+        return SynapseTable.from_numpy(csr, self.dev)
+
+    def set_input_events(self, in_ptr, in_events):
+        """Per-step event lists: events in_events[in_ptr[t]:in_ptr[t+1]] are
+        emitted in step t (their spike stamp is t+1)."""
+        if self.inp is None:
+            raise ValueError("no input synapse table")
+        in_ptr = np.ascontiguousarray(in_ptr, np.int64)
+        in_events = np.ascontiguousarray(in_events, np.int32)
+        if in_ptr[0] != 0 or np.any(np.diff(in_ptr) < 0) or in_ptr[-1] != in_events.size:
+            raise ValueError("in_ptr must be non-decreasing from 0 to len(in_events)")
+        if in_events.size and (in_events.min() < 0 or in_events.max() >= self.n_inputs * self.batch):
+            raise ValueError("input event id outside 0..n_inputs*batch-1")
+        self.in_ptr = torch.as_tensor(in_ptr, device=self.dev)
+        self.in_events = torch.as_tensor(in_events if in_events.size else np.zeros(1, np.int32), device=self.dev)
+        self.in_steps = in_ptr.size - 1
+
+    def _struct(self, bits=None, record=None):
+        s = _lib.Glif3Sim()
+        st = self.state
+        s.n_neurons, s.batch, s.ring_slots, s.h = self.n, self.batch, self.L, self.h
+        s.V, s.asc, s.y1, s.y2, s.ref = (_p(x) for x in (st.V, st.asc, st.y1, st.y2, st.ref))
+        s.prop, s.prop_stride, s.class_id = _p(self.prop), self.prop.shape[1], _p(self.class_id)
+        s.ring = _p(self.ring)
+        if self.rec is not None:
+            s.rec_indptr, s.rec_indices, s.rec_weights, s.rec_delays, s.rec_receptors = self.rec.pointers()
+        if self.inp is not None and self.in_ptr is not None:
+            s.n_inputs = self.n_inputs
+            s.in_ptr, s.in_events = _p(self.in_ptr), _p(self.in_events)
+            s.inp_indptr, s.inp_indices, s.inp_weights, s.inp_delays, s.inp_receptors = self.inp.pointers()
+        s.i_ext = _p(self.i_ext)
+        if bits is not None:
+            s.spike_bits, s.spike_bits_stride = _p(bits), bits.shape[1]
+        if record is not None:
+            s.spike_step, s.spike_elem, s.spike_frac = _p(record["step"]), _p(record["elem"]), _p(record["frac"])
+            s.spike_cap, s.spike_count = record["step"].numel(), _p(record["count"])
+        return s
+
+    def run(self, n_steps, spike_bits=True, record_cap=0):
+        """Advance ``n_steps`` steps.  Returns a dict with ``bits`` (int64
+        [n_steps, words], spike bits per step) and, when ``record_cap`` > 0,
+        the atomic spike record with crossing fractions.  Does not synchronise."""
+        if self.in_ptr is not None and self.step + n_steps > self.in_steps:
+            raise ValueError("input event lists cover {} steps, run would reach {}".format(
+                self.in_steps, self.step + n_steps))
+        bits = torch.zeros(n_steps, self.words, dtype=torch.int64, device=self.dev) if spike_bits else None
+        record = None
+        if record_cap:
+            record = dict(step=torch.zeros(record_cap, dtype=torch.int32, device=self.dev),
+                          elem=torch.zeros(record_cap, dtype=torch.int32, device=self.dev),
+                          frac=torch.zeros(record_cap, dtype=torch.float32, device=self.dev),
+                          count=torch.zeros(1, dtype=torch.int64, device=self.dev))
+        s = self._struct(bits, record)
+        _lib.check(self.lib.bmtk_glif3_simulate_fwd(C.byref(s), self.step, n_steps, _stream()))
+        self.step += n_steps
+        return dict(bits=bits, record=record)
+
+    def spikes_from_bits(self, bits, step0=0):
+        """Spike bits -> (step int64[], element int64[]) ascending, via the
+        compaction kernels (exactly ``numpy.nonzero`` of the raster)."""
+        n_steps, words = bits.shape
+        per = max(1, (2 ** 31 - 64) // (words * 64))
+        steps, elems = [], []
+        for k0 in range(0, n_steps, per):
+            chunk = bits[k0:k0 + per].contiguous()
+            n = chunk.numel() * 64
+            comp = SpikeCompactor(n, self.dev)
+            ids, count = comp(torch.cat([chunk.reshape(-1), chunk.new_zeros(1)]))
+            ids = ids[:int(count.item())].to(torch.int64)
+            steps.append(ids // (words * 64) + k0 + step0)
+            elems.append(ids % (words * 64))
+        return torch.cat(steps), torch.cat(elems)
+
+    def raster(self, bits):
+        """uint8 [n_steps, ne] from spike bits."""
+        return unpack_bits(bits, self.ne)
+
+    def synaptic_events(self, bits):
+        """Number of recurrent synaptic events the spikes in ``bits`` caused
+        (sum of the out-degree of every spiking neuron)."""
+        if self.rec is None:
+            return 0
+        _, elems = self.spikes_from_bits(bits)
+        deg = (self.rec.indptr[1:] - self.rec.indptr[:-1]).to(torch.int64)
+        return int(deg[elems // self.batch].sum().item())

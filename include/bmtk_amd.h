@@ -1,0 +1,153 @@
+/*
+ * C ABI of libbmtk_amd.so -- the GLIF3 point-neuron hot path on one MI355X.
+ *
+ * The reference (bmtk's PointNet driver) reaches this arithmetic through
+ * PyNEST, a Python module, not through an FFI of its own: nest.Create
+ * (bmtk/simulator/pointnet/sonata_adaptors.py:64-66), nest.Connect
+ * (bmtk/simulator/pointnet/pointnetwork.py:229-232) and nest.Simulate
+ * (bmtk/simulator/pointnet/pointsimulator.py:159-166).  The entry points below
+ * are the per-step operations NEST performs behind those calls, one function
+ * per operation, each citing the call it stands behind.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer unless the name ends in _host.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *    Calls enqueue work and return; they never synchronise and never allocate.
+ *  - Element index e = neuron * batch + trial ("trial-minor"): a 64-lane
+ *    wavefront covers 64 trials of one neuron when batch is a multiple of 64.
+ *  - State, SoA fp32: V[ne] (membrane potential minus E_L), asc[2][ne],
+ *    y1[4][ne], y2[4][ne], ref[ne] (int32 refractory steps left), ne = n*batch.
+ *  - Ring buffer: ring[L][4][ne] fp32, slot (t mod L) holds the weight sums
+ *    that arrive in step t; L must exceed the largest delay in steps.
+ *  - Synapse table: indptr int32[rows+1], indices int32[nnz], weights
+ *    fp32[nnz], delays uint8[nnz] in steps (>= 1), receptors uint8[nnz] 0-based.
+ *    "source-major": rows are presynaptic, indices are targets.
+ *    "target-major": rows are postsynaptic, indices are sources.
+ *  - Spike bits: uint64 words, bit (e mod 64) of word (e / 64) is element e;
+ *    arrays hold ceil(ne/64)+1 words (the last one is padding kernels may read).
+ *  - Return value: 0 on success, a negative BMTK_E_* code otherwise;
+ *    bmtk_amd_last_error() returns the message of the calling thread's last
+ *    failure.  Arguments are validated on the host before any launch; values
+ *    stored in device arrays (indices, delays, class ids) are NOT checked by
+ *    the kernels and must have been validated by the caller.
+ */
+#ifndef BMTK_AMD_H
+#define BMTK_AMD_H
+
+#include <stdint.h>
+
+#include "bmtk_amd_layout.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BMTK_OK 0
+#define BMTK_E_ARG (-1)    /* null pointer, non-positive size, unsupported combination */
+#define BMTK_E_LAUNCH (-2) /* HIP reported an error for the launch */
+#define BMTK_E_DEVICE (-3) /* no usable gfx950 device */
+
+int bmtk_amd_abi_version(void);
+const char *bmtk_amd_last_error(void);
+
+/* NEST glif_psc::pre_run_hook, run when bmtk calls nest.Create('glif_psc', n,
+ * params) (bmtk/simulator/pointnet/sonata_adaptors.py:64-66): NEST-unit
+ * parameters par[GLIF3_NPARAM][n] (fp64) and the resolution h (ms) ->
+ * propagators prop[GLIF3_NPROP][n] (fp32).  Computed in fp64, rounded once. */
+int bmtk_glif3_precompute(int64_t n, const double *par, double h, float *prop, void *stream);
+
+/* One glif_psc::update step for all n_neurons*batch elements (what
+ * nest.Simulate does per neuron per step, bmtk/simulator/pointnet/pointsimulator.py:159-166).
+ * prop is [GLIF3_NPROP][prop_stride]; column = neuron when class_id is NULL,
+ * else column = class_id[neuron].
+ * syn: [4][ne] weight sums arriving this step (one ring slot), may be NULL;
+ *      when clear_syn != 0 the slot is zeroed after it has been read.
+ * i_ext: [ne] external current used in this step, may be NULL.
+ * z (uint8[ne]), zbits (spike bits), frac (fp32[ne], fraction of the step at
+ * which threshold was crossed, written only where a spike occurred): outputs,
+ * each may be NULL. */
+int bmtk_glif3_step_fwd(int64_t n_neurons, int32_t batch,
+                        float *V, float *asc, float *y1, float *y2, int32_t *ref,
+                        const float *prop, int64_t prop_stride, const int32_t *class_id, float h,
+                        float *syn, int32_t clear_syn, const float *i_ext,
+                        uint8_t *z, uint64_t *zbits, float *frac, void *stream);
+
+/* Spike flags -> ascending list of active element ids (NEST keeps the same
+ * information as its per-slice spike register; bmtk maps ids back through
+ * GidPool, bmtk/simulator/pointnet/gids.py:24-107).
+ * ids must hold n entries, count is one int32; workspace must hold
+ * bmtk_spikes_compact_workspace_bytes(n) bytes.  Exactly numpy.flatnonzero. */
+int64_t bmtk_spikes_compact_workspace_bytes(int64_t n);
+int bmtk_spikes_compact(const uint8_t *z, int64_t n, int32_t *ids, int32_t *count, void *workspace, void *stream);
+/* Same from spike bits (n elements, ceil(n/64) words are read). */
+int bmtk_spikes_compact_bits(const uint64_t *zbits, int64_t n, int32_t *ids, int32_t *count, void *workspace,
+                             void *stream);
+
+/* Event-driven delivery (NEST static_synapse::send -> RingBuffer::add_value,
+ * wired by nest.Connect in bmtk/simulator/pointnet/pointnetwork.py:161-173,187-232):
+ * for every active element id = source*batch + trial in active[0..*n_active)
+ * and every synapse (source -> i, w, d, r) of the SOURCE-MAJOR table,
+ * ring[(step+d) mod L][r][i*batch+trial] += w with fp32 atomics.
+ * n_active is read on the device; max_active bounds it (grid sizing only). */
+int bmtk_csr_propagate_scatter(const int32_t *active, const int32_t *n_active, int64_t max_active, int32_t batch,
+                               const int32_t *indptr, const int32_t *indices, const float *weights,
+                               const uint8_t *delays, const uint8_t *receptors,
+                               float *ring, int32_t L, int64_t n_tgt, int64_t step, void *stream);
+
+/* The same sums taken row by row over the TARGET-MAJOR table from the spike
+ * bits of the emitting step: deterministic (each ring cell is updated by one
+ * wavefront, additions in stored synapse order), no atomics. */
+int bmtk_csr_propagate_gather(const uint64_t *zbits, int64_t n_src, int32_t batch,
+                              const int32_t *indptr, const int32_t *indices, const float *weights,
+                              const uint8_t *delays, const uint8_t *receptors,
+                              float *ring, int32_t L, int64_t n_tgt, int64_t step, void *stream);
+
+/* Everything nest.Simulate needs for a forward run (bmtk/simulator/pointnet/pointsimulator.py:159-166). */
+typedef struct bmtk_glif3_sim {
+    int64_t n_neurons;
+    int32_t batch;
+    int32_t ring_slots;          /* L */
+    float h;                     /* resolution, ms */
+    int32_t _pad0;
+    float *V, *asc, *y1, *y2;    /* state, see above */
+    int32_t *ref;
+    const float *prop;           /* [GLIF3_NPROP][prop_stride] */
+    int64_t prop_stride;
+    const int32_t *class_id;     /* NULL: one column per neuron */
+    float *ring;                 /* [L][4][ne] */
+    /* recurrent synapses, source-major (may be all NULL) */
+    const int32_t *rec_indptr, *rec_indices;
+    const float *rec_weights;
+    const uint8_t *rec_delays, *rec_receptors;
+    /* external spike sources: per-step event lists + source-major table */
+    int64_t n_inputs;
+    const int64_t *in_ptr;       /* [total steps + 1], indexed by absolute step */
+    const int32_t *in_events;    /* element ids source*batch+trial, emitted in that step */
+    const int32_t *inp_indptr, *inp_indices;
+    const float *inp_weights;
+    const uint8_t *inp_delays, *inp_receptors;
+    const float *i_ext;          /* [ne] constant external current or NULL */
+    /* outputs */
+    uint64_t *spike_bits;        /* [n_steps][words] spike bits per step, words = ceil(ne/64); or NULL.
+                                  * Row k belongs to step step0+k of the call that wrote it. */
+    int64_t spike_bits_stride;   /* words per row (>= ceil(ne/64)) */
+    /* optional spike record with sub-step crossing fractions, appended with
+     * atomics (unordered within a step); all NULL to disable */
+    int32_t *spike_step;
+    int32_t *spike_elem;
+    float *spike_frac;
+    int64_t spike_cap;
+    unsigned long long *spike_count; /* device counter, keeps counting past spike_cap */
+} bmtk_glif3_sim;
+
+/* Run steps step0 .. step0+n_steps-1: per step one fused kernel updates every
+ * element from ring slot (t mod L), clears the slot, and the wavefront that
+ * detects a spike walks that neuron's out-going synapses at once; input
+ * events of the step are delivered by the same launch.  Enqueues n_steps
+ * launches on `stream` and returns. */
+int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0, int64_t n_steps, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

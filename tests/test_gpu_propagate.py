@@ -1,0 +1,141 @@
+"""GPU parity of spike compaction and of the two delivery kernels."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import glif3_oracle as orc
+from bmtk_amd import network as net, ops
+from gpu_util import bits_of, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n", [1, 63, 64, 65, 1000, 16384, 16385, (1 << 20) + 3])
+@pytest.mark.parametrize("p", [0.0, 0.003, 0.3, 1.0])
+def test_compaction_is_flatnonzero(n, p):
+    rng = np.random.default_rng(n % 1000 + int(p * 1000))
+    z = (rng.random(n) < p).astype(np.uint8) if p < 1.0 else np.ones(n, np.uint8)
+    want = np.flatnonzero(z).astype(np.int32)
+    comp = ops.SpikeCompactor(n)
+    for src in (to_dev(z), to_dev(bits_of(z))):
+        ids, count = comp(src)
+        c = int(count.item())
+        assert c == want.size
+        np.testing.assert_array_equal(ids[:c].cpu().numpy(), want)
+
+
+def test_compaction_ignores_bits_beyond_n():
+    z = np.zeros(100, np.uint8)
+    z[[3, 99]] = 1
+    bits = bits_of(z).copy()
+    bits[1] |= np.int64(-1) << 40          # garbage above element 100 in the last word
+    comp = ops.SpikeCompactor(100)
+    ids, count = comp(to_dev(bits))
+    assert ids[:int(count.item())].cpu().tolist() == [3, 99]
+
+
+def _edges(rng, n_src, n_tgt, nnz, max_delay=5):
+    src = rng.integers(0, n_src, nnz).astype(np.int32)
+    tgt = rng.integers(0, n_tgt, nnz).astype(np.int32)
+    w = (rng.lognormal(0, 1, nnz) * rng.choice([-1, 1], nnz)).astype(np.float32)
+    d = rng.integers(1, max_delay + 1, nnz).astype(np.uint8)
+    r = rng.integers(0, 4, nnz).astype(np.uint8)
+    return src, tgt, w, d, r
+
+
+@pytest.mark.parametrize("batch,p", [(1, 0.05), (1, 1.0), (5, 0.2), (64, 0.02), (100, 0.1)])
+def test_scatter_matches_oracle(batch, p):
+    """fp32 atomics add in an arbitrary order, so the comparison is against the
+    fp64 oracle: |diff| <= 1e-5 * max(|want|, sum of |w| into the cell * 1e-2)
+    -- the floor is the magnitude rounding errors scale with when signed
+    weights cancel."""
+    rng = np.random.default_rng(30)
+    n_src, n_tgt, L = 300, 257, 6
+    src, tgt, w, d, r = _edges(rng, n_src, n_tgt, 20000)
+    csr = net.coo_to_csr(src, tgt, w, d, r, n_rows=n_src, major="source")
+    table = ops.SynapseTable.from_numpy(csr)
+    ring_d = torch.zeros(L, 4, n_tgt * batch, device="cuda")
+    ring_c = np.zeros((L, 4, n_tgt * batch))
+    mag_c = np.zeros((L, 4, n_tgt * batch))
+    csr_abs = (csr[0], csr[1], np.abs(csr[2]), csr[3], csr[4])
+    comp = ops.SpikeCompactor(n_src * batch)
+    for step in (0, 4, 11):
+        z = (rng.random(n_src * batch) < p).astype(np.uint8)
+        ids, count = comp(to_dev(z))
+        ops.csr_propagate_scatter(ids, count, table, ring_d, n_tgt, batch, step)
+        orc.deliver_events(np.flatnonzero(z), batch, csr, ring_c, n_tgt, step)
+        orc.deliver_events(np.flatnonzero(z), batch, csr_abs, mag_c, n_tgt, step)
+    got = ring_d.cpu().numpy()
+    assert np.abs(ring_c).max() > 0
+    assert np.max(np.abs(got - ring_c) / np.maximum(np.abs(ring_c), 1e-2 * mag_c + 1e-30)) < 1e-5
+    assert np.all(got[mag_c == 0] == 0)
+
+
+@pytest.mark.parametrize("batch,p", [(1, 0.1), (5, 0.2), (32, 0.05), (64, 0.02), (64, 0.6), (100, 0.1), (130, 0.05)])
+def test_gather_bit_exact_vs_fp32_oracle(batch, p):
+    """Each ring cell is updated by one wavefront in stored synapse order
+    starting from the value already there: identical to the scalar fp32 loop,
+    including on a ring that already holds values."""
+    rng = np.random.default_rng(31)
+    n_src, n_tgt, L = 211, 190, 6
+    src, tgt, w, d, r = _edges(rng, n_src, n_tgt, 15000)
+    csr = net.coo_to_csr(src, tgt, w, d, r, n_rows=n_tgt, major="target")
+    table = ops.SynapseTable.from_numpy(csr)
+    ring_c = rng.normal(0, 1, (L, 4, n_tgt * batch)).astype(np.float32)
+    ring_d = to_dev(ring_c)
+    for step in (0, 5, 9):
+        z = (rng.random(n_src * batch) < p).astype(np.uint8)
+        ops.csr_propagate_gather(to_dev(bits_of(z)), n_src, table, ring_d, n_tgt, batch, step)
+        orc.gather_rows(z, batch, csr, ring_c, n_tgt, step)
+        np.testing.assert_array_equal(ring_d.cpu().numpy(), ring_c)
+
+
+def test_gather_equals_scatter_and_dense_bruteforce():
+    rng = np.random.default_rng(32)
+    n, L, batch = 150, 6, 64
+    src, tgt, w, d, r = _edges(rng, n, n, 9000)
+    by_src = net.coo_to_csr(src, tgt, w, d, r, n_rows=n, major="source")
+    by_tgt = net.csr_transpose(by_src, n)
+    z = (rng.random(n * batch) < 0.05).astype(np.uint8)
+    want = orc.dense_deliver_bruteforce(z, batch, src, tgt, w, d, r, L, n, 7)
+    ring_g = torch.zeros(L, 4, n * batch, device="cuda")
+    ring_s = torch.zeros(L, 4, n * batch, device="cuda")
+    ops.csr_propagate_fwd("gather", ops.SynapseTable.from_numpy(by_tgt), ring_g, n, batch, 7,
+                          zbits=to_dev(bits_of(z)), n_src=n)
+    ids, count = ops.SpikeCompactor(n * batch)(to_dev(z))
+    ops.csr_propagate_fwd("scatter", ops.SynapseTable.from_numpy(by_src), ring_s, n, batch, 7,
+                          active=ids, n_active=count)
+    # floor 1e-2: a hundredth of the unit weight scale (lognormal(0,1) pA), sums of a few signed terms
+    assert rel_err(ring_g.cpu().numpy(), want, 1e-2) < 1e-5
+    assert rel_err(ring_s.cpu().numpy(), want, 1e-2) < 1e-5
+
+
+def test_empty_rows_and_no_spikes():
+    n, L = 70, 4
+    csr = net.coo_to_csr(np.array([5], np.int32), np.array([9], np.int32), np.array([2.0], np.float32),
+                         np.array([3], np.uint8), np.array([1], np.uint8), n_rows=n, major="source")
+    ring = torch.zeros(L, 4, n, device="cuda")
+    comp = ops.SpikeCompactor(n)
+    z = np.zeros(n, np.uint8)
+    ids, count = comp(to_dev(z))
+    ops.csr_propagate_scatter(ids, count, ops.SynapseTable.from_numpy(csr), ring, n, 1, 2)
+    assert not ring.any()
+    z[[5, 6]] = 1
+    ids, count = comp(to_dev(z))
+    ops.csr_propagate_scatter(ids, count, ops.SynapseTable.from_numpy(csr), ring, n, 1, 2)
+    assert ring[(2 + 3) % L, 1, 9].item() == 2.0 and ring.sum().item() == 2.0
+
+
+def test_propagate_argument_errors():
+    from bmtk_amd._lib import BmtkAmdError
+    n = 10
+    csr = net.coo_to_csr(np.array([1], np.int32), np.array([2], np.int32), np.array([1.0], np.float32),
+                         np.array([1], np.uint8), np.array([0], np.uint8), n_rows=n, major="target")
+    t = ops.SynapseTable.from_numpy(csr)
+    zb = torch.zeros(2, dtype=torch.int64, device="cuda")
+    with pytest.raises(BmtkAmdError):
+        ops.csr_propagate_gather(zb, n, t, torch.zeros(17, 4, n, device="cuda"), n, 1, 0)   # L > 16
+    with pytest.raises(ValueError):
+        ops.csr_propagate_gather(zb, n, t, torch.zeros(4, 4, n + 1, device="cuda"), n, 1, 0)
+    with pytest.raises(ValueError):
+        net.check_csr(csr, n, n, 1)         # delay 1 needs at least 2 slots
