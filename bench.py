@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the GLIF3 hot path on one MI355X.
+
+Workload (N=1): the V1-scale forward simulation -- 230,924 GLIF3 neurons in 111
+parameter classes, lognormal in-degree with mean 300 (~70 M recurrent
+synapses), 17,400 Poisson inputs at 5 Hz through ~8 M input synapses, 4
+receptors, delays 1-5 steps, dt = 1 ms, batch 1.  One "step" is one simulation
+step (1 ms) of the whole network; --steps defaults to the configuration's 3000.
+Recurrent weights are lognormal(0,1) pA signed by the source class as
+specified; input weights are scaled by 7 because at 1 pA the network stays
+silent and there would be no synaptic events to count (it settles at ~3 Hz).
+
+Prints ONE JSON line: value = neuron-updates/s of the whole job; synaptic
+events/s, the roofline of the dominant kernel, the isolated state-update and
+propagation kernels, and the CPU baseline ride along in the same object.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+B_PER_UPDATE_CLASS = 103       # 12 state words in + 12 out, 4 B current, 1 B flag, 2 B class id
+B_PER_UPDATE_PLAIN = 101       # same without the class id
+B_PER_EVENT = 18               # 4 index + 4 weight + 1 delay + 1 receptor + 8 ring read-modify-write
+
+N_V1, N_IN, MEAN_IN, N_IN_SYN, N_CLASSES = 230924, 17400, 300, 8_000_000, 111
+IN_RATE_HZ, IN_W_SCALE = 5.0, 7.0
+
+
+def build_v1(torch, steps_total):
+    import numpy as np
+    from bmtk_amd import synthetic
+    from bmtk_amd.simulator import Glif3Simulator
+    rng = np.random.default_rng(3)
+    par = synthetic.random_cells(rng, N_CLASSES)
+    class_id = rng.integers(0, N_CLASSES, N_V1).astype(np.int32)
+    by_tgt, by_src, _ = synthetic.device_network(N_V1, MEAN_IN, "lognormal", seed=3)
+    del by_tgt
+    inp = synthetic.device_input_table(N_IN, N_V1, N_IN_SYN, seed=4, w_scale=IN_W_SCALE)
+    in_ptr, in_ev = synthetic.device_poisson_events(N_IN, IN_RATE_HZ, 1.0, steps_total, seed=5)
+    sim = Glif3Simulator(N_V1, par, 1.0, class_id=class_id, rec=by_src, inp=inp)
+    sim.set_input_events(in_ptr, in_ev)
+    return sim, par, class_id
+
+
+def count_events(torch, sim, bits, step0):
+    """Synaptic events caused by the spikes in `bits` and by the input events of the same steps."""
+    rec = sim.synaptic_events(bits)
+    k0, k1 = int(sim.in_ptr[step0].item()), int(sim.in_ptr[step0 + bits.shape[0]].item())
+    ev = sim.in_events[k0:k1].long() // sim.batch
+    deg = (sim.inp.indptr[1:] - sim.inp.indptr[:-1]).long()
+    return rec, int(deg[ev].sum().item())
+
+
+def time_region(torch, fn):
+    """(wall seconds, HIP-event seconds on the current stream) around fn()."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0, e0.elapsed_time(e1) * 1e-3
+
+
+def bench_state_update(torch, steps=1000, warmup=50):
+    """Isolated fused state update: N = 1,048,576, per-neuron parameters,
+    Gaussian(0, 50 pA) currents from a pool of 8 pre-generated vectors."""
+    import numpy as np
+    from bmtk_amd import ops, synthetic
+    n = 1 << 20
+    rng = np.random.default_rng(1)
+    par = synthetic.random_cells(rng, n)
+    prop = ops.glif3_precompute(par, 1.0)
+    st = ops.Glif3State.from_numpy(synthetic.random_state(rng, par, n, 1))
+    pool = [torch.randn(n, device="cuda") * 50.0 for _ in range(8)]
+    z = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    for k in range(warmup):
+        ops.glif3_step_fwd(st, prop, 1.0, i_ext=pool[k % 8], z=z)
+    wall, dev = time_region(torch, lambda: [ops.glif3_step_fwd(st, prop, 1.0, i_ext=pool[k % 8], z=z)
+                                            for k in range(steps)])
+    per = dev / steps
+    # per-neuron parameters: 29 propagator words are read per update on top of the 101 B
+    alg = n * (B_PER_UPDATE_PLAIN + 29 * 4)
+    return {"kernel": "glif3_step_kernel", "workload": "state update N=1048576, per-neuron parameters, 1000 steps",
+            "neuron_updates_per_s": n / per, "us_per_launch": per * 1e6,
+            "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+            "bytes_per_update": B_PER_UPDATE_PLAIN + 29 * 4}
+
+
+def bench_propagation(torch, steps=200, warmup=20):
+    """Isolated spike propagation: 51,978 neurons, Poisson(1000) in-degree
+    (~52 M synapses), batch 64, Bernoulli spikes at 1, 5 and 20 Hz."""
+    from bmtk_amd import ops, synthetic
+    n, batch, L = 51978, 64, 6
+    by_tgt, by_src, _ = synthetic.device_network(n, 1000, "poisson", seed=2)
+    t_tgt = ops.SynapseTable.from_device(by_tgt, n, n, L)
+    t_src = ops.SynapseTable.from_device(by_src, n, n, L)
+    ne = n * batch
+    ring = torch.zeros(L, 4, ne, device="cuda")
+    comp = ops.SpikeCompactor(ne)
+    deg = (t_src.indptr[1:] - t_src.indptr[:-1]).long()
+    out = []
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    for rate in (1.0, 5.0, 20.0):
+        pool_bits, pool_ev = [], []
+        for _ in range(4):
+            z = (torch.rand(ne, device="cuda", generator=g) < rate * 1e-3)
+            zb = torch.zeros(ops.n_words(ne) + 1, dtype=torch.int64, device="cuda")
+            ids, count = comp(z.to(torch.uint8))
+            c = int(count.item())
+            pool_ev.append((ids[:c].clone(), count.clone(), int(deg[(ids[:c].long() // batch)].sum().item())))
+            # spike bits of the same flags
+            w = z.view(-1, 64).to(torch.int64)
+            zb[:-1] = (w << torch.arange(64, device="cuda")).sum(1)
+            pool_bits.append(zb)
+        events = sum(e for _, _, e in pool_ev) / len(pool_ev)
+        for mode in ("scatter", "gather"):
+            def one(k):
+                if mode == "scatter":
+                    ids, count, _ = pool_ev[k % 4]
+                    ops.csr_propagate_scatter(ids, count, t_src, ring, n, batch, k)
+                else:
+                    ops.csr_propagate_gather(pool_bits[k % 4], n, t_tgt, ring, n, batch, k)
+            for k in range(warmup):
+                one(k)
+            ring.zero_()
+            wall, dev = time_region(torch, lambda: [one(k) for k in range(steps)])
+            per = dev / steps
+            alg = events * B_PER_EVENT
+            out.append({"kernel": mode + "_kernel", "workload": "propagation N=51978 nnz=%d batch=64 rate=%gHz" %
+                        (t_src.nnz, rate), "events_per_launch": events, "synaptic_events_per_s": events / per,
+                        "us_per_launch": per * 1e6,
+                        "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS,
+                                     "unit": "GB/s", "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None}})
+    return out
+
+
+def cpu_baseline(torch, sim, par, class_id, sample_steps):
+    """The NEST-algorithm CPU restatement (fp64, event-driven source-major
+    delivery into per-neuron ring buffers, OpenMP) on the first `sample_steps`
+    steps of the same network, from rest."""
+    import numpy as np
+    from oracle import glif3_oracle as orc
+    rec = tuple(t.cpu().numpy() for t in (sim.rec.indptr, sim.rec.indices, sim.rec.weights, sim.rec.delays,
+                                          sim.rec.receptors))
+    inp = tuple(t.cpu().numpy() for t in (sim.inp.indptr, sim.inp.indices, sim.inp.weights, sim.inp.delays,
+                                          sim.inp.receptors))
+    in_ptr = sim.in_ptr.cpu().numpy()
+    in_ev = sim.in_events.cpu().numpy()
+    prop = orc.precompute(par, 1.0)
+    res = {}
+    for label, threads, steps in (("all", orc.max_threads(), sample_steps), ("one", 1, max(20, sample_steps // 8))):
+        orc.set_threads(threads)
+        st = orc.new_state(N_V1, 1, np.float64)
+        ring = np.zeros((sim.L, 4, N_V1))
+        t0 = time.perf_counter()
+        out = orc.simulate(st, prop, 1.0, steps, class_id=class_id, ring=ring, rec=rec, inp=inp, in_ptr=in_ptr,
+                           in_events=in_ev, spike_cap=steps * N_V1 // 16)
+        dt = time.perf_counter() - t0
+        deg = np.diff(rec[0])
+        ev = int(deg[out["elem"]].sum()) + int(np.diff(inp[0])[in_ev[:in_ptr[steps]]].sum())
+        res[label] = dict(threads=threads, steps=steps, seconds=dt, updates_per_s=N_V1 * steps / dt,
+                          events_per_s=ev / dt)
+    orc.set_threads(res["all"]["threads"])
+    a, o = res["all"], res["one"]
+    return {"value": a["updates_per_s"], "unit": "neuron-updates/s", "cores": a["threads"], "kind": "port",
+            "sample": "first %d steps of the same 230,924-neuron network from rest (%.1f s); NEST-algorithm "
+                      "restatement in C, fp64, OpenMP, not NEST" % (a["steps"], a["seconds"]),
+            "synaptic_events_per_s": a["events_per_s"],
+            "one_thread": {"value": o["updates_per_s"], "synaptic_events_per_s": o["events_per_s"],
+                           "steps": o["steps"], "seconds": o["seconds"]},
+            "host_cpu_count": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--cpu-steps", type=int, default=400, help="steps of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the isolated-kernel measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the path is not sharded); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    from bmtk_amd import _lib
+    _lib.load()
+
+    K, W = args.steps, args.warmup
+    sim, par, class_id = build_v1(torch, W + K)
+    sim.run(W, spike_bits=False)
+    res = {}
+    wall, dev = time_region(torch, lambda: res.update(sim.run(K)))
+    bits = res["bits"]
+    rec_ev, in_ev = count_events(torch, sim, bits, W)
+    events = rec_ev + in_ev
+    n_spikes = int(sim.raster(bits[::10]).sum().item()) * 10 if K >= 10 else 0
+    per_launch = dev / K
+    alg = N_V1 * B_PER_UPDATE_CLASS + events / K * B_PER_EVENT
+    line = {
+        "metric": "neuron-updates/s (with synaptic events/s) at 230k neurons; % of HBM roofline",
+        "value": N_V1 * K / wall, "unit": "neuron-updates/s",
+        "synaptic_events_per_s": events / wall,
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall / K * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "V1-scale forward simulation: 230,924 GLIF3 neurons, 111 classes, %d recurrent + %d "
+                               "input synapses, 17,400 Poisson inputs at 5 Hz, dt 1 ms, batch 1" %
+                               (sim.rec.nnz, sim.inp.nnz),
+                   "mean_rate_hz": n_spikes / (N_V1 * K * 1e-3) if K else 0.0,
+                   "recurrent_events": rec_ev, "input_events": in_ev, "input_weight_scale": IN_W_SCALE},
+        "roofline": {"bound": "hbm", "kernel": "sim_step_kernel", "achieved": alg / per_launch / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / per_launch / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_launch": alg, "us_per_launch": per_launch * 1e6},
+    }
+    if not args.no_kernels:
+        line["kernels"] = [bench_state_update(torch)] + bench_propagation(torch)
+    if args.cpu_steps > 0:
+        line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, args.cpu_steps)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

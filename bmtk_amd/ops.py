@@ -164,6 +164,22 @@ class SynapseTable:
         deg = np.diff(indptr)
         return cls(*t, n_rows=indptr.size - 1, max_row=int(deg.max()) if deg.size else 0)
 
+    @classmethod
+    def from_device(cls, csr, n_rows, n_cols, ring_slots):
+        """Adopt device tensors after the same checks ``network.check_csr`` makes on the host."""
+        indptr, indices, w, d, r = (t.contiguous() for t in csr)
+        nnz = indices.numel()
+        ok = indptr.numel() == n_rows + 1 and int(indptr[0]) == 0 and int(indptr[-1]) == nnz
+        ok = ok and bool((indptr[1:] >= indptr[:-1]).all())
+        ok = ok and w.numel() == nnz and d.numel() == nnz and r.numel() == nnz
+        if ok and nnz:
+            ok = bool((indices.min() >= 0) & (indices.max() < n_cols) & (d.min() >= 1) & (d.max() < ring_slots)
+                      & (r.max() < NREC))
+        if not ok:
+            raise ValueError("inconsistent synapse table (indptr, index range, delay range or receptor range)")
+        deg = indptr[1:] - indptr[:-1]
+        return cls(indptr, indices, w, d, r, n_rows=n_rows, max_row=int(deg.max()) if deg.numel() else 0)
+
     @property
     def nnz(self):
         return self.indices.numel()

@@ -46,7 +46,7 @@ class Glif3Simulator:
         self.class_id = None if class_id is None else torch.as_tensor(class_id, device=self.dev)
         max_delay = 1
         for t in (rec, inp):
-            if t is not None and t[3].size:
+            if t is not None and len(t[3]):
                 max_delay = max(max_delay, int(t[3].max()))
         self.L = int(ring_slots) if ring_slots else max_delay + 1
         self.rec = self._table(rec, self.n) if rec is not None else None
@@ -63,6 +63,9 @@ class Glif3Simulator:
         self.words = n_words(self.ne)
 
     def _table(self, csr, n_rows):
+        if torch.is_tensor(csr[0]):
+            rows = csr[0].numel() - 1 if n_rows is None else n_rows
+            return SynapseTable.from_device(csr, rows, self.n, self.L)
         rows = csr[0].size - 1 if n_rows is None else n_rows
         net.check_csr(csr, rows, self.n, self.L)
         return SynapseTable.from_numpy(csr, self.dev)
@@ -72,6 +75,16 @@ class Glif3Simulator:
         emitted in step t (their spike stamp is t+1)."""
         if self.inp is None:
             raise ValueError("no input synapse table")
+        if torch.is_tensor(in_ptr):
+            ok = bool((in_ptr[0] == 0) & (in_ptr[1:] >= in_ptr[:-1]).all() & (in_ptr[-1] == in_events.numel()))
+            if in_events.numel():
+                ok = ok and bool((in_events.min() >= 0) & (in_events.max() < self.n_inputs * self.batch))
+            if not ok or in_ptr.dtype != torch.int64 or in_events.dtype != torch.int32:
+                raise ValueError("device input event lists are inconsistent")
+            self.in_ptr = in_ptr.contiguous()
+            self.in_events = in_events.contiguous() if in_events.numel() else in_events.new_zeros(1)
+            self.in_steps = in_ptr.numel() - 1
+            return
         in_ptr = np.ascontiguousarray(in_ptr, np.int64)
         in_events = np.ascontiguousarray(in_events, np.int32)
         if in_ptr[0] != 0 or np.any(np.diff(in_ptr) < 0) or in_ptr[-1] != in_events.size:

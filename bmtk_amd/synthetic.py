@@ -111,3 +111,89 @@ def sparse_in_degree_network(rng, n, mean_in, degree="poisson", max_delay=5, inh
     d = rng.integers(1, max_delay + 1, nnz, dtype=np.uint8)
     r = _receptor(inh[src], inh[tgt])
     return (indptr.astype(np.int32), src, w.astype(np.float32), d, r), inh
+
+
+# ---------------------------------------------------------------------------
+# Large networks, generated on the device with torch's generator (the host
+# generators above would take minutes for 50-70 M synapses).
+# ---------------------------------------------------------------------------
+
+def _t_receptor(pre_inh, post_inh):
+    import torch
+    return (pre_inh.to(torch.uint8) + 2 * post_inh.to(torch.uint8)).to(torch.uint8)
+
+
+def device_network(n, mean_in, degree="lognormal", seed=3, max_delay=5, inh_frac=0.2, w_scale=1.0,
+                   inh_scale=1.0, device="cuda", sigma=0.5):
+    """Random recurrent network on the device: in-degree Poisson(mean_in) or
+    lognormal with mean ``mean_in``, uniformly random sources, weights
+    lognormal(0,1)*w_scale pA signed by the source class (inhibitory ones
+    also times ``inh_scale``), delays uniform 1..max_delay.
+    Returns (target-major table, source-major table, inh flags), each table a
+    tuple of device tensors (indptr, indices, weights, delays, receptors)."""
+    import torch
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    if degree == "poisson":
+        deg = torch.poisson(torch.full((n,), float(mean_in), device=device), generator=g).to(torch.int64)
+    else:
+        mu = float(np.log(mean_in) - sigma * sigma / 2)
+        deg = torch.exp(torch.randn(n, device=device, generator=g) * sigma + mu).round().to(torch.int64)
+    indptr = torch.zeros(n + 1, dtype=torch.int64, device=device)
+    indptr[1:] = torch.cumsum(deg, 0)
+    nnz = int(indptr[-1].item())
+    if nnz >= 2 ** 31:
+        raise ValueError("more than 2^31-1 synapses")
+    inh = torch.rand(n, device=device, generator=g) < inh_frac
+    tgt = torch.repeat_interleave(torch.arange(n, device=device, dtype=torch.int32), deg)
+    src = torch.randint(0, n, (nnz,), device=device, generator=g, dtype=torch.int32)
+    w = torch.exp(torch.randn(nnz, device=device, generator=g)) * w_scale
+    pre_inh = inh[src.long()]
+    w = torch.where(pre_inh, -w * inh_scale, w).to(torch.float32)
+    d = torch.randint(1, max_delay + 1, (nnz,), device=device, generator=g, dtype=torch.uint8)
+    r = _t_receptor(pre_inh, inh[tgt.long()])
+    by_tgt = (indptr.to(torch.int32), src, w, d, r)
+    order = torch.sort(src.long(), stable=True).indices
+    sp = torch.zeros(n + 1, dtype=torch.int64, device=device)
+    sp[1:] = torch.cumsum(torch.bincount(src.long(), minlength=n), 0)
+    by_src = (sp.to(torch.int32), tgt[order], w[order], d[order], r[order])
+    return by_tgt, by_src, inh
+
+
+def device_input_table(n_in, n, n_syn, seed=4, max_delay=5, w_scale=1.0, device="cuda"):
+    """External sources -> neurons, source-major on the device: ``n_syn``
+    synapses with uniformly random source and target, excitatory, receptor 0."""
+    import torch
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    src = torch.sort(torch.randint(0, n_in, (n_syn,), device=device, generator=g)).values
+    sp = torch.zeros(n_in + 1, dtype=torch.int64, device=device)
+    sp[1:] = torch.cumsum(torch.bincount(src, minlength=n_in), 0)
+    tgt = torch.randint(0, n, (n_syn,), device=device, generator=g, dtype=torch.int32)
+    w = (torch.exp(torch.randn(n_syn, device=device, generator=g)) * w_scale).to(torch.float32)
+    d = torch.randint(1, max_delay + 1, (n_syn,), device=device, generator=g, dtype=torch.uint8)
+    r = torch.zeros(n_syn, dtype=torch.uint8, device=device)
+    return (sp.to(torch.int32), tgt, w, d, r)
+
+
+def device_poisson_events(n_in, rate_hz, dt_ms, steps, batch=1, seed=5, device="cuda"):
+    """Bernoulli(rate*dt) spikes per (step, source, trial) -> step-sorted event
+    lists on the device (in_ptr int64[steps+1], in_events int32[])."""
+    import torch
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    p = rate_hz * dt_ms * 1e-3
+    ptr = [0]
+    chunks = []
+    block = max(1, (1 << 26) // max(1, n_in * batch))
+    for t0 in range(0, steps, block):
+        k = min(block, steps - t0)
+        z = torch.rand(k, n_in * batch, device=device, generator=g) < p
+        tt, ee = torch.nonzero(z, as_tuple=True)
+        counts = torch.bincount(tt, minlength=k)
+        ptr.append(counts)
+        chunks.append(ee.to(torch.int32))
+    counts = torch.cat([c if torch.is_tensor(c) else torch.zeros(0, dtype=torch.int64, device=device) for c in ptr[1:]])
+    in_ptr = torch.zeros(steps + 1, dtype=torch.int64, device=device)
+    in_ptr[1:] = torch.cumsum(counts, 0)
+    return in_ptr, torch.cat(chunks) if chunks else torch.zeros(0, dtype=torch.int32, device=device)
