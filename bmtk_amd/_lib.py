@@ -20,10 +20,13 @@ class Glif3Sim(C.Structure):
         ("V", c_void_p), ("asc", c_void_p), ("y1", c_void_p), ("y2", c_void_p), ("ref", c_void_p),
         ("prop", c_void_p), ("prop_stride", c_int64), ("class_id", c_void_p), ("ring", c_void_p),
         ("rec_indptr", c_void_p), ("rec_indices", c_void_p), ("rec_weights", c_void_p),
-        ("rec_delays", c_void_p), ("rec_receptors", c_void_p),
+        ("rec_delays", c_void_p), ("rec_receptors", c_void_p), ("rec_packed", c_void_p),
         ("n_inputs", c_int64), ("in_ptr", c_void_p), ("in_events", c_void_p),
         ("inp_indptr", c_void_p), ("inp_indices", c_void_p), ("inp_weights", c_void_p),
-        ("inp_delays", c_void_p), ("inp_receptors", c_void_p), ("i_ext", c_void_p),
+        ("inp_delays", c_void_p), ("inp_receptors", c_void_p), ("inp_packed", c_void_p), ("i_ext", c_void_p),
+        ("work_bits", c_void_p),
+        ("res_span", c_int32), ("res_groups", c_int32), ("rec_seg", c_void_p), ("inp_seg", c_void_p),
+        ("res_sync", c_void_p),
         ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
         ("spike_step", c_void_p), ("spike_elem", c_void_p), ("spike_frac", c_void_p),
         ("spike_cap", c_int64), ("spike_count", c_void_p),
@@ -45,6 +48,9 @@ SIGNATURES = {
                                              c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "bmtk_csr_propagate_gather": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
+    "bmtk_csr_pack": (c_int32, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "bmtk_csr_segment_offsets": (c_int32, [c_int64, c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p,
+                                           c_void_p]),
     "bmtk_glif3_simulate_fwd": (c_int32, [C.POINTER(Glif3Sim), c_int64, c_int64, c_void_p]),
 }
 

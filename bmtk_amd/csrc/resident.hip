@@ -1,0 +1,411 @@
+// Resident forward simulation: ONE cooperative launch for the whole run.
+//
+// Workgroup g owns elements [g*span, (g+1)*span): their state and propagators
+// live in registers, their slice of the delay ring in LDS, from the first step
+// to the last.  Per step a workgroup
+//   1. folds the arrivals of slot t-1 (LDS) into y1 and runs the GLIF3 update
+//      from registers, then publishes its wavefronts' spike ballots;
+//   2. signals the grid barrier of step t;
+//   3. while the barrier fills, pulls the spikes of step t-1: it scans the
+//      ballots every workgroup published before the previous barrier and, for
+//      each neuron that fired, reads ITS OWN segment of that neuron's synapse
+//      row (rows are sorted by target; a per-row offset table gives the
+//      segment bounds) and adds the weights into its LDS ring slice with LDS
+//      atomics; external input events of step t-1 are pulled the same way;
+//   4. waits for the barrier.
+// Nothing but spike ballots, segment offsets and the synapses actually used
+// crosses the memory system: no global atomics, no state traffic.
+//
+// Ballots are triple-buffered: buffer t%3 is written in step t, read in step
+// t+1 and next overwritten in step t+3, which a workgroup can only reach after
+// the barrier of step t+2, i.e. after every workgroup finished reading it.
+//
+// Every wait is bounded: a workgroup that spins too long on the barrier raises
+// the abort word, every other workgroup sees it and all leave the loop, so the
+// grid always drains.
+#include "glif3_update.hpp"
+#include "sim_internal.hpp"
+
+namespace bmtk {
+
+constexpr int kResBlock = 1024;
+constexpr unsigned kMaxSpin = 4000000u;  // polls of the barrier word before giving up (seconds)
+
+#ifdef BMTK_RES_PROFILE
+__device__ unsigned long long g_prof[8];
+#define PROF_T(var) const long long var = wall_clock64()
+#define PROF_ADD(i, a, b) if (threadIdx.x == 0 && blockIdx.x == 0) g_prof[i] += (unsigned long long)((b) - (a))
+#else
+#define PROF_T(var)
+#define PROF_ADD(i, a, b)
+#endif
+
+struct Resident {
+    int64_t step0, n_steps;
+    int span, n_groups;
+};
+
+__device__ __forceinline__ unsigned load_agent(const unsigned *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// add the weights of one row's synapses that target this workgroup's group,
+// positions [seg_row[g], seg_row[g+1]) of the packed table, to the LDS ring
+// slice.  The first four synapses are fetched together (a segment holds one or
+// two on average), the rest one by one.
+__device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_row, int g,
+                                             const bmtk_synapse *__restrict__ tab, float *ring_l, int span, int e0,
+                                             int L, int slot0)
+{
+    const uint32_t lo = seg_row[g], hi = seg_row[g + 1];
+    if (hi <= lo) return;
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(tab);
+    auto add = [&](const uint2 sy) {
+        int slot = slot0 + (int)(sy.x >> 26);
+        slot = slot >= L ? slot - L : slot;
+        const int r = (sy.x >> 24) & 3;
+        const int i = (int)(sy.x & 0xFFFFFFu) - e0;
+        atomicAdd(ring_l + (slot * GLIF3_NREC + r) * span + i, __uint_as_float(sy.y));
+    };
+    uint2 first[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) first[u] = rows[min(lo + (uint32_t)u, hi - 1u)];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (lo + (uint32_t)u < hi) add(first[u]);
+    for (uint32_t p = lo + 4u; p < hi; ++p) add(rows[p]);
+}
+
+constexpr int kActCap = 8192;   // active-row list in LDS (entries)
+constexpr int kScanWords = 4;   // ballot words per thread and round
+constexpr unsigned kInputTag = 0x80000000u;
+
+// Spikes and input events of step `tp` -> this workgroup's ring slice.
+// Round by round: every thread reads kScanWords ballot words and one input
+// event (independent loads), a workgroup-wide prefix sum packs the rows that
+// fired into one LDS list, then one thread per listed row pulls this
+// workgroup's segment of it.  Must be called by all threads of the workgroup.
+__device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int64_t tp,
+                                          float *ring_l, unsigned *act, unsigned *scan_l, int e0, int64_t words)
+{
+    const int tid = threadIdx.x;
+    const int L = s.ring_slots;
+    const int slot0 = (int)(tp % L);
+    const int wave = tid / kWave;
+    const bool has_rec = s.rec_seg != nullptr, has_in = s.in_ptr != nullptr;
+    int64_t k0 = 0, k1 = 0;
+    if (has_in) {
+        k0 = s.in_ptr[tp];
+        k1 = s.in_ptr[tp + 1];
+    }
+    const unsigned long long *bits =
+        reinterpret_cast<const unsigned long long *>(s.work_bits) + (tp % 3) * (words + 1);
+    const int64_t n_words = has_rec ? words : 0;
+    const int64_t word_rounds = (n_words + (int64_t)kScanWords * kResBlock - 1) / ((int64_t)kScanWords * kResBlock);
+    const int64_t event_rounds = (k1 - k0 + kResBlock - 1) / kResBlock;
+    const int64_t rounds = word_rounds > event_rounds ? word_rounds : event_rounds;
+    for (int64_t round = 0; round < rounds; ++round) {
+        const int64_t w0 = round * (int64_t)kScanWords * kResBlock;
+        PROF_T(p0);
+        unsigned long long v[kScanWords];
+        unsigned cnt = 0;
+#pragma unroll
+        for (int u = 0; u < kScanWords; ++u) {
+            const int64_t w = w0 + (int64_t)u * kResBlock + tid;
+            v[u] = w < n_words ? __hip_atomic_load(bits + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+        }
+        const int64_t ke = k0 + round * kResBlock + tid;
+        const bool has_event = ke < k1;
+        const unsigned event_row = has_event ? (unsigned)s.in_events[ke] : 0u;
+#pragma unroll
+        for (int u = 0; u < kScanWords; ++u) cnt += (unsigned)__popcll(v[u]);
+        cnt += has_event ? 1u : 0u;
+        const unsigned inc = wave_inclusive_scan(cnt);
+        if (lane_id() == kWave - 1) scan_l[wave] = inc;
+        __syncthreads();
+        PROF_T(p1);
+        unsigned base = 0, total = 0;
+#pragma unroll
+        for (int q = 0; q < kResBlock / kWave; ++q) {
+            const unsigned x = scan_l[q];
+            if (q < wave) base += x;
+            total += x;
+        }
+        const bool listed = total <= (unsigned)kActCap;
+        unsigned pos = base + inc - cnt;
+#pragma unroll
+        for (int u = 0; u < kScanWords; ++u) {
+            unsigned long long x = v[u];
+            const int64_t j0 = (w0 + (int64_t)u * kResBlock + tid) << 6;
+            while (x) {
+                const int bit = __ffsll((long long)x) - 1;
+                x &= x - 1ull;
+                if (listed)
+                    act[pos++] = (unsigned)(j0 + bit);
+                else  // more rows than the list holds: pull directly, unbalanced but correct
+                    pull_segment(s.rec_seg + (j0 + bit) * (r.n_groups + 1), g, s.rec_packed, ring_l, r.span, e0, L,
+                                 slot0);
+            }
+        }
+        if (has_event) {
+            if (listed)
+                act[pos++] = event_row | kInputTag;
+            else
+                pull_segment(s.inp_seg + (int64_t)event_row * (r.n_groups + 1), g, s.inp_packed, ring_l, r.span, e0,
+                             L, slot0);
+        }
+        __syncthreads();
+        PROF_T(p2);
+        if (listed) {
+            for (unsigned a = tid; a < total; a += kResBlock) {
+                const unsigned entry = act[a];
+                const int64_t row = entry & ~kInputTag;
+                if (entry & kInputTag)
+                    pull_segment(s.inp_seg + row * (r.n_groups + 1), g, s.inp_packed, ring_l, r.span, e0, L, slot0);
+                else
+                    pull_segment(s.rec_seg + row * (r.n_groups + 1), g, s.rec_packed, ring_l, r.span, e0, L, slot0);
+            }
+        }
+        __syncthreads();
+        PROF_T(p3);
+        PROF_ADD(4, p0, p1);
+        PROF_ADD(5, p1, p2);
+        PROF_ADD(6, p2, p3);
+    }
+}
+
+__global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim s, Resident r)
+{
+    extern __shared__ float ring_l[];  // [L*4][span], then the active-row list
+    __shared__ int go_on;
+    __shared__ unsigned scan_l[kResBlock / kWave];
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    // Workgroups are dispatched round-robin over the 8 XCDs (block b runs on XCD
+    // b % 8).  Give each XCD a run of consecutive groups so that the segments
+    // of a synapse row its workgroups read -- and their offsets -- are
+    // contiguous and are fetched into that XCD's L2 once.
+    const int per_xcd = (int)gridDim.x >> 3;
+    const int g = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    const int64_t ne = s.n_neurons;  // batch 1
+    const int64_t words = (ne + 63) >> 6;
+    const int L = s.ring_slots;
+    const int span = r.span;
+    const int e0 = g * span;
+    const int mine = (int)max((int64_t)0, min((int64_t)span, ne - e0));  // groups past the end own nothing
+    const bool own = tid < mine;
+    const int64_t e = e0 + tid;
+    unsigned *act = reinterpret_cast<unsigned *>(ring_l + s.ring_slots * GLIF3_NREC * r.span);
+    unsigned *barrier = s.res_sync;
+    unsigned *abort_word = s.res_sync + 1;
+
+    for (int c = tid; c < L * GLIF3_NREC * span; c += kResBlock) {
+        const int dr = c / span, i = c - dr * span;
+        ring_l[c] = i < mine ? s.ring[(int64_t)dr * ne + e0 + i] : 0.0f;
+    }
+    Glif3Elem st{};
+    Glif3Prop p{};
+    float I = 0.0f;
+    if (own) {
+        const int64_t col = s.class_id ? (int64_t)s.class_id[e] : e;
+        p.load(s.prop, s.prop_stride, col);
+        glif3_load(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
+        I = s.i_ext ? s.i_ext[e] : 0.0f;
+    }
+    __syncthreads();
+
+    const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
+    bool aborted = false;
+    int64_t done = 0;  // steps whose update has run
+    for (int64_t k = 0; k < r.n_steps; ++k) {
+        const int64_t t = r.step0 + k;
+        PROF_T(c0);
+        // 1. fold the arrivals of slot t-1 and update
+        bool spike = false;
+        float frac = 0.0f;
+        if (own) {
+            if (k > 0) {
+                float *prev = ring_l + (int)((t - 1) % L) * GLIF3_NREC * span + tid;
+#pragma unroll
+                for (int q = 0; q < GLIF3_NREC; ++q) {
+                    const float a = prev[q * span];
+                    prev[q * span] = 0.0f;
+                    st.y1[q] = st.y1[q] + a * p.psc0[q];
+                }
+            }
+            spike = glif3_update(st, p, s.h, zero, I, &frac);
+        }
+        const unsigned long long m = __ballot(spike);
+        // only the wavefronts that cover this workgroup's span own a ballot word
+        if (lane == 0 && tid < span && (e & ~(int64_t)(kWave - 1)) < ne) {
+            __hip_atomic_store(reinterpret_cast<unsigned long long *>(s.work_bits) + (t % 3) * (words + 1) + (e >> 6),
+                               m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (s.spike_bits) s.spike_bits[k * s.spike_bits_stride + (e >> 6)] = m;
+        }
+        if (s.spike_count && m != 0ull) {
+            const int leader = __ffsll((long long)m) - 1;
+            unsigned long long base = 0ull;
+            if (lane == leader) base = atomicAdd(s.spike_count, (unsigned long long)__popcll(m));
+            base = bcast_u64(base, leader);
+            const unsigned long long idx = base + (unsigned long long)lane_prefix(m);
+            if (spike && idx < (unsigned long long)s.spike_cap) {
+                s.spike_step[idx] = (int32_t)t;
+                s.spike_elem[idx] = (int32_t)e;
+                if (s.spike_frac) s.spike_frac[idx] = frac;
+            }
+        }
+        done = k + 1;
+        // Every wavefront waits until its own ballot store (a write-through, device-coherent
+        // store) has been acknowledged, then the workgroup meets; only after that does the
+        // barrier count move.  No L2 write-back is needed: nothing else written inside the
+        // loop is read by another workgroup before the kernel ends.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        PROF_T(c1);
+        // 2. arrive at the barrier of step t (ballots of this workgroup are out)
+        if (tid == 0) __hip_atomic_fetch_add(barrier, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        PROF_T(c2);
+        // 3. pull the spikes and input events of step t-1 while the barrier fills
+        if (k > 0 && mine > 0) pull_step(s, r, g, t - 1, ring_l, act, scan_l, e0, words);
+        __syncthreads();
+        PROF_T(c3);
+        // 4. wait for every workgroup's ballots of step t
+        if (tid == 0) {
+            const unsigned target = gridDim.x * (unsigned)(k + 1);
+            unsigned spins = 0;
+            int ok = 1;
+            while (load_agent(barrier) < target) {
+                if (load_agent(abort_word) != 0u) {
+                    ok = 0;
+                    break;
+                }
+                if (++spins > kMaxSpin) {
+                    __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ok = 0;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            // No acquire fence here: it would invalidate this XCD's L2 every step.  The only
+            // data other workgroups write during the run are the ballots, which are read with
+            // agent-scope loads that bypass the non-coherent caches.
+            go_on = ok;
+        }
+        __syncthreads();
+        PROF_T(c4);
+        PROF_ADD(0, c0, c1);
+        PROF_ADD(1, c1, c2);
+        PROF_ADD(2, c2, c3);
+        PROF_ADD(3, c3, c4);
+        if (!go_on) {
+            aborted = true;
+            break;
+        }
+    }
+
+    if (!aborted && done > 0) {
+        // closing: spikes and inputs of the last step, then fold the last slot
+        const int64_t tl = r.step0 + done - 1;
+        if (mine > 0) pull_step(s, r, g, tl, ring_l, act, scan_l, e0, words);
+        __syncthreads();
+        if (own) {
+            float *prev = ring_l + (int)(tl % L) * GLIF3_NREC * span + tid;
+#pragma unroll
+            for (int q = 0; q < GLIF3_NREC; ++q) {
+                const float a = prev[q * span];
+                prev[q * span] = 0.0f;
+                st.y1[q] = st.y1[q] + a * p.psc0[q];
+            }
+        }
+        __syncthreads();
+    }
+    if (own) glif3_store(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
+    for (int c = tid; c < L * GLIF3_NREC * span; c += kResBlock) {
+        const int dr = c / span, i = c - dr * span;
+        if (i < mine) s.ring[(int64_t)dr * ne + e0 + i] = ring_l[c];
+    }
+}
+
+__global__ void zero_words_kernel(unsigned *w, int n)
+{
+    if ((int)threadIdx.x < n) w[threadIdx.x] = 0u;
+}
+
+__global__ __launch_bounds__(kBlock) void segment_offsets_kernel(int64_t n_rows, const int32_t *__restrict__ indptr,
+                                                                 const int32_t *__restrict__ indices, int span,
+                                                                 int n_groups, uint32_t *__restrict__ seg,
+                                                                 int32_t *__restrict__ unsorted)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t total = n_rows * (int64_t)(n_groups + 1);
+    if (idx >= total) return;
+    const int64_t row = idx / (n_groups + 1);
+    const int g = (int)(idx - row * (n_groups + 1));
+    int lo = indptr[row], hi = indptr[row + 1];
+    if (g == 0) {
+        // one thread per row checks the ordering the binary searches rely on
+        for (int p = lo + 1; p < hi; ++p)
+            if (indices[p] < indices[p - 1]) {
+                *unsorted = 1;
+                break;
+            }
+    }
+    const int64_t bound = (int64_t)g * span;  // first position with target >= bound
+    while (lo < hi) {
+        const int mid = lo + ((hi - lo) >> 1);
+        if ((int64_t)indices[mid] < bound)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    seg[idx] = (uint32_t)lo;
+}
+
+int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream)
+{
+    Resident r{step0, n_steps, s.res_span, s.res_groups};
+    const size_t lds = (size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) + kActCap * sizeof(int);
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(sim_resident_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) {
+        set_error("glif3_simulate_fwd: resident mode needs %zu bytes of LDS: %s", lds, hipGetErrorString(err));
+        return BMTK_E_LAUNCH;
+    }
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, stream, s.res_sync, 4);
+    bmtk_glif3_sim s_copy = s;
+    void *args[] = {&s_copy, &r};
+    const unsigned grid = 8u * (unsigned)((s.res_groups + 7) / 8);
+    err = hipLaunchCooperativeKernel(reinterpret_cast<const void *>(sim_resident_kernel), dim3(grid),
+                                     dim3(kResBlock), args, lds, stream);
+    if (err != hipSuccess) {
+        set_error("glif3_simulate_fwd: cooperative launch of %d workgroups failed: %s", s.res_groups,
+                  hipGetErrorString(err));
+        return BMTK_E_LAUNCH;
+    }
+    return BMTK_OK;
+}
+
+}  // namespace bmtk
+
+using namespace bmtk;
+
+#ifdef BMTK_RES_PROFILE
+extern "C" void bmtk_debug_read_prof(unsigned long long *out)
+{
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_prof), sizeof(g_prof));
+}
+#endif
+
+extern "C" int bmtk_csr_segment_offsets(int64_t n_rows, const int32_t *indptr, const int32_t *indices, int32_t span,
+                                        int32_t n_groups, uint32_t *seg, int32_t *unsorted, void *stream)
+{
+    BMTK_REQUIRE(n_rows > 0 && indptr && indices && seg && unsorted, "csr_segment_offsets: bad sizes or null pointers");
+    BMTK_REQUIRE(span > 0 && n_groups > 0, "csr_segment_offsets: span and n_groups must be positive");
+    const int64_t total = n_rows * (int64_t)(n_groups + 1);
+    BMTK_REQUIRE(total < (1ll << 40), "csr_segment_offsets: table too large");
+    hipLaunchKernelGGL(segment_offsets_kernel, dim3((unsigned)((total + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, n_rows, indptr, indices, span, n_groups, seg, unsorted);
+    BMTK_CHECK_LAUNCH("csr_segment_offsets");
+    return BMTK_OK;
+}

@@ -1,71 +1,184 @@
-// Forward simulation driver: one fused kernel per step.
+// Forward simulation driver: one launch per step, update and delivery overlapped.
 //
-// Workgroups [0, n_update) each advance 256 elements: read and clear the ring
-// slot of this step, run the GLIF3 update, publish the wavefront's spike
-// ballot, and -- because every delay is at least one step, so nothing written
-// now is read before the next launch -- the wavefront that detected a spike
-// walks that neuron's out-going synapses immediately and adds the weights into
-// the future ring slots with fp32 atomics.  No compaction pass, no spike list
-// round trip through memory.  The remaining workgroups deliver the external
-// input events of the step the same way.
+// Launch for step t, three kinds of workgroups side by side:
+//   update   advance 1024 elements: fold the arrivals of ring slot t-1 into y1
+//            (and clear the slot), run the GLIF3 update, publish the
+//            wavefront's spike ballot;
+//   deliver  read the spike ballots of step t-1 and walk the out-going
+//            synapses of every neuron that fired, adding the weights into the
+//            ring slots t..t+D-1 with fp32 atomics;
+//   input    the same for the external events emitted in step t-1.
+//
+// Folding arrivals one launch late is exact: NEST adds the weights that arrive
+// in step t to y1 at the end of step t (y1 = y1*P11 + s*psc0) and nothing reads
+// y1 before the update of step t+1, so storing y1*P11 and adding s*psc0 at the
+// top of the next update performs the same two rounded operations.  It buys a
+// launch of slack: slot t must be complete when launch t+1 starts, not when
+// launch t starts, so the delivery of step t-1 runs concurrently with the
+// update of step t instead of after it.
+#include <stdlib.h>
 #include "common.hpp"
 #include "glif3_update.hpp"
 #include "propagate.hpp"
+#include "sim_internal.hpp"
 
 namespace bmtk {
 
-constexpr int kInputBlocks = 32;
+constexpr int kSimBlock = 512;
+constexpr int kSimWaves = kSimBlock / kWave;
+constexpr int kLdsTableBytes = 48 * 1024;
 
-__global__ __launch_bounds__(kBlock) void sim_step_kernel(bmtk_glif3_sim s, int64_t t, int64_t out_row,
-                                                          int n_update)
+struct SimLaunch {
+    int64_t t;        // step being updated (closing launch: one past the last step)
+    int64_t out_row;  // row of spike_bits to write
+    int n_update, n_deliver, n_input;
+    int do_update;     // 0 in the closing launch: fold only
+    int fold_prev;     // slot t-1 holds arrivals not yet folded into y1
+    int deliver_prev;  // work_bits buffer (t-1)%3 holds spikes not yet delivered
+    int lds_table;     // propagator table staged in LDS
+};
+
+// walk one row of a packed table, four 64-synapse chunks in flight at a time
+__device__ __forceinline__ void deliver_row_packed(const int32_t *__restrict__ indptr,
+                                                   const bmtk_synapse *__restrict__ syn, int j, int b, int batch,
+                                                   float *__restrict__ ring, int L, int slot0, int64_t ne)
 {
+    const int p0 = indptr[j], p1 = indptr[j + 1];
+    if (p1 <= p0) return;
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(syn);
+    for (int base = p0 + lane_id(); base < p1; base += 4 * kWave) {
+        uint2 s[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s[u] = rows[min(base + u * kWave, p1 - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (base + u * kWave < p1) {
+                const unsigned tdr = s[u].x;
+                int slot = slot0 + (int)(tdr >> 26);
+                slot = slot >= L ? slot - L : slot;
+                const int r = (tdr >> 24) & 3;
+                const int64_t i = tdr & 0xFFFFFFu;
+                atomicAdd(ring + ((int64_t)(slot * GLIF3_NREC + r) * ne + i * batch + b), __uint_as_float(s[u].y));
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, SimLaunch q)
+{
+    extern __shared__ float table[];  // [class][GLIF3_NPROP] when q.lds_table
     const int batch = s.batch;
     const int64_t ne = s.n_neurons * (int64_t)batch;
+    const int64_t words = (ne + 63) >> 6;
     const int L = s.ring_slots;
-    const int slot0 = (int)(t % L);
     const int lane = lane_id();
+    const int bid = (int)blockIdx.x;
 
-    if ((int)blockIdx.x >= n_update) {
-        // external input events emitted in this step
-        const Table inp{s.inp_indptr, s.inp_indices, s.inp_weights, s.inp_delays, s.inp_receptors};
-        const int64_t k0 = s.in_ptr[t], k1 = s.in_ptr[t + 1];
-        const int n_waves = ((int)gridDim.x - n_update) * (kBlock / kWave);
-        const int wave = ((int)blockIdx.x - n_update) * (kBlock / kWave) + threadIdx.x / kWave;
+    // Delivery workgroups take the lowest block ids so they are dispatched first and
+    // their dependent-load chains run under the streaming update, not after it.
+    if (bid < q.n_input) {
+        // ---- external input events emitted in step t-1 ----
+        // (not those of step t: with L = largest delay + 1 slots, a delay of L-1
+        //  from step t would land in slot t-1, which this launch is clearing)
+        const int slot0 = (int)((q.t - 1) % L);
+        const int64_t k0 = s.in_ptr[q.t - 1], k1 = s.in_ptr[q.t];
+        const int n_waves = q.n_input * kSimWaves;
+        const int wave = bid * kSimWaves + threadIdx.x / kWave;
         for (int64_t k = k0 + wave; k < k1; k += n_waves) {
             const int e = s.in_events[k];
             const int j = batch == 1 ? e : (int)((uint32_t)e / (uint32_t)batch);
-            deliver_row(inp, j, e - j * batch, batch, s.ring, L, slot0, ne);
+            deliver_row_packed(s.inp_indptr, s.inp_packed, j, e - j * batch, batch, s.ring, L, slot0, ne);
         }
         return;
     }
 
-    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (bid < q.n_input + q.n_deliver) {
+        // ---- spikes of step t-1 ----
+        if (!q.deliver_prev) return;
+        const int slot0 = (int)((q.t - 1) % L);
+        const uint64_t *__restrict__ bits = s.work_bits + ((q.t - 1) % 3) * (words + 1);
+        const int64_t n_waves = (int64_t)q.n_deliver * kSimWaves;
+        const int64_t wave = (int64_t)(bid - q.n_input) * kSimWaves + threadIdx.x / kWave;
+        const int64_t per = (words + n_waves - 1) / n_waves;
+        const int64_t w_end = min(words, (wave + 1) * per);
+        for (int64_t w0 = wave * per; w0 < w_end; w0 += kWave) {
+            const int64_t w = w0 + lane;
+            unsigned long long v = w < w_end ? bits[w] : 0ull;
+            unsigned long long act = __ballot(v != 0ull);
+            while (act) {
+                const int l = __ffsll((long long)act) - 1;
+                act &= act - 1ull;
+                unsigned long long vl = bcast_u64(v, l);
+                const int64_t e0 = (w0 + l) << 6;
+                while (vl) {
+                    const int bit = __ffsll((long long)vl) - 1;
+                    vl &= vl - 1ull;
+                    const int es = (int)(e0 + bit);
+                    const int j = batch == 1 ? es : (int)((uint32_t)es / (uint32_t)batch);
+                    deliver_row_packed(s.rec_indptr, s.rec_packed, j, es - j * batch, batch, s.ring, L, slot0, ne);
+                }
+            }
+        }
+        return;
+    }
+
+    // ---- update (or, in the closing launch, fold only) ----
+    const int n_cols = (int)s.prop_stride;
+    if (q.lds_table) {
+        for (int i = threadIdx.x; i < n_cols * GLIF3_NPROP; i += kSimBlock) {
+            const int k = i / n_cols, c = i - k * n_cols;
+            table[c * GLIF3_NPROP + k] = s.prop[i];
+        }
+        __syncthreads();
+    }
+    const int64_t e = (int64_t)(bid - q.n_input - q.n_deliver) * kSimBlock + threadIdx.x;
     bool spike = false;
     float frac = 0.0f;
     if (e < ne) {
         const int64_t n = batch == 1 ? e : (int64_t)((uint32_t)e / (uint32_t)batch);
         const int64_t col = s.class_id ? (int64_t)s.class_id[n] : n;
-        Glif3Prop p;
-        p.load(s.prop, s.prop_stride, col);
-        Glif3Elem st;
-        glif3_load(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
-        float *cur = s.ring + (int64_t)slot0 * GLIF3_NREC * ne + e;
-        float syn[GLIF3_NREC];
+        float *prev = s.ring + (int64_t)((q.t + L - 1) % L) * GLIF3_NREC * ne + e;
+        if (!q.do_update) {
+            if (q.fold_prev) {
 #pragma unroll
-        for (int k = 0; k < GLIF3_NREC; ++k) {
-            syn[k] = cur[k * ne];
-            cur[k * ne] = 0.0f;
+                for (int k = 0; k < GLIF3_NREC; ++k) {
+                    const float psc0 = q.lds_table ? table[col * GLIF3_NPROP + GLIF3_PSC0_0 + k]
+                                                   : s.prop[(GLIF3_PSC0_0 + k) * s.prop_stride + col];
+                    const float a = prev[k * ne];
+                    prev[k * ne] = 0.0f;
+                    s.y1[k * ne + e] = s.y1[k * ne + e] + a * psc0;
+                }
+            }
+        } else {
+            Glif3Prop p;
+            if (q.lds_table)
+                p.load(table + col * GLIF3_NPROP, 1, 0);
+            else
+                p.load(s.prop, s.prop_stride, col);
+            Glif3Elem st;
+            glif3_load(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
+            if (q.fold_prev) {
+#pragma unroll
+                for (int k = 0; k < GLIF3_NREC; ++k) {
+                    const float a = prev[k * ne];
+                    prev[k * ne] = 0.0f;
+                    st.y1[k] = st.y1[k] + a * p.psc0[k];
+                }
+            }
+            const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
+            const float I = s.i_ext ? s.i_ext[e] : 0.0f;
+            spike = glif3_update(st, p, s.h, zero, I, &frac);
+            glif3_store(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
         }
-        const float I = s.i_ext ? s.i_ext[e] : 0.0f;
-        spike = glif3_update(st, p, s.h, syn, I, &frac);
-        glif3_store(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
     }
-    unsigned long long m = __ballot(spike);
+    if (!q.do_update) return;
+    const unsigned long long m = __ballot(spike);
     const int64_t wave_base = e & ~(int64_t)(kWave - 1);
-    if (s.spike_bits && lane == 0 && wave_base < ne) s.spike_bits[out_row * s.spike_bits_stride + (e >> 6)] = m;
-    if (m == 0ull) return;
-
-    if (s.spike_count) {
+    if (lane == 0 && wave_base < ne) {
+        s.work_bits[(q.t % 3) * (words + 1) + (e >> 6)] = m;
+        if (s.spike_bits) s.spike_bits[q.out_row * s.spike_bits_stride + (e >> 6)] = m;
+    }
+    if (s.spike_count && m != 0ull) {
         // one counter bump per wavefront, record slots handed out in lane order
         const int leader = __ffsll((long long)m) - 1;
         unsigned long long base = 0ull;
@@ -73,26 +186,42 @@ __global__ __launch_bounds__(kBlock) void sim_step_kernel(bmtk_glif3_sim s, int6
         base = bcast_u64(base, leader);
         const unsigned long long idx = base + (unsigned long long)lane_prefix(m);
         if (spike && idx < (unsigned long long)s.spike_cap) {
-            s.spike_step[idx] = (int32_t)t;
+            s.spike_step[idx] = (int32_t)q.t;
             s.spike_elem[idx] = (int32_t)e;
             if (s.spike_frac) s.spike_frac[idx] = frac;
         }
     }
-    if (s.rec_indptr) {
-        const Table rec{s.rec_indptr, s.rec_indices, s.rec_weights, s.rec_delays, s.rec_receptors};
-        while (m) {
-            const int l = __ffsll((long long)m) - 1;
-            m &= m - 1ull;
-            const int es = (int)wave_base + l;
-            const int j = batch == 1 ? es : (int)((uint32_t)es / (uint32_t)batch);
-            deliver_row(rec, j, es - j * batch, batch, s.ring, L, slot0, ne);
-        }
-    }
+}
+
+__global__ __launch_bounds__(kBlock) void pack_kernel(int64_t nnz, const int32_t *__restrict__ indices,
+                                                      const float *__restrict__ weights,
+                                                      const uint8_t *__restrict__ delays,
+                                                      const uint8_t *__restrict__ receptors,
+                                                      bmtk_synapse *__restrict__ packed)
+{
+    const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (p >= nnz) return;
+    bmtk_synapse o;
+    o.tdr = (uint32_t)indices[p] | ((uint32_t)receptors[p] << 24) | ((uint32_t)delays[p] << 26);
+    o.weight = weights[p];
+    packed[p] = o;
 }
 
 }  // namespace bmtk
 
 using namespace bmtk;
+
+extern "C" int bmtk_csr_pack(int64_t nnz, const int32_t *indices, const float *weights, const uint8_t *delays,
+                             const uint8_t *receptors, bmtk_synapse *packed, void *stream)
+{
+    BMTK_REQUIRE(nnz >= 0 && nnz < (1ll << 31), "csr_pack: nnz must lie in 0..2^31-1");
+    if (nnz == 0) return BMTK_OK;
+    BMTK_REQUIRE(indices && weights && delays && receptors && packed, "csr_pack: pointers must be non-null");
+    hipLaunchKernelGGL(pack_kernel, dim3((unsigned)((nnz + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, nnz, indices, weights, delays, receptors, packed);
+    BMTK_CHECK_LAUNCH("csr_pack");
+    return BMTK_OK;
+}
 
 extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0, int64_t n_steps, void *stream)
 {
@@ -101,29 +230,63 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     BMTK_REQUIRE(s.n_neurons > 0 && s.batch > 0, "glif3_simulate_fwd: n_neurons and batch must be positive");
     const int64_t ne = s.n_neurons * (int64_t)s.batch;
     BMTK_REQUIRE(ne < (1ll << 31), "glif3_simulate_fwd: n_neurons*batch must stay below 2^31");
-    BMTK_REQUIRE(s.ring_slots > 1, "glif3_simulate_fwd: ring_slots must exceed the largest delay (>= 2)");
+    BMTK_REQUIRE(s.n_neurons < (1ll << 24), "glif3_simulate_fwd: the packed tables index at most 2^24 neurons");
+    BMTK_REQUIRE(s.ring_slots > 1 && s.ring_slots <= 64,
+                 "glif3_simulate_fwd: ring_slots must exceed the largest delay and stay within 2..64");
     BMTK_REQUIRE(s.h > 0.0f, "glif3_simulate_fwd: resolution h must be positive");
-    BMTK_REQUIRE(s.V && s.asc && s.y1 && s.y2 && s.ref && s.prop && s.ring,
-                 "glif3_simulate_fwd: state, prop and ring pointers must be non-null");
+    BMTK_REQUIRE(s.V && s.asc && s.y1 && s.y2 && s.ref && s.prop && s.ring && s.work_bits,
+                 "glif3_simulate_fwd: state, prop, ring and work_bits pointers must be non-null");
     BMTK_REQUIRE(s.prop_stride > 0 && (s.class_id || s.prop_stride >= s.n_neurons),
                  "glif3_simulate_fwd: prop_stride too small");
     const bool has_rec = s.rec_indptr != nullptr;
-    BMTK_REQUIRE(!has_rec || (s.rec_indices && s.rec_weights && s.rec_delays && s.rec_receptors),
-                 "glif3_simulate_fwd: recurrent table is incomplete");
+    BMTK_REQUIRE(!has_rec || s.rec_packed, "glif3_simulate_fwd: recurrent table needs rec_packed");
     const bool has_inp = s.in_ptr != nullptr;
-    BMTK_REQUIRE(!has_inp || (s.in_events && s.inp_indptr && s.inp_indices && s.inp_weights && s.inp_delays &&
-                              s.inp_receptors),
-                 "glif3_simulate_fwd: input event list or input table is incomplete");
+    BMTK_REQUIRE(!has_inp || (s.in_events && s.inp_indptr && s.inp_packed),
+                 "glif3_simulate_fwd: input event list needs in_events, inp_indptr and inp_packed");
     BMTK_REQUIRE(!s.spike_bits || s.spike_bits_stride >= (ne + 63) / 64,
                  "glif3_simulate_fwd: spike_bits_stride smaller than ceil(ne/64)");
     BMTK_REQUIRE(!s.spike_count || (s.spike_step && s.spike_elem && s.spike_cap > 0),
                  "glif3_simulate_fwd: spike record needs spike_step, spike_elem and a positive spike_cap");
     BMTK_REQUIRE(step0 >= 0 && n_steps >= 0, "glif3_simulate_fwd: step0 and n_steps must be non-negative");
-    const int n_update = (int)((ne + kBlock - 1) / kBlock);
-    const unsigned grid = (unsigned)(n_update + (has_inp ? kInputBlocks : 0));
-    for (int64_t k = 0; k < n_steps; ++k) {
-        hipLaunchKernelGGL(sim_step_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, s, step0 + k, k,
-                           n_update);
+    if (n_steps == 0) return BMTK_OK;
+    if (s.res_span > 0) {
+        BMTK_REQUIRE(s.batch == 1, "glif3_simulate_fwd: resident mode runs batch 1 only");
+        BMTK_REQUIRE(s.res_span % 64 == 0 && s.res_span <= 1024, "glif3_simulate_fwd: res_span must be a multiple of 64, at most 1024");
+        BMTK_REQUIRE(s.res_groups == (ne + s.res_span - 1) / s.res_span, "glif3_simulate_fwd: res_groups must equal ceil(ne/res_span)");
+        BMTK_REQUIRE(s.res_sync, "glif3_simulate_fwd: resident mode needs res_sync");
+        BMTK_REQUIRE(!has_rec || s.rec_seg, "glif3_simulate_fwd: resident mode needs rec_seg");
+        BMTK_REQUIRE(!has_inp || s.inp_seg, "glif3_simulate_fwd: resident mode needs inp_seg");
+        BMTK_REQUIRE((size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) <= 150u * 1024u,
+                     "glif3_simulate_fwd: ring slice does not fit in LDS");
+        bmtk_glif3_sim r = s;
+        if (!has_rec) r.rec_seg = nullptr;
+        if (!has_inp) r.inp_seg = nullptr;
+        return simulate_resident(r, step0, n_steps, (hipStream_t)stream);
+    }
+
+    const int64_t words = (ne + 63) / 64;
+    SimLaunch q{};
+    q.n_update = (int)((ne + kSimBlock - 1) / kSimBlock);
+    const int64_t max_deliver = (words + kSimWaves - 1) / kSimWaves;  // at least one word per wavefront
+    q.n_deliver = has_rec ? (int)(max_deliver < 128 ? max_deliver : 128) : 0;
+    const int n_input = has_inp ? 64 : 0;
+    const size_t table_bytes = (size_t)s.prop_stride * GLIF3_NPROP * sizeof(float);
+    q.lds_table = (s.class_id && table_bytes <= (size_t)kLdsTableBytes) ? 1 : 0;
+    const size_t lds = q.lds_table ? table_bytes : 0;
+    const char *dbg_env = getenv("BMTK_SIM_DEBUG");
+    const int dbg = dbg_env ? atoi(dbg_env) : 0;
+    if (dbg & 4) q.n_deliver = 32;
+    if (dbg & 8) q.n_deliver = 256;
+    for (int64_t k = 0; k <= n_steps; ++k) {
+        const bool closing = k == n_steps;
+        q.t = step0 + k;
+        q.out_row = k;
+        q.do_update = closing ? 0 : 1;
+        q.fold_prev = k > 0;
+        q.deliver_prev = (k > 0 && has_rec && !(dbg & 1)) ? 1 : 0;
+        q.n_input = (k > 0 && !(dbg & 2)) ? n_input : 0;
+        const unsigned grid = (unsigned)(q.n_update + q.n_deliver + q.n_input);
+        hipLaunchKernelGGL(sim_step_kernel, dim3(grid), dim3(kSimBlock), lds, (hipStream_t)stream, s, q);
     }
     BMTK_CHECK_LAUNCH("glif3_simulate_fwd");
     return BMTK_OK;

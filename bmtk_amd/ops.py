@@ -184,6 +184,38 @@ class SynapseTable:
     def nnz(self):
         return self.indices.numel()
 
+    def packed(self):
+        """The table as 8-byte {index | receptor<<24 | delay<<26, weight} records (built once)."""
+        if getattr(self, "_packed", None) is None:
+            if self.nnz and int(self.delays.max()) >= 64:
+                raise ValueError("packed tables hold delays below 64 steps")
+            lib = _lib.load()
+            out = torch.empty(max(self.nnz, 1), 2, dtype=torch.int32, device=self.indices.device)
+            _lib.check(lib.bmtk_csr_pack(self.nnz, *self.pointers()[1:], _p(out), _stream()))
+            self._packed = out
+        return self._packed
+
+    def sorted_by_index(self):
+        """The same table with every row ordered by index (stable), as the segment offsets need."""
+        rows = torch.repeat_interleave(torch.arange(self.n_rows, device=self.indices.device),
+                                       (self.indptr[1:] - self.indptr[:-1]).long())
+        order = torch.sort(rows * (1 << 24) + self.indices.long(), stable=True).indices
+        return SynapseTable(self.indptr, self.indices[order].contiguous(), self.weights[order].contiguous(),
+                            self.delays[order].contiguous(), self.receptors[order].contiguous(),
+                            n_rows=self.n_rows, max_row=self.max_row)
+
+    def segment_offsets(self, span, n_groups):
+        """uint32 [n_rows, n_groups+1] offsets of the first synapse per row whose index is >= g*span
+        (stored in an int32 tensor).  Raises if a row is not sorted by index."""
+        lib = _lib.load()
+        seg = torch.empty(self.n_rows, n_groups + 1, dtype=torch.int32, device=self.indices.device)
+        flag = torch.zeros(1, dtype=torch.int32, device=self.indices.device)
+        _lib.check(lib.bmtk_csr_segment_offsets(self.n_rows, _p(self.indptr), _p(self.indices), span, n_groups,
+                                                _p(seg), _p(flag), _stream()))
+        if int(flag.item()):
+            raise ValueError("synapse table rows are not sorted by index")
+        return seg
+
     def pointers(self):
         nnz = self.nnz
         return (_p(self.indptr, torch.int32, self.n_rows + 1, "indptr"), _p(self.indices, torch.int32, nnz, "indices"),

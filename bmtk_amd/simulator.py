@@ -26,7 +26,7 @@ class Glif3Simulator:
     """
 
     def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
-                 asc_init=None, u_init=None, i_ext=None, device=None):
+                 asc_init=None, u_init=None, i_ext=None, device=None, resident="auto"):
         self.lib = _lib.load()
         self.dev = device or _dev()
         self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
@@ -61,6 +61,43 @@ class Glif3Simulator:
         self.in_steps = 0
         self.step = 0
         self.words = n_words(self.ne)
+        self.work_bits = torch.zeros(3 * (self.words + 1), dtype=torch.int64, device=self.dev)
+        if self.n >= 2 ** 24:
+            raise ValueError("the packed synapse tables index at most 2^24 neurons")
+        self.res_sync = torch.zeros(4, dtype=torch.int32, device=self.dev)
+        self.res_span = self.res_groups = 0
+        self.rec_seg = self.inp_seg = None
+        self._pending_check = False
+        if resident:
+            self._setup_resident(required=(resident is True))
+
+    def _setup_resident(self, required):
+        """Resident mode keeps state in registers and the ring in LDS for a whole
+        run; it needs batch 1, at most 1024 elements per compute unit and a ring
+        slice that fits in LDS."""
+        n_cu = torch.cuda.get_device_properties(self.dev).multi_processor_count
+        span = -(-(-(-self.ne // (n_cu - n_cu % 8))) // 64) * 64
+        fits = self.batch == 1 and span <= 1024 and self.L * NREC * span * 4 <= 150 * 1024
+        if not fits:
+            if required:
+                raise ValueError("network does not fit resident mode (batch 1, <= 1024 elements per compute unit, "
+                                 "ring slice <= 150 KB)")
+            return
+        groups = -(-self.ne // span)
+        if self.rec is not None:
+            self.rec = self.rec.sorted_by_index()
+            self.rec_seg = self.rec.segment_offsets(span, groups)
+        if self.inp is not None:
+            self.inp = self.inp.sorted_by_index()
+            self.inp_seg = self.inp.segment_offsets(span, groups)
+        self.res_span, self.res_groups = span, groups
+
+    def check(self):
+        """Raise if the last resident run gave up on its grid barrier (synchronises)."""
+        if self._pending_check:
+            self._pending_check = False
+            if int(self.res_sync[1].item()) != 0:
+                raise RuntimeError("resident simulation aborted: grid barrier timed out; results are invalid")
 
     def _table(self, csr, n_rows):
         if torch.is_tensor(csr[0]):
@@ -104,11 +141,17 @@ class Glif3Simulator:
         s.ring = _p(self.ring)
         if self.rec is not None:
             s.rec_indptr, s.rec_indices, s.rec_weights, s.rec_delays, s.rec_receptors = self.rec.pointers()
+            s.rec_packed = _p(self.rec.packed())
         if self.inp is not None and self.in_ptr is not None:
             s.n_inputs = self.n_inputs
             s.in_ptr, s.in_events = _p(self.in_ptr), _p(self.in_events)
             s.inp_indptr, s.inp_indices, s.inp_weights, s.inp_delays, s.inp_receptors = self.inp.pointers()
+            s.inp_packed = _p(self.inp.packed())
         s.i_ext = _p(self.i_ext)
+        s.work_bits = _p(self.work_bits)
+        if self.res_span:
+            s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
+            s.rec_seg, s.inp_seg = _p(self.rec_seg), _p(self.inp_seg)
         if bits is not None:
             s.spike_bits, s.spike_bits_stride = _p(bits), bits.shape[1]
         if record is not None:
@@ -133,11 +176,13 @@ class Glif3Simulator:
         s = self._struct(bits, record)
         _lib.check(self.lib.bmtk_glif3_simulate_fwd(C.byref(s), self.step, n_steps, _stream()))
         self.step += n_steps
+        self._pending_check = bool(self.res_span)
         return dict(bits=bits, record=record)
 
     def spikes_from_bits(self, bits, step0=0):
         """Spike bits -> (step int64[], element int64[]) ascending, via the
         compaction kernels (exactly ``numpy.nonzero`` of the raster)."""
+        self.check()
         n_steps, words = bits.shape
         per = max(1, (2 ** 31 - 64) // (words * 64))
         steps, elems = [], []
@@ -153,6 +198,7 @@ class Glif3Simulator:
 
     def raster(self, bits):
         """uint8 [n_steps, ne] from spike bits."""
+        self.check()
         return unpack_bits(bits, self.ne)
 
     def synaptic_events(self, bits):

@@ -102,6 +102,24 @@ int bmtk_csr_propagate_gather(const uint64_t *zbits, int64_t n_src, int32_t batc
                               const uint8_t *delays, const uint8_t *receptors,
                               float *ring, int32_t L, int64_t n_tgt, int64_t step, void *stream);
 
+/* Packed synapse format used by the fused simulation: one 8-byte record per
+ * synapse, {uint32 tdr, float weight} with tdr = index | receptor << 24 |
+ * delay << 26 (index < 2^24, delay < 64 steps).  bmtk_csr_pack converts the
+ * four plain arrays of a table; packed must hold nnz records. */
+typedef struct bmtk_synapse {
+    uint32_t tdr;
+    float weight;
+} bmtk_synapse;
+int bmtk_csr_pack(int64_t nnz, const int32_t *indices, const float *weights, const uint8_t *delays,
+                  const uint8_t *receptors, bmtk_synapse *packed, void *stream);
+
+/* Per-row segment offsets of a SOURCE-MAJOR table whose rows are sorted by
+ * target: seg[row*(n_groups+1) + g] = position of the first synapse of the row
+ * whose target is >= g*span (g = 0..n_groups; the last entry is the row end).
+ * *unsorted (one int32) is set to 1 if some row is not sorted by target. */
+int bmtk_csr_segment_offsets(int64_t n_rows, const int32_t *indptr, const int32_t *indices, int32_t span,
+                             int32_t n_groups, uint32_t *seg, int32_t *unsorted, void *stream);
+
 /* Everything nest.Simulate needs for a forward run (bmtk/simulator/pointnet/pointsimulator.py:159-166). */
 typedef struct bmtk_glif3_sim {
     int64_t n_neurons;
@@ -119,6 +137,7 @@ typedef struct bmtk_glif3_sim {
     const int32_t *rec_indptr, *rec_indices;
     const float *rec_weights;
     const uint8_t *rec_delays, *rec_receptors;
+    const bmtk_synapse *rec_packed; /* same table packed (bmtk_csr_pack); required when rec_indptr is set */
     /* external spike sources: per-step event lists + source-major table */
     int64_t n_inputs;
     const int64_t *in_ptr;       /* [total steps + 1], indexed by absolute step */
@@ -126,7 +145,22 @@ typedef struct bmtk_glif3_sim {
     const int32_t *inp_indptr, *inp_indices;
     const float *inp_weights;
     const uint8_t *inp_delays, *inp_receptors;
+    const bmtk_synapse *inp_packed; /* required when in_ptr is set */
     const float *i_ext;          /* [ne] constant external current or NULL */
+    uint64_t *work_bits;         /* scratch, 3*(ceil(ne/64)+1) words: spike bits of the last steps */
+    /* Resident mode (optional, batch 1 only; res_span == 0 disables it): the
+     * network is split into res_groups = ceil(ne/res_span) workgroups that keep
+     * their elements' state in registers and their slice of the ring in LDS for
+     * the whole run.  rec_seg / inp_seg are bmtk_csr_segment_offsets tables
+     * built with the same span over tables whose rows are sorted by target;
+     * rec_packed / inp_packed are those same tables packed. */
+    int32_t res_span;            /* elements per workgroup: multiple of 64, at most 1024 */
+    int32_t res_groups;
+    const uint32_t *rec_seg;     /* [neurons][res_groups+1] */
+    const uint32_t *inp_seg;     /* [inputs][res_groups+1] */
+    uint32_t *res_sync;          /* 4 words of scratch: barrier counter, abort flag; zeroed by the call.
+                                  * After the run, word 1 != 0 means the grid barrier timed out and the
+                                  * results are invalid. */
     /* outputs */
     uint64_t *spike_bits;        /* [n_steps][words] spike bits per step, words = ceil(ne/64); or NULL.
                                   * Row k belongs to step step0+k of the call that wrote it. */
@@ -140,11 +174,25 @@ typedef struct bmtk_glif3_sim {
     unsigned long long *spike_count; /* device counter, keeps counting past spike_cap */
 } bmtk_glif3_sim;
 
-/* Run steps step0 .. step0+n_steps-1: per step one fused kernel updates every
- * element from ring slot (t mod L), clears the slot, and the wavefront that
- * detects a spike walks that neuron's out-going synapses at once; input
- * events of the step are delivered by the same launch.  Enqueues n_steps
- * launches on `stream` and returns. */
+/* Run steps step0 .. step0+n_steps-1.  One launch per step plus one closing
+ * launch.  A launch updates every element for step t while, in other
+ * workgroups of the same launch, the spikes of step t-1 are delivered through
+ * the packed recurrent table and the input events of step t-1 through the
+ * packed input table (fp32 atomics into the ring).  The two halves can overlap
+ * because weights arriving in step t only enter y1 at the end of that step and
+ * move no membrane potential before step t+1: the update of step t+1 folds the
+ * arrivals of slot t into y1 first (same two roundings as adding them at the
+ * end of step t), so slot t need only be complete when launch t+1 starts.  The
+ * closing launch delivers the spikes and input events of the last step and folds the last
+ * slot, after which state and ring are what a step-by-step evaluation gives.
+ * Enqueues n_steps+1 launches on `stream` and returns.
+ *
+ * With res_span > 0 the whole run is ONE cooperative launch instead: each
+ * workgroup updates its elements from registers, publishes its spike ballots,
+ * passes a grid barrier (one per step) and pulls, for every neuron that fired
+ * anywhere in the previous step, its own segment of that neuron's synapses
+ * into its LDS ring slice with LDS atomics -- no global atomics and no state
+ * traffic.  The barrier spins a bounded number of times; see res_sync. */
 int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0, int64_t n_steps, void *stream);
 
 #ifdef __cplusplus

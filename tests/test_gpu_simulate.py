@@ -27,26 +27,28 @@ def _oracle_run(cfg, dtype, steps=None, batch=1, in_ptr=None, in_events=None):
     return out, st, ring
 
 
-def _gpu_sim(cfg, batch=1, in_ptr=None, in_events=None):
+def _gpu_sim(cfg, batch=1, in_ptr=None, in_events=None, resident=False):
     sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
-                         inp=cfg["inp_src"], ring_slots=cfg["L"])
+                         inp=cfg["inp_src"], ring_slots=cfg["L"], resident=resident)
+    assert bool(sim.res_span) == bool(resident)
     sim.set_input_events(cfg["in_ptr"] if in_ptr is None else in_ptr,
                          cfg["in_events"] if in_events is None else in_events)
     return sim
 
 
+@pytest.mark.parametrize("resident", [False, True])
 @pytest.mark.parametrize("classes", [None, 11])
-def test_450_neuron_network_raster_and_state(classes):
+def test_450_neuron_network_raster_and_state(classes, resident):
     """The 450-GLIF3 shape (Erdos-Renyi p=0.1, 1000 Poisson inputs at 10 Hz x 50
     targets, delays 1-4, dt 1 ms, 1000 steps); input weights doubled so the
     network fires at ~5 Hz.  Raster: >= 99.9 % of (neuron, step) entries equal
     to the fp64 oracle's.  State after the first 100 steps (compared only while
     the rasters are still identical): 1e-5 relative against the fp32 oracle,
-    2e-4 against the fp64 oracle, floor 1e-3 (mV / pA).  The 1e-5 single-step
+    2e-4 against the fp64 oracle, values below one unit (mV / pA) held absolutely.  The 1e-5 single-step
     bound against fp64 is checked in test_gpu_state_update.py."""
     cfg = synthetic.small_glif3_network(n=450, n_in=1000, steps=1000, seed=0, in_w_scale=2.0, n_classes=classes)
     want, _, _ = _oracle_run(cfg, np.float64)
-    sim = _gpu_sim(cfg)
+    sim = _gpu_sim(cfg, resident=resident)
     out = sim.run(100)
     w100, st100, ring100 = _oracle_run(cfg, np.float64, steps=100)
     f100, sf100, rf100 = _oracle_run(cfg, np.float32, steps=100)
@@ -55,13 +57,13 @@ def test_450_neuron_network_raster_and_state(classes):
     if np.array_equal(ras100, f100["raster"]):
         # same fp32 update; only the order of the atomic additions differs
         for k in ("V", "asc", "y1", "y2"):
-            assert rel_err(got[k], sf100[k], 1e-3) < 1e-5, k
+            assert rel_err(got[k], sf100[k], 1.0) < 1e-5, k
         np.testing.assert_array_equal(got["ref"], sf100["ref"])
-        assert rel_err(sim.ring.cpu().numpy(), rf100, 1e-3) < 1e-5
+        assert rel_err(sim.ring.cpu().numpy(), rf100, 1.0) < 1e-5
     if np.array_equal(ras100, w100["raster"]):
         # against fp64 the fp32 rounding of 100 chained steps has accumulated: 2e-4
         for k in ("V", "asc", "y1", "y2"):
-            assert rel_err(got[k], st100[k], 1e-3) < 2e-4, k
+            assert rel_err(got[k], st100[k], 1.0) < 2e-4, k
     assert (ras100 == w100["raster"]).mean() >= 0.999
     out2 = sim.run(900)
     ras = np.concatenate([ras100, sim.raster(out2["bits"]).cpu().numpy()])
@@ -76,7 +78,8 @@ def test_450_neuron_network_raster_and_state(classes):
     assert sim.synaptic_events(out2["bits"]) == int(np.diff(cfg["rec_src"][0])[ee].sum())
 
 
-def test_reference_known_answer_on_gpu(golden_dir):
+@pytest.mark.parametrize("resident", [False, True])
+def test_reference_known_answer_on_gpu(golden_dir, resident):
     """The reference's GLIF3 known-answer protocol run through the GPU path:
     spike time = (step + crossing fraction) * h must hit 14.46548367 ms
     (bmtk/tests/simulator/pointnet/test_glif_utils.py:19) to 1e-3 ms in fp32."""
@@ -94,7 +97,7 @@ def test_reference_known_answer_on_gpu(golden_dir):
         stamps = np.rint(np.array(pr["spike_times_ms"]) / h).astype(np.int64)
         in_ptr = np.zeros(n_steps + 1, np.int64)
         np.add.at(in_ptr, stamps, 1)
-        sim = Glif3Simulator(1, par, h, inp=inp, asc_init=asc_init, u_init=u_init)
+        sim = Glif3Simulator(1, par, h, inp=inp, asc_init=asc_init, u_init=u_init, resident=resident)
         sim.set_input_events(np.cumsum(in_ptr), np.zeros(len(stamps), np.int32))
         out = sim.run(n_steps, record_cap=16)
         rec = out["record"]
@@ -118,7 +121,7 @@ def test_batched_trials_are_independent():
         step_ev = np.concatenate([e[p[t]:p[t + 1]].astype(np.int64) * B + b for b, (p, e) in enumerate(per_trial)])
         ev.append(np.sort(step_ev))
     in_events = np.concatenate(ev).astype(np.int32)
-    sim = _gpu_sim(cfg, batch=B, in_ptr=in_ptr, in_events=in_events)
+    sim = _gpu_sim(cfg, batch=B, in_ptr=in_ptr, in_events=in_events)   # batched runs use the per-step launches
     out = sim.run(300)
     ras = sim.raster(out["bits"]).cpu().numpy().reshape(300, cfg["n"], B)
     total = 0
@@ -132,13 +135,14 @@ def test_batched_trials_are_independent():
     assert (ras.reshape(300, -1) == wb["raster"]).mean() >= 0.999
 
 
-def test_no_synapses_and_constant_current():
+@pytest.mark.parametrize("resident", [False, True])
+def test_no_synapses_and_constant_current(resident):
     """Neither table present: the run is the bare state update driven by i_ext."""
     rng = np.random.default_rng(6)
     n, h = 1000, 1.0
     par = synthetic.random_cells(rng, n)
     I = rng.uniform(0, 600, n).astype(np.float32)
-    sim = Glif3Simulator(n, par, h, i_ext=I, ring_slots=2)
+    sim = Glif3Simulator(n, par, h, i_ext=I, ring_slots=2, resident=resident)
     out = sim.run(400)
     ras = sim.raster(out["bits"]).cpu().numpy()
     prop = orc.precompute(par, h)
@@ -158,3 +162,21 @@ def test_simulate_argument_errors():
         sim.run(21)                                                                          # beyond the input lists
     with pytest.raises(ValueError):
         sim.set_input_events(np.array([0, 1]), np.array([10 ** 6], np.int32))
+
+
+def test_resident_mode_multiple_workgroups_and_split_runs():
+    """A 3000-neuron network spans dozens of resident workgroups, so spikes
+    cross the grid barrier; two runs back to back must continue seamlessly and
+    both modes must agree with the oracle."""
+    cfg = synthetic.small_glif3_network(n=3000, n_in=500, steps=400, seed=8, in_w_scale=3.0, in_fanout=300,
+                                        p_conn=0.03, w_scale=1.5)
+    want, _, _ = _oracle_run(cfg, np.float64)
+    assert want["count"] > 2000
+    for resident in (True, False):
+        sim = _gpu_sim(cfg, resident=resident)
+        if resident:
+            assert sim.res_groups > 8
+        a = sim.run(150)
+        b = sim.run(250)
+        ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
+        assert (ras == want["raster"]).mean() >= 0.999

@@ -34,7 +34,9 @@ def test_step_bit_exact_vs_fp32_oracle_and_close_to_fp64(n, batch, classes):
     the oracle's operation order without fused multiply-add, so against the
     fp32 oracle every state word and every spike flag must be identical.
     Against the fp64 oracle a single step from identical fp32 states must
-    agree to 1e-5 relative (floor 1e-3 of the unit: mV, pA)."""
+    agree to 1e-5 relative; values below one unit (1 mV, 1 pA) are held to 1e-5
+    of a unit instead, since a membrane potential near zero is a sum of cancelling
+    terms of the order of 10 mV."""
     rng = np.random.default_rng(21)
     h = 1.0
     par = synthetic.random_cells(rng, classes or n)
@@ -77,7 +79,7 @@ def test_step_bit_exact_vs_fp32_oracle_and_close_to_fp64(n, batch, classes):
             for k in ("V", "asc", "y1", "y2"):
                 g = got[k].reshape(-1, ne)[:, keep]
                 w = c64[k].reshape(-1, ne)[:, keep]
-                assert rel_err(g, w, 1e-3) < 1e-5, k
+                assert rel_err(g, w, 1.0) < 1e-5, k
         n_spk += int(z_c.sum())
     assert n_spk > 0
 
