@@ -30,9 +30,12 @@ B_PER_EVENT = 18               # 4 index + 4 weight + 1 delay + 1 receptor + 8 r
 
 N_V1, N_IN, MEAN_IN, N_IN_SYN, N_CLASSES = 230924, 17400, 300, 8_000_000, 111
 IN_RATE_HZ, IN_W_SCALE = 5.0, 7.0
+# HBM bytes per simulated step of the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# (filled in from the counter runs summarised under profiles/; None = not measured)
+TRAFFIC_BYTES_PER_STEP = None
 
 
-def build_v1(torch, steps_total):
+def build_v1(torch, steps_total, resident="auto"):
     import numpy as np
     from bmtk_amd import synthetic
     from bmtk_amd.simulator import Glif3Simulator
@@ -43,7 +46,7 @@ def build_v1(torch, steps_total):
     del by_tgt
     inp = synthetic.device_input_table(N_IN, N_V1, N_IN_SYN, seed=4, w_scale=IN_W_SCALE)
     in_ptr, in_ev = synthetic.device_poisson_events(N_IN, IN_RATE_HZ, 1.0, steps_total, seed=5)
-    sim = Glif3Simulator(N_V1, par, 1.0, class_id=class_id, rec=by_src, inp=inp)
+    sim = Glif3Simulator(N_V1, par, 1.0, class_id=class_id, rec=by_src, inp=inp, resident=resident)
     sim.set_input_events(in_ptr, in_ev)
     return sim, par, class_id
 
@@ -158,7 +161,7 @@ def cpu_baseline(torch, sim, par, class_id, sample_steps):
     in_ev = sim.in_events.cpu().numpy()
     prop = orc.precompute(par, 1.0)
     res = {}
-    for label, threads, steps in (("all", orc.max_threads(), sample_steps), ("one", 1, max(20, sample_steps // 8))):
+    for label, threads, steps in (("all", orc.max_threads(), sample_steps), ("one", 1, max(20, sample_steps // 3))):
         orc.set_threads(threads)
         st = orc.new_state(N_V1, 1, np.float64)
         ring = np.zeros((sim.L, 4, N_V1))
@@ -186,8 +189,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--cpu-steps", type=int, default=400, help="steps of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-steps", type=int, default=3000, help="steps of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the isolated-kernel measurements")
+    ap.add_argument("--per-step", action="store_true", help="force one launch per step instead of resident mode")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a 1 GiB device-to-device copy 10 times (reference for scaling the FETCH_SIZE / "
+                         "WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path is not sharded); use --gpus 1", file=sys.stderr)
@@ -198,9 +205,17 @@ def main():
         sys.exit(2)
     from bmtk_amd import _lib
     _lib.load()
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, device="cuda")       # 1 GiB of fp32
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "copies": 10}))
+        return
 
     K, W = args.steps, args.warmup
-    sim, par, class_id = build_v1(torch, W + K)
+    sim, par, class_id = build_v1(torch, W + K, resident=False if args.per_step else "auto")
     sim.run(W, spike_bits=False)
     res = {}
     wall, dev = time_region(torch, lambda: res.update(sim.run(K)))
@@ -208,8 +223,14 @@ def main():
     rec_ev, in_ev = count_events(torch, sim, bits, W)
     events = rec_ev + in_ev
     n_spikes = int(sim.raster(bits[::10]).sum().item()) * 10 if K >= 10 else 0
-    per_launch = dev / K
-    alg = N_V1 * B_PER_UPDATE_CLASS + events / K * B_PER_EVENT
+    sim.check()
+    resident = bool(sim.res_span)
+    # resident mode: the timed region is ONE launch of sim_resident_kernel covering all K steps;
+    # otherwise K+1 launches of sim_step_kernel
+    launches = 1 if resident else K + 1
+    per_launch = dev / launches
+    alg_step = N_V1 * B_PER_UPDATE_CLASS + events / K * B_PER_EVENT
+    alg = alg_step * K / launches
     line = {
         "metric": "neuron-updates/s (with synaptic events/s) at 230k neurons; % of HBM roofline",
         "value": N_V1 * K / wall, "unit": "neuron-updates/s",
@@ -219,16 +240,20 @@ def main():
         "config": {"workload": "V1-scale forward simulation: 230,924 GLIF3 neurons, 111 classes, %d recurrent + %d "
                                "input synapses, 17,400 Poisson inputs at 5 Hz, dt 1 ms, batch 1" %
                                (sim.rec.nnz, sim.inp.nnz),
+                   "mode": "resident (one cooperative launch)" if resident else "one launch per step",
                    "mean_rate_hz": n_spikes / (N_V1 * K * 1e-3) if K else 0.0,
                    "recurrent_events": rec_ev, "input_events": in_ev, "input_weight_scale": IN_W_SCALE},
-        "roofline": {"bound": "hbm", "kernel": "sim_step_kernel", "achieved": alg / per_launch / 1e9,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / per_launch / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes_per_launch": alg, "us_per_launch": per_launch * 1e6},
+        "roofline": {"bound": "hbm", "kernel": "sim_resident_kernel" if resident else "sim_step_kernel",
+                     "achieved": alg / per_launch / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg / per_launch / 1e9 / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES_PER_STEP * K / launches
+                     if TRAFFIC_BYTES_PER_STEP else None,
+                     "launches": launches, "algorithmic_bytes_per_launch": alg, "us_per_launch": per_launch * 1e6,
+                     "algorithmic_bytes_per_step": alg_step, "us_per_step": dev / K * 1e6},
     }
     if not args.no_kernels:
         line["kernels"] = [bench_state_update(torch)] + bench_propagation(torch)
     if args.cpu_steps > 0:
-        line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, args.cpu_steps)
+        line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, min(args.cpu_steps, W + K))
     print(json.dumps(line))
 
 

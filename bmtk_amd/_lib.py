@@ -37,6 +37,7 @@ class Glif3Sim(C.Structure):
 SIGNATURES = {
     "bmtk_amd_abi_version": (c_int32, []),
     "bmtk_amd_last_error": (C.c_char_p, []),
+    "bmtk_glif3_sim_sizeof": (c_int64, []),
     "bmtk_glif3_precompute": (c_int32, [c_int64, c_void_p, c_double, c_void_p, c_void_p]),
     "bmtk_glif3_step_fwd": (c_int32, [c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int32, c_void_p,
@@ -76,6 +77,9 @@ def load(build_if_missing=True):
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = res, args
+    if lib.bmtk_glif3_sim_sizeof() != C.sizeof(Glif3Sim):
+        raise LibraryMissing("{} was built from a different include/bmtk_amd.h (struct size {} vs {}); rebuild it"
+                             .format(LIB_PATH, lib.bmtk_glif3_sim_sizeof(), C.sizeof(Glif3Sim)))
     _lib = lib
     return lib
 

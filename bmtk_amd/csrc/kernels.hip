@@ -317,6 +317,8 @@ int bmtk_amd_abi_version(void) { return 1; }
 
 const char *bmtk_amd_last_error(void) { return g_error; }
 
+int64_t bmtk_glif3_sim_sizeof(void) { return (int64_t)sizeof(bmtk_glif3_sim); }
+
 int bmtk_glif3_precompute(int64_t n, const double *par, double h, float *prop, void *stream)
 {
     BMTK_REQUIRE(n > 0 && par && prop, "glif3_precompute: n must be positive and pointers non-null");

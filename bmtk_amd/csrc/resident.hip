@@ -23,6 +23,8 @@
 // Every wait is bounded: a workgroup that spins too long on the barrier raises
 // the abort word, every other workgroup sees it and all leave the loop, so the
 // grid always drains.
+#include <stdlib.h>
+
 #include "glif3_update.hpp"
 #include "sim_internal.hpp"
 
@@ -372,15 +374,32 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
         set_error("glif3_simulate_fwd: resident mode needs %zu bytes of LDS: %s", lds, hipGetErrorString(err));
         return BMTK_E_LAUNCH;
     }
+    const unsigned grid = 8u * (unsigned)((s.res_groups + 7) / 8);
+    // every workgroup must be on the device at once: the grid barrier has no other way to fill
+    int dev = 0, n_cu = 0, per_cu = 0;
+    (void)hipGetDevice(&dev);
+    (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, sim_resident_kernel, kResBlock, lds);
+    if ((int64_t)per_cu * n_cu < (int64_t)grid) {
+        set_error("glif3_simulate_fwd: %u resident workgroups do not fit the device (%d compute units x %d)", grid,
+                  n_cu, per_cu);
+        return BMTK_E_LAUNCH;
+    }
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, stream, s.res_sync, 4);
     bmtk_glif3_sim s_copy = s;
-    void *args[] = {&s_copy, &r};
-    const unsigned grid = 8u * (unsigned)((s.res_groups + 7) / 8);
-    err = hipLaunchCooperativeKernel(reinterpret_cast<const void *>(sim_resident_kernel), dim3(grid),
-                                     dim3(kResBlock), args, lds, stream);
+    // BMTK_AMD_PLAIN_LAUNCH=1 uses an ordinary launch (co-residency then rests on the occupancy check
+    // above and an otherwise idle device); for tools that cannot follow cooperative launches.
+    const char *plain = getenv("BMTK_AMD_PLAIN_LAUNCH");
+    if (plain && plain[0] == '1') {
+        hipLaunchKernelGGL(sim_resident_kernel, dim3(grid), dim3(kResBlock), lds, stream, s_copy, r);
+        err = hipGetLastError();
+    } else {
+        void *args[] = {&s_copy, &r};
+        err = hipLaunchCooperativeKernel(reinterpret_cast<const void *>(sim_resident_kernel), dim3(grid),
+                                         dim3(kResBlock), args, lds, stream);
+    }
     if (err != hipSuccess) {
-        set_error("glif3_simulate_fwd: cooperative launch of %d workgroups failed: %s", s.res_groups,
-                  hipGetErrorString(err));
+        set_error("glif3_simulate_fwd: launch of %u resident workgroups failed: %s", grid, hipGetErrorString(err));
         return BMTK_E_LAUNCH;
     }
     return BMTK_OK;

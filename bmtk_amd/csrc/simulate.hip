@@ -16,7 +16,6 @@
 // launch of slack: slot t must be complete when launch t+1 starts, not when
 // launch t starts, so the delivery of step t-1 runs concurrently with the
 // update of step t instead of after it.
-#include <stdlib.h>
 #include "common.hpp"
 #include "glif3_update.hpp"
 #include "propagate.hpp"
@@ -273,18 +272,14 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     const size_t table_bytes = (size_t)s.prop_stride * GLIF3_NPROP * sizeof(float);
     q.lds_table = (s.class_id && table_bytes <= (size_t)kLdsTableBytes) ? 1 : 0;
     const size_t lds = q.lds_table ? table_bytes : 0;
-    const char *dbg_env = getenv("BMTK_SIM_DEBUG");
-    const int dbg = dbg_env ? atoi(dbg_env) : 0;
-    if (dbg & 4) q.n_deliver = 32;
-    if (dbg & 8) q.n_deliver = 256;
     for (int64_t k = 0; k <= n_steps; ++k) {
         const bool closing = k == n_steps;
         q.t = step0 + k;
         q.out_row = k;
         q.do_update = closing ? 0 : 1;
         q.fold_prev = k > 0;
-        q.deliver_prev = (k > 0 && has_rec && !(dbg & 1)) ? 1 : 0;
-        q.n_input = (k > 0 && !(dbg & 2)) ? n_input : 0;
+        q.deliver_prev = (k > 0 && has_rec) ? 1 : 0;
+        q.n_input = k > 0 ? n_input : 0;
         const unsigned grid = (unsigned)(q.n_update + q.n_deliver + q.n_input);
         hipLaunchKernelGGL(sim_step_kernel, dim3(grid), dim3(kSimBlock), lds, (hipStream_t)stream, s, q);
     }

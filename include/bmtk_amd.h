@@ -49,6 +49,8 @@ extern "C" {
 
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
+/* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
+int64_t bmtk_glif3_sim_sizeof(void);
 
 /* NEST glif_psc::pre_run_hook, run when bmtk calls nest.Create('glif_psc', n,
  * params) (bmtk/simulator/pointnet/sonata_adaptors.py:64-66): NEST-unit

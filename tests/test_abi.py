@@ -1,0 +1,73 @@
+"""The C ABI library loads without a GPU and exports every symbol the header
+declares; the Python mirrors of its tables and struct agree with the header."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from bmtk_amd import _lib, layout
+from oracle import glif3_oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    txt = open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    return sorted(set(re.findall(r"\b(bmtk_[a-z0-9_]+)\s*\(", txt)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert len(names) >= 12
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
+    assert lib.bmtk_amd_abi_version() >= 1
+
+
+def test_struct_mirror_matches_the_header():
+    lib = _lib.load()
+    assert lib.bmtk_glif3_sim_sizeof() == ctypes.sizeof(_lib.Glif3Sim)
+    txt = open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()
+    body = re.search(r"typedef struct bmtk_glif3_sim \{(.*?)\} bmtk_glif3_sim;", txt, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        for part in decl.split(","):
+            fields.append(re.findall(r"[A-Za-z_][A-Za-z0-9_]*", part)[-1])
+    assert fields == [f[0] for f in _lib.Glif3Sim._fields_]
+
+
+def test_layout_mirror_matches_the_header():
+    L = orc.L    # parsed from include/bmtk_amd_layout.h
+    assert L["GLIF3_NPROP"] == layout.NPROP and L["GLIF3_NPARAM"] == layout.NPARAM
+    for name, i in layout.PROP.items():
+        assert L["GLIF3_" + name] == i
+    for name, i in layout.PAR.items():
+        assert L["GLIF3_PAR_" + name] == i
+
+
+def test_argument_validation_needs_no_gpu():
+    lib = _lib.load()
+    assert lib.bmtk_glif3_precompute(0, None, 0.1, None, None) == -1
+    assert b"precompute" in lib.bmtk_amd_last_error()
+    assert lib.bmtk_spikes_compact_workspace_bytes(0) == 0
+    assert lib.bmtk_spikes_compact_workspace_bytes(1 << 20) > (1 << 20) // 8
+    assert lib.bmtk_glif3_simulate_fwd(None, 0, 1, None) == -1
+    with pytest.raises(_lib.BmtkAmdError):
+        _lib.check(lib.bmtk_csr_pack(-1, None, None, None, None, None, None))
+
+
+def test_ops_refuse_to_run_without_a_gpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from bmtk_amd import ops
+    with pytest.raises(RuntimeError):
+        ops.Glif3State.zeros(4)

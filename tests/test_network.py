@@ -1,0 +1,47 @@
+"""Host-side edge assembly rules (bmtk/simulator/pointnet/sonata_adaptors.py:268-357,
+bmtk/simulator/pointnet/pointnetwork.py:229-248)."""
+import numpy as np
+import pytest
+
+from bmtk_amd import network as net
+
+
+def test_weight_is_nsyns_times_syn_weight():
+    np.testing.assert_array_equal(net.edge_weights(np.array([1, 2, 3]), 2.5), [2.5, 5.0, 7.5])
+    assert net.edge_weights(None, -6.5) == -6.5
+    with pytest.raises(Exception, match="syn_weight"):
+        net.edge_weights(np.array([1]), None)
+
+
+def test_syn_spec_conversion():
+    w, d, r = net.syn_spec_to_arrays(3, {"weight": np.array([1.0, 2.0, 3.0]), "delay": 2.0, "receptor_type": 3}, dt=0.5)
+    assert w.dtype == np.float32 and d.tolist() == [4, 4, 4] and r.tolist() == [2, 2, 2]
+    w, d, r = net.syn_spec_to_arrays(2, {"weight": 5.0, "delay": np.array([1.0, 1.6])}, dt=1.0)
+    assert w.tolist() == [5.0, 5.0] and d.tolist() == [1, 2] and r.tolist() == [0, 0]
+
+
+def test_bad_delay_and_receptor():
+    with pytest.raises(net.BadDelay):
+        net.syn_spec_to_arrays(1, {"weight": 1.0, "delay": 0.05}, dt=0.1)
+    with pytest.raises(ValueError):
+        net.syn_spec_to_arrays(1, {"weight": 1.0, "delay": 1.0, "receptor_type": 5}, dt=0.1)
+    with pytest.raises(ValueError):
+        net.syn_spec_to_arrays(1, {"weight": 1.0, "delay": 1.0, "receptor_type": 0}, dt=0.1)
+    with pytest.raises(ValueError):
+        net.syn_spec_to_arrays(1, {"weight": 1.0, "delay": 300.0}, dt=1.0)
+
+
+def test_check_csr_rejects_what_a_kernel_would_trip_over():
+    good = net.coo_to_csr([0, 1], [1, 0], [1.0, 2.0], [1, 2], [0, 3], n_rows=2, major="source")
+    net.check_csr(good, 2, 2, 3)
+    indptr, indices, w, d, r = good
+    with pytest.raises(ValueError):
+        net.check_csr((indptr, indices + 5, w, d, r), 2, 2, 3)
+    with pytest.raises(ValueError):
+        net.check_csr((indptr, indices, w, d, r), 2, 2, 2)           # delay 2 needs 3 slots
+    with pytest.raises(ValueError):
+        net.check_csr((indptr[::-1].copy(), indices, w, d, r), 2, 2, 3)
+    with pytest.raises(ValueError):
+        net.check_csr((indptr, indices, w[:1], d, r), 2, 2, 3)
+    with pytest.raises(ValueError):
+        net.coo_to_csr([5], [0], [1.0], [1], [0], n_rows=2, major="source")
