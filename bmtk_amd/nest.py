@@ -1,0 +1,464 @@
+"""A PyNEST-shaped front end over the GPU path.
+
+bmtk's PointNet driver talks to its engine only through the ``nest`` module:
+``ResetKernel``/``SetKernelStatus`` (bmtk/simulator/pointnet/pointsimulator.py:73-74),
+``Create`` (bmtk/simulator/pointnet/sonata_adaptors.py:64-66,
+bmtk/simulator/pointnet/pointnetwork.py:198, modules/record_spikes.py:56-64),
+``Connect`` (pointnetwork.py:229-232, record_spikes.py:136), ``SetStatus``
+(pointnetwork.py:49,61), ``Simulate`` (pointsimulator.py:159-166),
+``GetStatus``/``GetConnections`` (bmtk/tests/simulator/pointnet/test_glif_utils.py:42,
+test_pointnetwork.py:43), ``Rank``/``NumProcesses``/``SyncProcesses``
+(bmtk/simulator/pointnet/io_tools.py:33-50).  This module offers the same names
+with the same argument meaning for the part of that surface the GLIF3 path
+covers, so ``import bmtk_amd.nest as nest`` can stand where ``import nest``
+does.  Supported models: ``glif_psc`` (LIF and LIF with after-spike currents),
+``spike_generator``, ``spike_recorder``/``spike_detector``,
+``step_current_generator``; ``static_synapse`` connections.  Anything else
+raises ``NESTError`` rather than being approximated.
+
+Nodes are numbered from 1 in creation order, as NEST does.  The network is
+assembled on the first ``Simulate`` call; ``Create``/``Connect`` after that
+raise.
+"""
+import os
+
+import numpy as np
+
+from . import network as _net
+from .glif_utils import params_table
+
+__version__ = "3.3-bmtk_amd"
+
+
+def version():
+    return "NEST " + __version__
+
+
+class NESTError(Exception):
+    """Base of the errors this front end raises (NEST's ``nest.kernel.NESTError``)."""
+
+    def __init__(self, message, errorname=None):
+        super().__init__(message)
+        self.errorname = errorname or type(self).__name__
+        self.errormessage = message
+
+
+class _Errors:
+    NESTError = NESTError
+
+    class BadDelay(NESTError):
+        pass
+
+    class BadProperty(NESTError):
+        pass
+
+    class UnknownModelName(NESTError):
+        pass
+
+    class UnknownReceptorType(NESTError):
+        pass
+
+
+class _Kernel:
+    NESTErrors = _Errors
+    NESTError = NESTError
+
+
+kernel = _Kernel()
+
+
+class NodeCollection(object):
+    """An ordered set of node ids (NEST 3's ``NodeCollection``)."""
+
+    def __init__(self, ids):
+        self._ids = [int(i) for i in ids]
+
+    def tolist(self):
+        return list(self._ids)
+
+    def __len__(self):
+        return len(self._ids)
+
+    def __iter__(self):
+        return (NodeCollection([i]) for i in self._ids)
+
+    def __getitem__(self, k):
+        got = self._ids[k]
+        return NodeCollection(got if isinstance(got, list) else [got])
+
+    def __add__(self, other):
+        return NodeCollection(self._ids + _ids_of(other))
+
+    def __repr__(self):
+        return "NodeCollection({})".format(self._ids if len(self._ids) < 8 else "{} nodes".format(len(self._ids)))
+
+
+def _ids_of(nodes):
+    if isinstance(nodes, NodeCollection):
+        return nodes.tolist()
+    if np.isscalar(nodes):
+        return [int(nodes)]
+    return [int(i) for i in nodes]
+
+
+_NEURON, _GENERATOR, _RECORDER, _CURRENT = "glif_psc", "spike_generator", "spike_recorder", "step_current_generator"
+_MODELS = {"glif_psc": _NEURON, "spike_generator": _GENERATOR, "spike_recorder": _RECORDER,
+           "spike_detector": _RECORDER, "step_current_generator": _CURRENT}
+
+
+class _State(object):
+    def __init__(self):
+        self.status = {"resolution": 0.1, "overwrite_files": False, "print_time": False, "local_num_threads": 1,
+                       "min_delay": 0.1, "max_delay": 0.1, "biological_time": 0.0, "data_path": "", "data_prefix": ""}
+        self.kind = []          # per node (index = id-1)
+        self.params = []        # per node dict
+        self.edges = []         # (src ids, tgt ids, weights f64, delay ms f64, receptor 1-based)
+        self.rec_links = []     # (neuron ids, recorder id)
+        self.cur_links = []     # (generator id, neuron ids)
+        self.sim = None         # built Glif3Simulator and its id maps
+        self.events = {}        # recorder id -> (senders, times)
+
+
+_S = _State()
+
+
+def ResetKernel():
+    global _S
+    _S = _State()
+    _written.clear()
+
+
+def SetKernelStatus(params):
+    if _S.sim is not None and "resolution" in params:
+        raise NESTError("resolution cannot change after the network has been simulated")
+    if "resolution" in params and not params["resolution"] > 0:
+        raise _Errors.BadProperty("resolution must be positive")
+    _S.status.update(params)
+    if "resolution" in params and not _S.edges:
+        _S.status["min_delay"] = _S.status["max_delay"] = params["resolution"]
+
+
+def GetKernelStatus(keys=None):
+    if keys is None:
+        return dict(_S.status)
+    if isinstance(keys, str):
+        return _S.status[keys]
+    return tuple(_S.status[k] for k in keys)
+
+
+def Rank():
+    return 0
+
+
+def NumProcesses():
+    return 1
+
+
+def SyncProcesses():
+    return None
+
+
+def set_verbosity(level):
+    return None
+
+
+def Install(module):
+    raise NESTError("dynamic modules are not supported: glif_psc is built in", "DynamicModuleManagementError")
+
+
+def CopyModel(existing, new, params=None):
+    raise NESTError("CopyModel is not supported by this front end")
+
+
+def Create(model, n=1, params=None):
+    if _S.sim is not None:
+        raise NESTError("nodes cannot be created after the first Simulate")
+    if model not in _MODELS:
+        raise _Errors.UnknownModelName("model '{}' is not available on the GPU path".format(model))
+    kind = _MODELS[model]
+    first = len(_S.kind) + 1
+    plist = params if isinstance(params, (list, tuple)) else [params] * n
+    if len(plist) != n:
+        raise _Errors.BadProperty("need one parameter dictionary per node")
+    for p in plist:
+        p = dict(p or {})
+        if kind == _NEURON:
+            _check_neuron(p)
+        _S.kind.append(kind)
+        _S.params.append(p)
+    nodes = NodeCollection(range(first, first + n))
+    for p_i, node in zip(plist, nodes.tolist()):
+        if kind in (_GENERATOR, _CURRENT) and p_i:
+            _set_one(node, dict(p_i))
+    return nodes
+
+
+_GLIF_DEFAULTS = dict(V_m=-78.85, V_th=-51.68, g=9.43, E_L=-78.85, C_m=58.72, t_ref=3.75, V_reset=-78.85,
+                      asc_init=(0.0, 0.0), asc_decay=(0.003, 0.1), asc_amps=(-9.18, -198.94), asc_r=(1.0, 1.0),
+                      tau_syn=(2.0,), spike_dependent_threshold=False, after_spike_currents=False,
+                      adapting_threshold=False)
+
+
+def _check_neuron(p):
+    full = dict(_GLIF_DEFAULTS)
+    full.update(p)
+    try:
+        params_table([full])
+    except NotImplementedError as exc:
+        raise _Errors.BadProperty(str(exc))
+    except ValueError as exc:
+        raise _Errors.BadProperty(str(exc))
+    p.clear()
+    p.update(full)
+
+
+def _set_one(node, params):
+    kind = _S.kind[node - 1]
+    if kind == _GENERATOR and "spike_times" in params:
+        st = np.array(params["spike_times"], np.float64)
+        if st.size and (np.any(st <= 0.0) or np.any(np.diff(st) < 0)):
+            raise _Errors.BadProperty("spike_times must be strictly positive and sorted")
+        dt = _S.status["resolution"]
+        if st.size and not params.get("allow_offgrid_times", _S.params[node - 1].get("allow_offgrid_times", False)) \
+                and not params.get("precise_times", _S.params[node - 1].get("precise_times", False)):
+            if np.any(np.abs(st / dt - np.rint(st / dt)) > 1e-6):
+                raise _Errors.BadProperty("spike_times must be multiples of the resolution unless precise_times "
+                                          "or allow_offgrid_times is set")
+    if kind == _GENERATOR and "spike_weights" in params:
+        sw = np.atleast_1d(np.asarray(params["spike_weights"], np.float64))
+        if sw.size and np.any(sw != sw[0]):
+            raise NESTError("per-spike spike_weights that differ are not supported")
+    _S.params[node - 1].update(params)
+
+
+def SetStatus(nodes, params, val=None):
+    if isinstance(params, str):
+        params = {params: val}
+    ids = _ids_of(nodes)
+    plist = params if isinstance(params, (list, tuple)) else [params] * len(ids)
+    for node, p in zip(ids, plist):
+        if _S.sim is not None and _S.kind[node - 1] != _RECORDER:
+            raise NESTError("node parameters cannot change after the first Simulate")
+        _set_one(node, dict(p))
+
+
+def GetStatus(nodes, keys=None):
+    out = []
+    for node in _ids_of(nodes):
+        d = dict(_S.params[node - 1])
+        d["model"] = _S.kind[node - 1]
+        if _S.kind[node - 1] == _RECORDER:
+            senders, times = _S.events.get(node, (np.zeros(0, np.int64), np.zeros(0)))
+            d["events"] = {"senders": senders, "times": times}
+            d["n_events"] = len(times)
+        out.append(d if keys is None else d[keys] if isinstance(keys, str) else tuple(d[k] for k in keys))
+    return tuple(out)
+
+
+def Connect(pre, post, conn_spec=None, syn_spec=None):
+    if _S.sim is not None:
+        raise NESTError("connections cannot be created after the first Simulate")
+    src, tgt = _ids_of(pre), _ids_of(post)
+    rule = conn_spec if isinstance(conn_spec, str) else (conn_spec or {}).get("rule", "all_to_all")
+    kinds_src = {_S.kind[i - 1] for i in src}
+    kinds_tgt = {_S.kind[i - 1] for i in tgt}
+    if kinds_tgt == {_RECORDER}:
+        if kinds_src != {_NEURON}:
+            raise NESTError("only neurons can be connected to a spike recorder")
+        for r in tgt:
+            _S.rec_links.append((np.array(src, np.int64), r))
+        return
+    if kinds_src == {_CURRENT}:
+        if kinds_tgt != {_NEURON}:
+            raise NESTError("a current generator connects to neurons")
+        for g in src:
+            _S.cur_links.append((g, np.array(tgt, np.int64)))
+        return
+    if not kinds_src <= {_NEURON, _GENERATOR} or kinds_tgt != {_NEURON}:
+        raise NESTError("unsupported connection {} -> {}".format(sorted(kinds_src), sorted(kinds_tgt)))
+    if rule == "one_to_one":
+        if len(src) != len(tgt):
+            raise NESTError("one_to_one needs as many sources as targets", "DimensionMismatch")
+        s, t = np.array(src, np.int64), np.array(tgt, np.int64)
+    elif rule == "all_to_all":
+        s, t = np.repeat(np.array(src, np.int64), len(tgt)), np.tile(np.array(tgt, np.int64), len(src))
+    else:
+        raise NESTError("connection rule '{}' is not supported".format(rule))
+    spec = dict(syn_spec or {})
+    model = spec.get("synapse_model", spec.get("model", "static_synapse"))
+    if model != "static_synapse":
+        raise _Errors.UnknownModelName("synapse model '{}' is not available on the GPU path".format(model))
+    dt = _S.status["resolution"]
+    n = s.size
+    spec.setdefault("weight", 1.0)
+    spec.setdefault("delay", 1.0)
+    spec.setdefault("receptor_type", 1)
+    try:
+        w, steps, rec0 = _net.syn_spec_to_arrays(n, spec, dt)
+    except _net.BadDelay as exc:
+        raise _Errors.BadDelay(str(exc), "BadDelay")
+    except ValueError as exc:
+        raise _Errors.UnknownReceptorType(str(exc)) if "receptor" in str(exc) else _Errors.BadProperty(str(exc))
+    n_rec = max(len(np.atleast_1d(_S.params[i - 1]["tau_syn"])) for i in set(t.tolist()))
+    if int(rec0[0]) + 1 > n_rec:
+        raise _Errors.UnknownReceptorType("receptor_type {} exceeds the {} receptor ports of the target".format(
+            int(rec0[0]) + 1, n_rec))
+    delay_ms = np.broadcast_to(np.asarray(spec["delay"], np.float64), (n,))
+    _S.edges.append((s, t, np.broadcast_to(np.asarray(spec["weight"], np.float64), (n,)).copy(), delay_ms.copy(),
+                     int(rec0[0]) + 1))
+    _S.status["min_delay"] = float(min(_S.status["min_delay"], delay_ms.min())) if len(_S.edges) > 1 \
+        else float(delay_ms.min())
+    _S.status["max_delay"] = float(max(_S.status["max_delay"], delay_ms.max()))
+
+
+def GetConnections(source=None, target=None):
+    out = []
+    for s, t, w, d, r in _S.edges:
+        out.extend(zip(s.tolist(), t.tolist()))
+    for ids, r in _S.rec_links:
+        out.extend((int(i), r) for i in ids)
+    for g, ids in _S.cur_links:
+        out.extend((g, int(i)) for i in ids)
+    return out
+
+
+def _build():
+    """Assemble the device simulator from everything created and connected so far."""
+    from .simulator import Glif3Simulator
+    dt = _S.status["resolution"]
+    kinds = np.array(_S.kind)
+    neuron_ids = np.flatnonzero(kinds == _NEURON) + 1
+    gen_ids = np.flatnonzero(kinds == _GENERATOR) + 1
+    if neuron_ids.size == 0:
+        raise NESTError("nothing to simulate: no glif_psc neurons were created")
+    n_of = np.full(len(kinds) + 1, -1, np.int64)
+    n_of[neuron_ids] = np.arange(neuron_ids.size)
+    g_of = np.full(len(kinds) + 1, -1, np.int64)
+    g_of[gen_ids] = np.arange(gen_ids.size)
+    par, asc_init, u_init = params_table([_S.params[i - 1] for i in neuron_ids])
+    rs, rt, rw, rd, rr = [], [], [], [], []
+    is_, it, iw, id_, ir = [], [], [], [], []
+    for s, t, w, d_ms, rec in _S.edges:
+        steps = np.rint(d_ms / dt).astype(np.int64)
+        from_gen = g_of[s] >= 0
+        for mask, (a, b, c, d, e), src_map in ((~from_gen, (rs, rt, rw, rd, rr), n_of),
+                                                (from_gen, (is_, it, iw, id_, ir), g_of)):
+            if mask.any():
+                ww = w[mask]
+                if src_map is g_of:   # a generator's uniform spike_weights multiply the synapse weight
+                    mult = np.array([np.atleast_1d(_S.params[i - 1].get("spike_weights", [1.0]))[0]
+                                     if len(np.atleast_1d(_S.params[i - 1].get("spike_weights", [1.0]))) else 1.0
+                                     for i in s[mask]])
+                    ww = ww * mult
+                a.append(src_map[s[mask]]); b.append(n_of[t[mask]]); c.append(ww); d.append(steps[mask])
+                e.append(np.full(int(mask.sum()), rec - 1))
+    cat = lambda xs, dt_: np.concatenate(xs).astype(dt_) if xs else np.zeros(0, dt_)
+    max_delay = int(max([1] + [int(x.max()) for x in rd + id_ if x.size]))
+    if max_delay > 62:
+        raise _Errors.BadDelay("delays above 62 steps do not fit the delay ring buffer", "BadDelay")
+    n = neuron_ids.size
+    rec = _net.coo_to_csr(cat(rs, np.int64), cat(rt, np.int64), cat(rw, np.float32), cat(rd, np.uint8),
+                          cat(rr, np.uint8), n_rows=n, major="source") if rs else None
+    inp = _net.coo_to_csr(cat(is_, np.int64), cat(it, np.int64), cat(iw, np.float32), cat(id_, np.uint8),
+                          cat(ir, np.uint8), n_rows=max(1, gen_ids.size), major="source") if is_ else None
+    sim = Glif3Simulator(n, par, dt, rec=rec, inp=inp, ring_slots=max_delay + 1, asc_init=asc_init, u_init=u_init)
+    _S.sim = dict(sim=sim, neuron_ids=neuron_ids, gen_ids=gen_ids, n_of=n_of, steps_done=0)
+
+
+def _current_at(step):
+    """Per-neuron external current (pA) used in update step `step`: a
+    step_current_generator's amplitude set at time T acts from the step that
+    starts at T + delay (its connection delay is one resolution, as bmtk sets it)."""
+    s = _S.sim
+    dt = _S.status["resolution"]
+    cur = np.zeros(s["neuron_ids"].size, np.float32)
+    t_ms = step * dt
+    for g, ids in _S.cur_links:
+        p = _S.params[g - 1]
+        times = np.atleast_1d(np.asarray(p.get("amplitude_times", []), np.float64))
+        amps = np.atleast_1d(np.asarray(p.get("amplitude_values", []), np.float64))
+        k = int(np.searchsorted(times + dt, t_ms + 1e-9, side="right")) - 1
+        if k >= 0:
+            cur[s["n_of"][ids]] += amps[k]
+    return cur
+
+
+def Simulate(t_ms):
+    from .spike_trains import bin_spike_times
+    import torch
+    dt = _S.status["resolution"]
+    n_steps = int(round(t_ms / dt))
+    if n_steps <= 0:
+        return
+    if _S.sim is None:
+        _build()
+    s = _S.sim
+    sim = s["sim"]
+    step0 = s["steps_done"]
+    if sim.inp is not None:
+        trains = []
+        for g in s["gen_ids"]:
+            st = np.asarray(_S.params[g - 1].get("spike_times", []), np.float64)
+            origin = float(_S.params[g - 1].get("origin", 0.0))
+            trains.append(st + origin if st.size else None)
+        in_ptr, in_ev = bin_spike_times(trains, dt, step0 + n_steps)
+        sim.set_input_events(in_ptr, in_ev)
+    # piecewise-constant external currents: run segment by segment
+    bounds = {step0, step0 + n_steps}
+    for g, ids in _S.cur_links:
+        for tt in np.atleast_1d(np.asarray(_S.params[g - 1].get("amplitude_times", []), np.float64)):
+            k = int(round((tt + dt) / dt))
+            if step0 < k < step0 + n_steps:
+                bounds.add(k)
+    bounds = sorted(bounds)
+    want_record = bool(_S.rec_links)
+    senders, times = [], []
+    for a, b in zip(bounds[:-1], bounds[1:]):
+        if _S.cur_links:
+            sim.i_ext = torch.as_tensor(_current_at(a), device=sim.dev)
+        cap = int(min(max(4096, (b - a) * sim.ne), 1 << 26)) if want_record else 0
+        out = sim.run(b - a, spike_bits=False, record_cap=cap)
+        if want_record:
+            rec = out["record"]
+            sim.check()
+            c = int(rec["count"].item())
+            if c > cap:
+                raise NESTError("more than {} spikes in one Simulate call; simulate in shorter pieces".format(cap))
+            st = rec["step"][:c].cpu().numpy().astype(np.float64)
+            fr = rec["frac"][:c].cpu().numpy().astype(np.float64)
+            el = rec["elem"][:c].cpu().numpy()
+            order = np.lexsort((el, st + fr))
+            # NEST stamps a spike at the end of its step and records stamp - offset, i.e. the
+            # interpolated threshold crossing (step + fraction) * resolution
+            times.append(((st + fr) * dt)[order])
+            senders.append(s["neuron_ids"][el[order]])
+    s["steps_done"] = step0 + n_steps
+    _S.status["biological_time"] = s["steps_done"] * dt
+    if want_record:
+        all_s, all_t = np.concatenate(senders), np.concatenate(times)
+        for ids, r in _S.rec_links:
+            keep = np.isin(all_s, ids)
+            old_s, old_t = _S.events.get(r, (np.zeros(0, np.int64), np.zeros(0)))
+            _S.events[r] = (np.concatenate([old_s, all_s[keep]]), np.concatenate([old_t, all_t[keep]]))
+            _write_ascii(r, all_s[keep], all_t[keep])
+
+
+def _write_ascii(recorder, senders, times):
+    """NEST 3 ``record_to: 'ascii'`` file, the form bmtk reads back
+    (bmtk/simulator/pointnet/modules/record_spikes.py:76-82): '#' comment
+    lines, a tab-separated header ``sender time_ms``, one row per spike."""
+    p = _S.params[recorder - 1]
+    if p.get("record_to") != "ascii" and not p.get("to_file", False):
+        return
+    label = p.get("label") or "spike_recorder"
+    path = os.path.join(_S.status.get("data_path", "") or "", "{}-{}-0.dat".format(label, recorder))
+    new = not os.path.exists(path) or (_S.status.get("overwrite_files") and recorder not in _written)
+    _written.add(recorder)
+    with open(path, "w" if new else "a") as f:
+        if new:
+            f.write("# NEST version: {}\n# RecordingBackendASCII version: 2\nsender\ttime_ms\n".format(__version__))
+        for sdr, t in zip(senders, times):
+            f.write("{}\t{:.3f}\n".format(int(sdr), t))
+
+
+_written = set()

@@ -211,25 +211,24 @@ def check_spike_times(st):
     return st
 
 
-def bin_spike_times(trains, dt, n_steps, batch=1, trial=0, precise_times=True):
+def bin_spike_times(trains, dt, n_steps, batch=1, trial=0):
     """Per-source spike times (ms) -> (in_ptr int64[n_steps+1], in_events int32[]).
 
     ``trains`` is a sequence indexed by source id (entries may be None).  A
-    spike at time t gets the stamp ``round(t/dt)`` steps (NEST ``spike_generator``
-    with on-grid delivery; ``precise_times`` only keeps the sub-step offset,
-    which ``static_synapse`` delivery ignores) and is emitted in step stamp-1.
-    An event is the element id ``source*batch + trial``; events of one step are
-    ascending.  Stamps of 0 (times below dt/2) cannot be emitted and raise, as
-    NEST does for a spike time that rounds to the current time.
+    spike at time t gets the stamp ``ceil(t/dt)`` steps (on-grid times keep
+    their step; an off-grid time is carried to the end of the step that
+    contains it, which is what NEST's ``spike_generator`` does with
+    ``precise_times`` -- the sub-step offset it also keeps is ignored by
+    ``static_synapse`` delivery) and is emitted in step stamp-1.  An event is
+    the element id ``source*batch + trial``; events of one step are ascending.
     """
     steps, elems = [], []
     for j, st in enumerate(trains):
         st = check_spike_times(st)
         if st is None:
             continue
-        stamp = np.rint(st / dt).astype(np.int64)
-        if np.any(stamp < 1):
-            raise ValueError("spike time rounds to step 0 at resolution {}".format(dt))
+        stamp = np.ceil(st / dt - 1e-6).astype(np.int64)
+        stamp = np.maximum(stamp, 1)
         emit = stamp - 1
         emit = emit[emit < n_steps]
         steps.append(emit)

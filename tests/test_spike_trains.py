@@ -102,5 +102,6 @@ def test_binning_to_step_events():
     assert ev.tolist() == [1, 5, 1, 5]
     in_ptr, ev = bin_spike_times(trains, dt=1.0, n_steps=10)
     assert in_ptr[-1] == 5 and ev[in_ptr[7]:in_ptr[8]].tolist() == [2]
-    with pytest.raises(ValueError):
-        bin_spike_times([[0.2]], dt=1.0, n_steps=4)
+    # off-grid times are carried to the end of their step; on-grid times stay put
+    in_ptr, ev = bin_spike_times([[0.2, 1.0, 1.01]], dt=1.0, n_steps=4)
+    assert in_ptr.tolist() == [0, 2, 3, 3, 3]
