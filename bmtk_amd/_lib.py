@@ -28,8 +28,24 @@ class Glif3Sim(C.Structure):
         ("res_span", c_int32), ("res_groups", c_int32), ("rec_seg", c_void_p), ("inp_seg", c_void_p),
         ("res_sync", c_void_p),
         ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
+        ("save_v", c_void_p), ("save_flags", c_void_p),
         ("spike_step", c_void_p), ("spike_elem", c_void_p), ("spike_frac", c_void_p),
         ("spike_cap", c_int64), ("spike_count", c_void_p),
+    ]
+
+
+class Glif3Bwd(C.Structure):
+    """``bmtk_glif3_bwd`` of include/bmtk_amd.h, field for field."""
+    _fields_ = [
+        ("n_neurons", c_int64), ("batch", c_int32), ("ring_slots", c_int32), ("h", c_float), ("dampening", c_float),
+        ("prop", c_void_p), ("prop_stride", c_int64), ("class_id", c_void_p),
+        ("save_v", c_void_p), ("save_flags", c_void_p), ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
+        ("rec_indptr", c_void_p), ("rec_packed", c_void_p),
+        ("in_ptr", c_void_p), ("in_events", c_void_p), ("inp_indptr", c_void_p), ("inp_packed", c_void_p),
+        ("dl_dz", c_void_p), ("dl_dz_const", c_void_p),
+        ("lam_V", c_void_p), ("lam_asc", c_void_p), ("lam_y1", c_void_p), ("lam_y2", c_void_p),
+        ("lam_ring", c_void_p), ("gz", c_void_p),
+        ("d_rec_w", c_void_p), ("d_inp_w", c_void_p),
     ]
 
 
@@ -38,6 +54,7 @@ SIGNATURES = {
     "bmtk_amd_abi_version": (c_int32, []),
     "bmtk_amd_last_error": (C.c_char_p, []),
     "bmtk_glif3_sim_sizeof": (c_int64, []),
+    "bmtk_glif3_bwd_sizeof": (c_int64, []),
     "bmtk_glif3_precompute": (c_int32, [c_int64, c_void_p, c_double, c_void_p, c_void_p]),
     "bmtk_glif3_step_fwd": (c_int32, [c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int32, c_void_p,
@@ -53,6 +70,8 @@ SIGNATURES = {
     "bmtk_csr_segment_offsets": (c_int32, [c_int64, c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p,
                                            c_void_p]),
     "bmtk_glif3_simulate_fwd": (c_int32, [C.POINTER(Glif3Sim), c_int64, c_int64, c_void_p]),
+    "bmtk_glif3_simulate_bwd": (c_int32, [C.POINTER(Glif3Bwd), c_int64, c_int64, c_void_p]),
+    "bmtk_spike_counts": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
 }
 
 
@@ -77,7 +96,7 @@ def load(build_if_missing=True):
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = res, args
-    if lib.bmtk_glif3_sim_sizeof() != C.sizeof(Glif3Sim):
+    if lib.bmtk_glif3_sim_sizeof() != C.sizeof(Glif3Sim) or lib.bmtk_glif3_bwd_sizeof() != C.sizeof(Glif3Bwd):
         raise LibraryMissing("{} was built from a different include/bmtk_amd.h (struct size {} vs {}); rebuild it"
                              .format(LIB_PATH, lib.bmtk_glif3_sim_sizeof(), C.sizeof(Glif3Sim)))
     _lib = lib

@@ -1,0 +1,281 @@
+// Reverse-time adjoint of the forward simulation: transposed propagation,
+// state adjoint, event-driven weight gradients.  The differentiable model
+// these kernels transpose is stated in include/bmtk_amd.h (bmtk_glif3_bwd).
+#include "common.hpp"
+#include "glif3_update.hpp"
+
+namespace bmtk {
+
+struct BwdStep {
+    int64_t t;    // absolute step being differentiated
+    int64_t row;  // its row in the forward record
+};
+
+__device__ __forceinline__ float surrogate(float U, float th, float dampening)
+{
+    const float vhat = (U - th) / th;
+    return dampening * fmaxf(0.0f, 1.0f - fabsf(vhat)) / th;
+}
+
+// gz[j*B+b] = sum over out-going synapses (j -> i, w, d, r) of w * lam_ring[(t+d)%L][r][i*B+b]:
+// one wavefront per source neuron and 64-trial tile, lane = trial.  Rows whose
+// every trial has a zero surrogate derivative in this step are skipped.
+__global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, BwdStep q)
+{
+    const int batch = a.batch;
+    const int64_t ne = a.n_neurons * (int64_t)batch;
+    const int L = a.ring_slots;
+    const int lane = lane_id();
+    const int64_t j = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (j >= a.n_neurons) return;
+    const int tile0 = blockIdx.y * kWave;
+    const bool lane_on = tile0 + lane < batch;
+    const int64_t e = j * batch + tile0 + lane;
+    bool active = false;
+    if (lane_on) {
+        const uint8_t f = a.save_flags[q.row * ne + e];
+        if (f & BMTK_F_INTEGRATING) {
+            const int64_t col = a.class_id ? (int64_t)a.class_id[j] : j;
+            const float th = a.prop[GLIF3_TH * a.prop_stride + col];
+            active = fabsf((a.save_v[q.row * ne + e] - th) / th) < 1.0f;
+        }
+    }
+    if (__ballot(active) == 0ull) {
+        if (lane_on) a.gz[e] = 0.0f;
+        return;
+    }
+    const int slot0 = (int)(q.t % L);
+    const int p0 = a.rec_indptr[j], p1 = a.rec_indptr[j + 1];
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.rec_packed);
+    const float *__restrict__ ring = a.lam_ring + tile0 + lane;
+    float acc = 0.0f;
+    for (int base = p0; base < p1; base += kWave) {
+        const int p = base + lane;
+        uint2 sy = make_uint2(0u, 0u);
+        if (p < p1) sy = rows[p];
+        const int n_here = min(kWave, p1 - base);
+        for (int l = 0; l < n_here; ++l) {
+            const unsigned tdr = (unsigned)bcast_i((int)sy.x, l);
+            const float w = __uint_as_float((unsigned)bcast_i((int)sy.y, l));
+            int slot = slot0 + (int)(tdr >> 26);
+            slot = slot >= L ? slot - L : slot;
+            const int r = (tdr >> 24) & 3;
+            const int64_t i = tdr & 0xFFFFFFu;
+            if (active) acc += w * ring[(int64_t)(slot * GLIF3_NREC + r) * ne + i * batch];
+        }
+    }
+    if (lane_on) a.gz[e] = acc;
+}
+
+// state adjoint of one step, one thread per element; writes the adjoint of
+// this step's arrivals into ring slot t
+__global__ __launch_bounds__(kBlock) void bwd_state_kernel(bmtk_glif3_bwd a, BwdStep q)
+{
+    const int64_t ne = a.n_neurons * (int64_t)a.batch;
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= ne) return;
+    const int64_t n = a.batch == 1 ? e : (int64_t)((uint32_t)e / (uint32_t)a.batch);
+    const int64_t col = a.class_id ? (int64_t)a.class_id[n] : n;
+    Glif3Prop p;
+    p.load(a.prop, a.prop_stride, col);
+    const uint8_t f = a.save_flags[q.row * ne + e];
+    float lV = a.lam_V[e];
+    float lA[GLIF3_NASC], l1[GLIF3_NREC], l2[GLIF3_NREC];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NASC; ++k) lA[k] = a.lam_asc[k * ne + e];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) {
+        l1[k] = a.lam_y1[k * ne + e];
+        l2[k] = a.lam_y2[k * ne + e];
+    }
+    // y1' = P11*y1 + psc0*s ; y2' = P21*y1 + P11*y2
+    float *slot = a.lam_ring + (int64_t)(q.t % a.ring_slots) * GLIF3_NREC * ne + e;
+    float n1[GLIF3_NREC], n2[GLIF3_NREC];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) {
+        slot[k * ne] = p.psc0[k] * l1[k];
+        n1[k] = p.P11[k] * l1[k] + (a.h * p.P11[k]) * l2[k];
+        n2[k] = p.P11[k] * l2[k];
+    }
+    float nV, nA[GLIF3_NASC];
+    if (f & BMTK_F_INTEGRATING) {
+        float g = a.gz[e];
+        if (a.dl_dz) g += a.dl_dz[q.row * ne + e];
+        if (a.dl_dz_const) g += a.dl_dz_const[e];
+        const float lU = lV + surrogate(a.save_v[q.row * ne + e], p.th, a.dampening) * g;
+        nV = p.P33 * lU;
+        const float lS = p.P30 * lU;
+#pragma unroll
+        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = p.c[k] * lS + p.d[k] * lA[k];
+#pragma unroll
+        for (int k = 0; k < GLIF3_NREC; ++k) {
+            n1[k] += p.P31[k] * lU;
+            n2[k] += p.P32[k] * lU;
+        }
+    } else if (f & BMTK_F_RESET) {
+        nV = 0.0f;
+#pragma unroll
+        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = p.r[k] * lA[k];
+    } else {
+        nV = lV;
+#pragma unroll
+        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = lA[k];
+    }
+    a.lam_V[e] = nV;
+#pragma unroll
+    for (int k = 0; k < GLIF3_NASC; ++k) a.lam_asc[k * ne + e] = nA[k];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) {
+        a.lam_y1[k * ne + e] = n1[k];
+        a.lam_y2[k * ne + e] = n2[k];
+    }
+}
+
+__device__ __forceinline__ unsigned long long trial_mask(const uint64_t *__restrict__ bits, int64_t j, int batch,
+                                                         int tile0, int width)
+{
+    const int64_t bit = j * batch + tile0;
+    const int64_t w = bit >> 6;
+    const int sh = (int)(bit & 63);
+    unsigned long long m = bits[w] >> sh;
+    if (sh + width > 64) m |= bits[w + 1] << (64 - sh);
+    if (width < 64) m &= (1ull << width) - 1ull;
+    return m;
+}
+
+// d_rec_w[p] += sum over trials b in which source j spiked in step t of
+// lam_ring[(t+d)%L][r][i*B+b]: one wavefront owns the whole row of a source, so
+// the accumulation needs no atomics; lane = synapse.
+__global__ __launch_bounds__(kBlock) void bwd_rec_grad_kernel(bmtk_glif3_bwd a, BwdStep q)
+{
+    const int batch = a.batch;
+    const int64_t ne = a.n_neurons * (int64_t)batch;
+    const int L = a.ring_slots;
+    const int64_t j = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (j >= a.n_neurons) return;
+    const uint64_t *__restrict__ bits = a.spike_bits + q.row * a.spike_bits_stride;
+    const int slot0 = (int)(q.t % L);
+    const int p0 = a.rec_indptr[j], p1 = a.rec_indptr[j + 1];
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.rec_packed);
+    for (int tile0 = 0; tile0 < batch; tile0 += kWave) {
+        const unsigned long long m = trial_mask(bits, j, batch, tile0, min(kWave, batch - tile0));
+        if (m == 0ull) continue;
+        for (int p = p0 + lane_id(); p < p1; p += kWave) {
+            const uint2 sy = rows[p];
+            int slot = slot0 + (int)(sy.x >> 26);
+            slot = slot >= L ? slot - L : slot;
+            const int r = (sy.x >> 24) & 3;
+            const int64_t i = sy.x & 0xFFFFFFu;
+            const float *cell = a.lam_ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch + tile0;
+            float acc = 0.0f;
+            unsigned long long mm = m;
+            while (mm) {
+                const int b = __ffsll((long long)mm) - 1;
+                mm &= mm - 1ull;
+                acc += cell[b];
+            }
+            a.d_rec_w[p] += acc;
+        }
+    }
+}
+
+// input weights: one wavefront per input event, atomics (several trials of one source may fire together)
+__global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, BwdStep q)
+{
+    const int batch = a.batch;
+    const int64_t ne = a.n_neurons * (int64_t)batch;
+    const int L = a.ring_slots;
+    const int slot0 = (int)(q.t % L);
+    const int64_t k0 = a.in_ptr[q.t], k1 = a.in_ptr[q.t + 1];
+    const int n_waves = gridDim.x * (kBlock / kWave);
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.inp_packed);
+    for (int64_t k = k0 + blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; k < k1; k += n_waves) {
+        const int ev = a.in_events[k];
+        const int j = batch == 1 ? ev : (int)((uint32_t)ev / (uint32_t)batch);
+        const int b = ev - j * batch;
+        const int p0 = a.inp_indptr[j], p1 = a.inp_indptr[j + 1];
+        for (int p = p0 + lane_id(); p < p1; p += kWave) {
+            const uint2 sy = rows[p];
+            int slot = slot0 + (int)(sy.x >> 26);
+            slot = slot >= L ? slot - L : slot;
+            const int r = (sy.x >> 24) & 3;
+            const int64_t i = sy.x & 0xFFFFFFu;
+            atomicAdd(a.d_inp_w + p, a.lam_ring[(int64_t)(slot * GLIF3_NREC + r) * ne + i * batch + b]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void fill_zero_kernel(float *x, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) x[i] = 0.0f;
+}
+
+__global__ __launch_bounds__(kBlock) void spike_counts_kernel(const uint64_t *__restrict__ bits, int64_t stride,
+                                                              int64_t n_steps, int64_t ne,
+                                                              int32_t *__restrict__ counts)
+{
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= ne) return;
+    const int64_t w = e >> 6;
+    const int sh = (int)(e & 63);
+    int c = 0;
+    for (int64_t k = 0; k < n_steps; ++k) c += (int)((bits[k * stride + w] >> sh) & 1ull);
+    counts[e] = c;
+}
+
+}  // namespace bmtk
+
+using namespace bmtk;
+
+extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_steps, void *stream)
+{
+    BMTK_REQUIRE(bwd != nullptr, "glif3_simulate_bwd: bwd is null");
+    const bmtk_glif3_bwd &a = *bwd;
+    BMTK_REQUIRE(a.n_neurons > 0 && a.batch > 0, "glif3_simulate_bwd: n_neurons and batch must be positive");
+    const int64_t ne = a.n_neurons * (int64_t)a.batch;
+    BMTK_REQUIRE(ne < (1ll << 31) && a.n_neurons < (1ll << 24), "glif3_simulate_bwd: network too large");
+    BMTK_REQUIRE(a.ring_slots > 1 && a.ring_slots <= 64, "glif3_simulate_bwd: ring_slots must lie in 2..64");
+    BMTK_REQUIRE(a.h > 0.0f && a.dampening >= 0.0f, "glif3_simulate_bwd: h must be positive, dampening non-negative");
+    BMTK_REQUIRE(a.prop && a.prop_stride > 0 && (a.class_id || a.prop_stride >= a.n_neurons),
+                 "glif3_simulate_bwd: prop table missing or too small");
+    BMTK_REQUIRE(a.save_v && a.save_flags && a.spike_bits, "glif3_simulate_bwd: the forward record is incomplete");
+    BMTK_REQUIRE(a.spike_bits_stride >= (ne + 63) / 64, "glif3_simulate_bwd: spike_bits_stride too small");
+    BMTK_REQUIRE(a.lam_V && a.lam_asc && a.lam_y1 && a.lam_y2 && a.lam_ring && a.gz,
+                 "glif3_simulate_bwd: adjoint state pointers must be non-null");
+    BMTK_REQUIRE(!(a.dl_dz && a.dl_dz_const), "glif3_simulate_bwd: give dl_dz or dl_dz_const, not both");
+    const bool has_rec = a.rec_indptr != nullptr;
+    BMTK_REQUIRE(!has_rec || a.rec_packed, "glif3_simulate_bwd: recurrent table needs rec_packed");
+    BMTK_REQUIRE(!a.d_rec_w || has_rec, "glif3_simulate_bwd: d_rec_w without a recurrent table");
+    const bool inp_grad = a.d_inp_w != nullptr;
+    BMTK_REQUIRE(!inp_grad || (a.in_ptr && a.in_events && a.inp_indptr && a.inp_packed),
+                 "glif3_simulate_bwd: d_inp_w needs the input events and the input table");
+    BMTK_REQUIRE(step0 >= 0 && n_steps >= 0, "glif3_simulate_bwd: step0 and n_steps must be non-negative");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned rows_grid = (unsigned)((a.n_neurons + kBlock / kWave - 1) / (kBlock / kWave));
+    const unsigned tiles = (unsigned)((a.batch + kWave - 1) / kWave);
+    const unsigned elem_grid = (unsigned)((ne + kBlock - 1) / kBlock);
+    for (int64_t k = n_steps - 1; k >= 0; --k) {
+        BwdStep q{step0 + k, k};
+        if (has_rec)
+            hipLaunchKernelGGL(bwd_gather_kernel, dim3(rows_grid, tiles), dim3(kBlock), 0, st, a, q);
+        else
+            hipLaunchKernelGGL(fill_zero_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a.gz, ne);
+        hipLaunchKernelGGL(bwd_state_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q);
+        if (a.d_rec_w) hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
+        if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(64), dim3(kBlock), 0, st, a, q);
+    }
+    BMTK_CHECK_LAUNCH("glif3_simulate_bwd");
+    return BMTK_OK;
+}
+
+extern "C" int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_steps, int64_t ne,
+                                 int32_t *counts, void *stream)
+{
+    BMTK_REQUIRE(spike_bits && counts && ne > 0 && n_steps >= 0 && stride >= (ne + 63) / 64,
+                 "spike_counts: bad sizes or null pointers");
+    hipLaunchKernelGGL(spike_counts_kernel, dim3((unsigned)((ne + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, spike_bits, stride, n_steps, ne, counts);
+    BMTK_CHECK_LAUNCH("spike_counts");
+    return BMTK_OK;
+}

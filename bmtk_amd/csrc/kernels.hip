@@ -319,6 +319,8 @@ const char *bmtk_amd_last_error(void) { return g_error; }
 
 int64_t bmtk_glif3_sim_sizeof(void) { return (int64_t)sizeof(bmtk_glif3_sim); }
 
+int64_t bmtk_glif3_bwd_sizeof(void) { return (int64_t)sizeof(bmtk_glif3_bwd); }
+
 int bmtk_glif3_precompute(int64_t n, const double *par, double h, float *prop, void *stream)
 {
     BMTK_REQUIRE(n > 0 && par && prop, "glif3_precompute: n must be positive and pointers non-null");

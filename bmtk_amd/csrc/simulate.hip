@@ -166,8 +166,15 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
             }
             const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
             const float I = s.i_ext ? s.i_ext[e] : 0.0f;
+            const int ref_before = st.ref;
             spike = glif3_update(st, p, s.h, zero, I, &frac);
             glif3_store(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
+            if (s.save_v) {
+                s.save_v[q.out_row * ne + e] = st.V;
+                s.save_flags[q.out_row * ne + e] = (uint8_t)((spike ? BMTK_F_SPIKE : 0) |
+                                                              (ref_before == 0 ? BMTK_F_INTEGRATING : 0) |
+                                                              (ref_before > 0 && st.ref == 0 ? BMTK_F_RESET : 0));
+            }
         }
     }
     if (!q.do_update) return;
@@ -248,6 +255,9 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
                  "glif3_simulate_fwd: spike record needs spike_step, spike_elem and a positive spike_cap");
     BMTK_REQUIRE(step0 >= 0 && n_steps >= 0, "glif3_simulate_fwd: step0 and n_steps must be non-negative");
     if (n_steps == 0) return BMTK_OK;
+    BMTK_REQUIRE((s.save_v == nullptr) == (s.save_flags == nullptr),
+                 "glif3_simulate_fwd: save_v and save_flags go together");
+    BMTK_REQUIRE(!(s.save_v && s.res_span > 0), "glif3_simulate_fwd: the per-step record needs launch-per-step mode");
     if (s.res_span > 0) {
         BMTK_REQUIRE(s.batch == 1, "glif3_simulate_fwd: resident mode runs batch 1 only");
         BMTK_REQUIRE(s.res_span % 64 == 0 && s.res_span <= 1024, "glif3_simulate_fwd: res_span must be a multiple of 64, at most 1024");

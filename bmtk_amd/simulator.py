@@ -159,10 +159,12 @@ class Glif3Simulator:
             s.spike_cap, s.spike_count = record["step"].numel(), _p(record["count"])
         return s
 
-    def run(self, n_steps, spike_bits=True, record_cap=0):
+    def run(self, n_steps, spike_bits=True, record_cap=0, save_state=False):
         """Advance ``n_steps`` steps.  Returns a dict with ``bits`` (int64
         [n_steps, words], spike bits per step) and, when ``record_cap`` > 0,
-        the atomic spike record with crossing fractions.  Does not synchronise."""
+        the atomic spike record with crossing fractions; ``save_state`` adds the
+        per-step record (potentials and flags) the backward pass reads.  Does not
+        synchronise."""
         if self.in_ptr is not None and self.step + n_steps > self.in_steps:
             raise ValueError("input event lists cover {} steps, run would reach {}".format(
                 self.in_steps, self.step + n_steps))
@@ -174,10 +176,17 @@ class Glif3Simulator:
                           frac=torch.zeros(record_cap, dtype=torch.float32, device=self.dev),
                           count=torch.zeros(1, dtype=torch.int64, device=self.dev))
         s = self._struct(bits, record)
+        saved = None
+        if save_state:
+            if self.res_span:
+                raise ValueError("save_state needs a simulator built with resident=False")
+            saved = dict(v=torch.empty(n_steps, self.ne, device=self.dev),
+                         flags=torch.empty(n_steps, self.ne, dtype=torch.uint8, device=self.dev), step0=self.step)
+            s.save_v, s.save_flags = _p(saved["v"]), _p(saved["flags"])
         _lib.check(self.lib.bmtk_glif3_simulate_fwd(C.byref(s), self.step, n_steps, _stream()))
         self.step += n_steps
         self._pending_check = bool(self.res_span)
-        return dict(bits=bits, record=record)
+        return dict(bits=bits, record=record, saved=saved)
 
     def spikes_from_bits(self, bits, step0=0):
         """Spike bits -> (step int64[], element int64[]) ascending, via the

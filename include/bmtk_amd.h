@@ -51,6 +51,7 @@ int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
 int64_t bmtk_glif3_sim_sizeof(void);
+int64_t bmtk_glif3_bwd_sizeof(void);
 
 /* NEST glif_psc::pre_run_hook, run when bmtk calls nest.Create('glif_psc', n,
  * params) (bmtk/simulator/pointnet/sonata_adaptors.py:64-66): NEST-unit
@@ -167,6 +168,10 @@ typedef struct bmtk_glif3_sim {
     uint64_t *spike_bits;        /* [n_steps][words] spike bits per step, words = ceil(ne/64); or NULL.
                                   * Row k belongs to step step0+k of the call that wrote it. */
     int64_t spike_bits_stride;   /* words per row (>= ceil(ne/64)) */
+    /* optional per-step record for the backward pass (launch-per-step mode only; both or neither):
+     * save_v[k][e] = membrane potential after step step0+k, save_flags[k][e] = BMTK_F_* bits */
+    float *save_v;
+    uint8_t *save_flags;
     /* optional spike record with sub-step crossing fractions, appended with
      * atomics (unordered within a step); all NULL to disable */
     int32_t *spike_step;
@@ -175,6 +180,10 @@ typedef struct bmtk_glif3_sim {
     int64_t spike_cap;
     unsigned long long *spike_count; /* device counter, keeps counting past spike_cap */
 } bmtk_glif3_sim;
+
+#define BMTK_F_SPIKE 1       /* the element spiked in this step */
+#define BMTK_F_INTEGRATING 2 /* it was not refractory when the step began */
+#define BMTK_F_RESET 4       /* it left refractoriness in this step (U and ASC were reset) */
 
 /* Run steps step0 .. step0+n_steps-1.  One launch per step plus one closing
  * launch.  A launch updates every element for step t while, in other
@@ -197,7 +206,67 @@ typedef struct bmtk_glif3_sim {
  * traffic.  The barrier spins a bounded number of times; see res_sync. */
 int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0, int64_t n_steps, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * Backward pass (reverse-time adjoint) of the forward simulation.
+ *
+ * bmtk and NEST have no gradient code: this part has no counterpart in the
+ * reference; its definition is this library's own and is stated here.
+ *  - The spike z = H(U' - th) gets the surrogate derivative
+ *      dz/dU' = dampening * max(0, 1 - |(U' - th)/th|) / th      (th = V_th - E_L)
+ *    in steps where the element was integrating; 0 otherwise.
+ *  - Refractory bookkeeping is not differentiated: the hold U' = U passes the
+ *    adjoint through, the reset U' = V_reset - E_L stops it, the after-spike
+ *    reset ASC' = amp + r*ASC passes r.
+ *  - Everything else is the exact transpose of the linear forward update.
+ * The loss enters through dl_dz[k][e] (its derivative with respect to the spike
+ * of element e in step step0+k), or through dl_dz_const[e] when it is the same
+ * in every step (a loss on time-averaged rates).
+ * Outputs: gradients with respect to every weight of the recurrent and input
+ * tables, in packed-table order, accumulated (+=) into d_rec_w / d_inp_w.
+ */
+typedef struct bmtk_glif3_bwd {
+    int64_t n_neurons;
+    int32_t batch;
+    int32_t ring_slots;
+    float h;
+    float dampening;
+    const float *prop;
+    int64_t prop_stride;
+    const int32_t *class_id;
+    /* forward record of the steps being differentiated, row k = step step0+k */
+    const float *save_v;           /* [n_steps][ne] */
+    const uint8_t *save_flags;     /* [n_steps][ne] */
+    const uint64_t *spike_bits;    /* [n_steps][spike_bits_stride] */
+    int64_t spike_bits_stride;
+    /* the tables the forward run used (source-major, packed) */
+    const int32_t *rec_indptr;
+    const bmtk_synapse *rec_packed;
+    const int64_t *in_ptr;         /* absolute step index, as in the forward run */
+    const int32_t *in_events;
+    const int32_t *inp_indptr;
+    const bmtk_synapse *inp_packed;
+    /* loss derivative: at most one of the two, the other NULL */
+    const float *dl_dz;            /* [n_steps][ne] */
+    const float *dl_dz_const;      /* [ne] */
+    /* adjoint state, in/out (zero before the last step of the whole run) */
+    float *lam_V, *lam_asc, *lam_y1, *lam_y2; /* [ne], [2][ne], [4][ne], [4][ne] */
+    float *lam_ring;               /* [L][4][ne]: adjoint of the arrivals of the steps still ahead */
+    float *gz;                     /* [ne] scratch */
+    /* outputs */
+    float *d_rec_w;                /* [rec nnz] or NULL */
+    float *d_inp_w;                /* [inp nnz] or NULL */
+} bmtk_glif3_bwd;
+
+/* Differentiate steps step0+n_steps-1 down to step0 (three launches per step:
+ * transposed propagation, state adjoint, weight gradients). */
+int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_steps, void *stream);
+
+/* Number of spikes of every element over n_steps rows of spike bits: counts[e] (int32). */
+int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_steps, int64_t ne, int32_t *counts,
+                      void *stream);
+
 #ifdef __cplusplus
 }
 #endif
 #endif
+

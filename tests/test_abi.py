@@ -28,11 +28,14 @@ def test_library_exports_every_declared_symbol():
     assert lib.bmtk_amd_abi_version() >= 1
 
 
-def test_struct_mirror_matches_the_header():
+@pytest.mark.parametrize("cname,mirror,sizeof", [("bmtk_glif3_sim", "Glif3Sim", "bmtk_glif3_sim_sizeof"),
+                                                 ("bmtk_glif3_bwd", "Glif3Bwd", "bmtk_glif3_bwd_sizeof")])
+def test_struct_mirror_matches_the_header(cname, mirror, sizeof):
     lib = _lib.load()
-    assert lib.bmtk_glif3_sim_sizeof() == ctypes.sizeof(_lib.Glif3Sim)
+    cls = getattr(_lib, mirror)
+    assert getattr(lib, sizeof)() == ctypes.sizeof(cls)
     txt = open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()
-    body = re.search(r"typedef struct bmtk_glif3_sim \{(.*?)\} bmtk_glif3_sim;", txt, flags=re.S).group(1)
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), txt, flags=re.S).group(1)
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
     fields = []
     for decl in body.split(";"):
@@ -41,7 +44,7 @@ def test_struct_mirror_matches_the_header():
             continue
         for part in decl.split(","):
             fields.append(re.findall(r"[A-Za-z_][A-Za-z0-9_]*", part)[-1])
-    assert fields == [f[0] for f in _lib.Glif3Sim._fields_]
+    assert fields == [f[0] for f in cls._fields_]
 
 
 def test_layout_mirror_matches_the_header():

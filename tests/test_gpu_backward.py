@@ -1,0 +1,117 @@
+"""GPU adjoint (BPTT) kernels against torch.autograd over an independent fp64
+restatement of the same model.  Gradients have no counterpart in the
+reference (parity unpinned); the tolerance is the 1e-4 relative the build
+states, taken relative to the largest gradient magnitude of the table."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import glif3_oracle as orc
+from oracle import glif3_adjoint_ref as adj
+from bmtk_amd import synthetic, training
+from bmtk_amd.simulator import Glif3Simulator
+
+pytestmark = pytest.mark.gpu
+
+
+def _quarter_weights(csr):
+    indptr, indices, w, d, r = csr
+    return indptr, indices, (np.round(w * 4.0) / 4.0 + np.sign(w) * 0.25).astype(np.float32), d, r
+
+
+def _net(batch, seed, n=40, n_in=30, steps=70):
+    cfg = synthetic.small_glif3_network(n=n, n_in=n_in, steps=steps, seed=seed, in_rate=40.0, in_w_scale=15.0,
+                                        w_scale=4.0, in_fanout=n // 2, p_conn=0.2, batch=batch)
+    # exact weights keep the fp32 and fp64 forward rasters identical, so both sides differentiate the same run
+    cfg["rec_src"] = _quarter_weights(cfg["rec_src"])
+    cfg["inp_src"] = _quarter_weights(cfg["inp_src"])
+    return cfg
+
+
+def _rel(got, want):
+    return float(np.max(np.abs(got - want)) / max(np.max(np.abs(want)), 1e-30))
+
+
+@pytest.mark.parametrize("batch,seed,loss_kind", [(1, 2, "per_step"), (3, 4, "per_step"), (1, 5, "rates"), (4, 6, "rates")])
+def test_weight_gradients_match_autograd(batch, seed, loss_kind):
+    cfg = _net(batch, seed)
+    n, T, h = cfg["n"], cfg["steps"], cfg["h"]
+    ne = n * batch
+    prop = orc.precompute(cfg["par"], h)
+    rng = np.random.default_rng(seed)
+    sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                         resident=False)
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    fwd = sim.run(T, save_state=True)
+    ras = sim.raster(fwd["bits"]).cpu().numpy()
+    bptt = training.Glif3Bptt(sim, dampening=0.3)
+    if loss_kind == "per_step":
+        a = rng.normal(size=(T, ne))
+        loss_fn = lambda z: (z * torch.as_tensor(a)).sum()
+        bptt.backward(fwd, dl_dz=torch.as_tensor(a.astype(np.float32), device="cuda"))
+    else:
+        pop = rng.integers(0, 3, n)
+        targets = rng.uniform(0, 0.05, (batch, 3))
+        pop_t = torch.as_tensor(pop)
+
+        def loss_fn(z):
+            c = z.sum(0).view(n, batch)
+            size = torch.bincount(pop_t, minlength=3).to(z.dtype)
+            rate = torch.zeros(3, batch, dtype=z.dtype).index_add_(0, pop_t, c) / (size.view(-1, 1) * T)
+            return ((rate.t() - torch.as_tensor(targets)) ** 2).mean()
+        counts = training.spike_counts(fwd["bits"], ne)
+        np.testing.assert_array_equal(counts.cpu().numpy(), ras.sum(0))
+        loss, g = training.rate_mse(counts, T, batch, pop_t.cuda(), torch.as_tensor(targets, dtype=torch.float32,
+                                                                                    device="cuda"))
+        bptt.backward(fwd, dl_dz_const=g)
+    want = adj.simulate_with_grad(prop, h, T, n, batch, cfg["L"], cfg["rec_src"], cfg["inp_src"], cfg["in_ptr"],
+                                  cfg["in_events"], loss_fn, dampening=0.3)
+    np.testing.assert_array_equal(ras, want["raster"])
+    assert ras.sum() > 30 * batch
+    if loss_kind == "rates":
+        assert float(loss) == pytest.approx(want["loss"], rel=1e-5)
+    got_rec, got_inp = bptt.d_rec_w.cpu().numpy(), bptt.d_inp_w.cpu().numpy()
+    assert np.abs(want["d_rec_w"]).max() > 0 and np.abs(want["d_inp_w"]).max() > 0
+    assert _rel(got_rec, want["d_rec_w"]) < 1e-4
+    assert _rel(got_inp, want["d_inp_w"]) < 1e-4
+
+
+def test_chunked_backward_equals_one_call():
+    cfg = _net(2, 7)
+    n, T, h = cfg["n"], cfg["steps"], cfg["h"]
+    a = torch.as_tensor(np.random.default_rng(1).normal(size=(T, n * 2)).astype(np.float32), device="cuda")
+    grads = []
+    for chunks in ([T], [30, 25, 15]):
+        sim = Glif3Simulator(n, cfg["par"], h, batch=2, rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                             resident=False)
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        runs, k0 = [], 0
+        for c in chunks:
+            runs.append((sim.run(c, save_state=True), k0, c)); k0 += c
+        bptt = training.Glif3Bptt(sim)
+        for fwd, k0, c in reversed(runs):
+            bptt.backward(fwd, dl_dz=a[k0:k0 + c].contiguous())
+        grads.append((bptt.d_rec_w.cpu().numpy(), bptt.d_inp_w.cpu().numpy()))
+    np.testing.assert_allclose(grads[0][0], grads[1][0], rtol=0, atol=1e-6 * np.abs(grads[0][0]).max())
+    np.testing.assert_allclose(grads[0][1], grads[1][1], rtol=0, atol=1e-6 * np.abs(grads[0][1]).max())
+
+
+def test_backward_argument_errors():
+    cfg = _net(1, 3)
+    sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                         resident=True)
+    with pytest.raises(ValueError):
+        training.Glif3Bptt(sim)
+    with pytest.raises(ValueError):
+        sim.run(5, save_state=True)
+    sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                         resident=False)
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    bptt = training.Glif3Bptt(sim)
+    with pytest.raises(ValueError):
+        bptt.backward(sim.run(5))                                 # no record
+    from bmtk_amd._lib import BmtkAmdError
+    fwd = sim.run(5, save_state=True)
+    z = torch.zeros(5, cfg["n"], device="cuda")
+    with pytest.raises(BmtkAmdError):
+        bptt.backward(fwd, dl_dz=z, dl_dz_const=z[0].contiguous())
