@@ -147,6 +147,53 @@ def bench_propagation(torch, steps=200, warmup=20):
     return out
 
 
+def bench_bptt(torch, steps=600):
+    """One BPTT training step: 51,978 neurons (Poisson in-degree 1000, ~52 M synapses) plus 17,400
+    Poisson inputs at 5 Hz, batch 32, 600 steps; triangular surrogate (dampening 0.3); MSE between
+    the rates of 17 random populations and random targets; gradients for every recurrent and input
+    weight.  Recurrent weights are scaled by 0.2 and input weights by 2 so that the network settles
+    near 3 Hz (unit weights at this in-degree saturate it)."""
+    import numpy as np
+    from bmtk_amd import synthetic, training
+    from bmtk_amd.simulator import Glif3Simulator
+    n, n_in, batch = 51978, 17400, 32
+    rng = np.random.default_rng(4)
+    par = synthetic.random_cells(rng, n)
+    _, by_src, _ = synthetic.device_network(n, 1000, "poisson", seed=2, w_scale=0.2)
+    inp = synthetic.device_input_table(n_in, n, 8_000_000, seed=4, w_scale=2.0)
+    in_ptr, in_ev = synthetic.device_poisson_events(n_in, 5.0, 1.0, 2 * steps, batch=batch, seed=5)
+    sim = Glif3Simulator(n, par, 1.0, batch=batch, rec=by_src, inp=inp, resident=False)
+    sim.set_input_events(in_ptr, in_ev)
+    pop = torch.randint(0, 17, (n,), device="cuda")
+    targets = torch.rand(batch, 17, device="cuda") * 0.01
+    bptt = training.Glif3Bptt(sim, dampening=0.3)
+    res = {}
+
+    def fwd():
+        res["fwd"] = sim.run(steps, save_state=True)
+
+    def bwd():
+        counts = training.spike_counts(res["fwd"]["bits"], sim.ne)
+        res["loss"], g = training.rate_mse(counts, steps, batch, pop, targets)
+        res["counts"] = counts
+        bptt.zero()
+        bptt.backward(res["fwd"], dl_dz_const=g)
+
+    fwd(); bwd()                              # warm-up step (also leaves the transient from rest behind)
+    t_f, _ = time_region(torch, fwd)
+    t_b, _ = time_region(torch, bwd)
+    deg = (sim.rec.indptr[1:] - sim.rec.indptr[:-1]).long()
+    spikes = res["counts"].view(n, batch).sum(1)
+    events = int((spikes.long() * deg).sum().item())
+    return {"kernel": "sim_step_kernel + bwd_gather_kernel + bwd_state_kernel + bwd_rec_grad_kernel",
+            "workload": "BPTT step N=51978 nnz=%d inputs=17400 batch=32 steps=%d" % (sim.rec.nnz, steps),
+            "seconds_per_training_step": t_f + t_b, "forward_s": t_f, "backward_s": t_b,
+            "mean_rate_hz": float(res["counts"].float().mean().item()) / steps * 1e3,
+            "recurrent_events_forward": events, "loss": float(res["loss"]),
+            "weight_grad_events_per_s": events / t_b,
+            "grad_norm_rec": float(bptt.d_rec_w.norm().item()), "grad_norm_inp": float(bptt.d_inp_w.norm().item())}
+
+
 def cpu_baseline(torch, sim, par, class_id, sample_steps):
     """The NEST-algorithm CPU restatement (fp64, event-driven source-major
     delivery into per-neuron ring buffers, OpenMP) on the first `sample_steps`
@@ -251,7 +298,7 @@ def main():
                      "algorithmic_bytes_per_step": alg_step, "us_per_step": dev / K * 1e6},
     }
     if not args.no_kernels:
-        line["kernels"] = [bench_state_update(torch)] + bench_propagation(torch)
+        line["kernels"] = [bench_state_update(torch)] + bench_propagation(torch) + [bench_bptt(torch)]
     if args.cpu_steps > 0:
         line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, min(args.cpu_steps, W + K))
     print(json.dumps(line))
