@@ -126,13 +126,17 @@ def bench_propagation(torch, steps=200, warmup=20):
             zb[:-1] = (w << torch.arange(64, device="cuda")).sum(1)
             pool_bits.append(zb)
         events = sum(e for _, _, e in pool_ev) / len(pool_ev)
-        for mode in ("scatter", "gather"):
+        hist = torch.stack([pool_bits[k % 4] for k in range(L)])   # spike bits of the last L steps
+        syn = torch.zeros(4, ne, device="cuda")
+        for mode in ("scatter", "gather", "pull"):
             def one(k):
                 if mode == "scatter":
                     ids, count, _ = pool_ev[k % 4]
                     ops.csr_propagate_scatter(ids, count, t_src, ring, n, batch, k)
-                else:
+                elif mode == "gather":
                     ops.csr_propagate_gather(pool_bits[k % 4], n, t_tgt, ring, n, batch, k)
+                else:
+                    ops.csr_propagate_pull(hist, n, t_tgt, syn, n, batch, k + L)
             for k in range(warmup):
                 one(k)
             ring.zero_()

@@ -66,6 +66,9 @@ SIGNATURES = {
                                              c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "bmtk_csr_propagate_gather": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
+    "bmtk_csr_propagate_pull_workspace_bytes": (c_int64, [c_int32, c_int64]),
+    "bmtk_csr_propagate_pull": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
+                                          c_int64, c_int64, c_void_p, c_void_p]),
     "bmtk_csr_pack": (c_int32, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "bmtk_csr_segment_offsets": (c_int32, [c_int64, c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p,
                                            c_void_p]),

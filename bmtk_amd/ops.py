@@ -184,10 +184,16 @@ class SynapseTable:
     def nnz(self):
         return self.indices.numel()
 
+    def max_delay(self):
+        """Largest delay in steps (computed once; synchronises the first time)."""
+        if getattr(self, "_max_delay", None) is None:
+            self._max_delay = int(self.delays.max()) if self.nnz else 0
+        return self._max_delay
+
     def packed(self):
         """The table as 8-byte {index | receptor<<24 | delay<<26, weight} records (built once)."""
         if getattr(self, "_packed", None) is None:
-            if self.nnz and int(self.delays.max()) >= 64:
+            if self.max_delay() >= 64:
                 raise ValueError("packed tables hold delays below 64 steps")
             lib = _lib.load()
             out = torch.empty(max(self.nnz, 1), 2, dtype=torch.int32, device=self.indices.device)
@@ -247,6 +253,25 @@ def csr_propagate_gather(zbits, n_src, table, ring, n_tgt, batch, step):
     _lib.check(lib.bmtk_csr_propagate_gather(
         _p(zbits, torch.int64, n_words(n_src * batch) + 1, "zbits"), n_src, batch, *table.pointers(),
         _p(ring, torch.float32), L, n_tgt, int(step), _stream()))
+
+
+def csr_propagate_pull(spike_hist, n_src, table, syn, n_tgt, batch, t_arrive):
+    """Everything arriving in step ``t_arrive`` from the spike bits of the last L steps
+    (``spike_hist`` int64 [L, words+1], row k mod L = bits of step k) through a target-major table;
+    overwrites ``syn`` [4, n_tgt*batch]."""
+    lib = _lib.load()
+    if table.n_rows != n_tgt or syn.numel() != NREC * n_tgt * batch:
+        raise ValueError("target-major table must have one row per target and syn must be [4, n_tgt*batch]")
+    L = spike_hist.shape[0]
+    if table.max_delay() >= L:
+        raise ValueError("spike history of {} steps is shorter than the largest delay".format(L))
+    ws = getattr(table, "_pull_ws", None)
+    need = lib.bmtk_csr_propagate_pull_workspace_bytes(L, n_src)
+    if ws is None or ws.numel() * 4 < need:
+        ws = table._pull_ws = torch.zeros(need // 4 + 1, dtype=torch.int32, device=syn.device)
+    _lib.check(lib.bmtk_csr_propagate_pull(_p(spike_hist, torch.int64), spike_hist.shape[1], L, n_src, batch,
+                                           _p(table.indptr), _p(table.packed()), _p(syn, torch.float32), n_tgt,
+                                           int(t_arrive), _p(ws), _stream()))
 
 
 def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_active=None, zbits=None, n_src=None):

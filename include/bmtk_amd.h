@@ -105,14 +105,36 @@ int bmtk_csr_propagate_gather(const uint64_t *zbits, int64_t n_src, int32_t batc
                               const uint8_t *delays, const uint8_t *receptors,
                               float *ring, int32_t L, int64_t n_tgt, int64_t step, void *stream);
 
-/* Packed synapse format used by the fused simulation: one 8-byte record per
- * synapse, {uint32 tdr, float weight} with tdr = index | receptor << 24 |
- * delay << 26 (index < 2^24, delay < 64 steps).  bmtk_csr_pack converts the
- * four plain arrays of a table; packed must hold nnz records. */
+/* One packed synapse: tdr = index | receptor << 24 | delay << 26 (index < 2^24, delay < 64 steps). */
 typedef struct bmtk_synapse {
     uint32_t tdr;
     float weight;
 } bmtk_synapse;
+
+/* Pull form of the same sums, for batched runs: instead of pushing weights
+ * into future ring slots, keep the spike bits of the last L steps
+ * (spike_hist[L][hist_stride] uint64 words, row (k mod L) = spike bits of step
+ * k) and compute everything that ARRIVES in step t_arrive in one pass over a
+ * packed TARGET-MAJOR table:
+ *   syn[r][i*batch+b] = sum over synapses (j -> i, w, d, r) of w * bit(spike_hist[(t_arrive-d) mod L], j*batch+b)
+ * syn ([4][n_tgt*batch]) is overwritten and is exactly the `syn` argument of
+ * bmtk_glif3_step_fwd for step t_arrive.  One wavefront per target row, lane =
+ * synapse, each lane adds its weight once per trial bit into LDS accumulators
+ * (LDS atomics: the order of additions is not fixed).  A per-source "fired in
+ * any trial" bit map of the L steps (built into `workspace`,
+ * bmtk_csr_propagate_pull_workspace_bytes bytes, and staged in LDS) filters the
+ * synapses whose source was silent, so the cost is one read of the table per
+ * step plus one mask fetch per synapse with an active source.  L must exceed
+ * the largest delay. */
+int64_t bmtk_csr_propagate_pull_workspace_bytes(int32_t L, int64_t n_src);
+int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src, int32_t batch,
+                            const int32_t *indptr, const bmtk_synapse *packed, float *syn, int64_t n_tgt,
+                            int64_t t_arrive, void *workspace, void *stream);
+
+/* Packed synapse format used by the fused simulation: one 8-byte record per
+ * synapse, {uint32 tdr, float weight} with tdr = index | receptor << 24 |
+ * delay << 26 (index < 2^24, delay < 64 steps).  bmtk_csr_pack converts the
+ * four plain arrays of a table; packed must hold nnz records. */
 int bmtk_csr_pack(int64_t nnz, const int32_t *indices, const float *weights, const uint8_t *delays,
                   const uint8_t *receptors, bmtk_synapse *packed, void *stream);
 

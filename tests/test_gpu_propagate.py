@@ -139,3 +139,36 @@ def test_propagate_argument_errors():
         ops.csr_propagate_gather(zb, n, t, torch.zeros(4, 4, n + 1, device="cuda"), n, 1, 0)
     with pytest.raises(ValueError):
         net.check_csr(csr, n, n, 1)         # delay 1 needs at least 2 slots
+
+
+@pytest.mark.parametrize("batch,p", [(1, 0.3), (5, 0.2), (32, 0.05), (64, 0.01), (64, 0.3), (100, 0.1), (130, 0.05)])
+def test_pull_matches_oracle(batch, p):
+    """Pull form: what arrives in step tau computed from the spike bits of the
+    last L steps.  LDS atomics add in arbitrary order, so the comparison is with
+    the fp64 oracle at 1e-5 of max(|want|, 1e-2 * sum of |w| into the cell)."""
+    rng = np.random.default_rng(40 + batch)
+    n_src, n_tgt, L = 211, 190, 6
+    src, tgt, w, d, r = _edges(rng, n_src, n_tgt, 15000)
+    by_src = net.coo_to_csr(src, tgt, w, d, r, n_rows=n_src, major="source")
+    by_tgt = net.coo_to_csr(src, tgt, w, d, r, n_rows=n_tgt, major="target")
+    table = ops.SynapseTable.from_numpy(by_tgt)
+    words = ops.n_words(n_src * batch)
+    hist = torch.zeros(L, words + 1, dtype=torch.int64, device="cuda")
+    abs_src = (by_src[0], by_src[1], np.abs(by_src[2]), by_src[3], by_src[4])
+    z_of = {}
+    syn = torch.full((4, n_tgt * batch), 7.0, device="cuda")      # must be overwritten, not accumulated
+    for tau in range(1, 14):
+        k = tau - 1                                                  # the newest emitting step
+        z_of[k] = (rng.random(n_src * batch) < p).astype(np.uint8)
+        hist[k % L] = to_dev(bits_of(z_of[k]))
+        ring = np.zeros((L, 4, n_tgt * batch))
+        mag = np.zeros((L, 4, n_tgt * batch))
+        for kk in range(max(0, tau - (L - 1)), tau):
+            orc.deliver_events(np.flatnonzero(z_of[kk]), batch, by_src, ring, n_tgt, kk)
+            orc.deliver_events(np.flatnonzero(z_of[kk]), batch, abs_src, mag, n_tgt, kk)
+        ops.csr_propagate_pull(hist, n_src, table, syn, n_tgt, batch, tau)
+        got = syn.cpu().numpy()
+        want, m = ring[tau % L], mag[tau % L]
+        assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-2 * m + 1e-30)) < 1e-5
+        assert np.all(got[m == 0] == 0)
+    assert np.abs(want).max() > 0
