@@ -89,18 +89,14 @@ constexpr unsigned kInputTag = 0x80000000u;
 // fired into one LDS list, then one thread per listed row pulls this
 // workgroup's segment of it.  Must be called by all threads of the workgroup.
 __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int64_t tp,
-                                          float *ring_l, unsigned *act, unsigned *scan_l, int e0, int64_t words)
+                                          float *ring_l, unsigned *act, unsigned *scan_l, int e0, int64_t words,
+                                          int64_t k0, int64_t k1)
 {
     const int tid = threadIdx.x;
     const int L = s.ring_slots;
     const int slot0 = (int)(tp % L);
     const int wave = tid / kWave;
-    const bool has_rec = s.rec_seg != nullptr, has_in = s.in_ptr != nullptr;
-    int64_t k0 = 0, k1 = 0;
-    if (has_in) {
-        k0 = s.in_ptr[tp];
-        k1 = s.in_ptr[tp + 1];
-    }
+    const bool has_rec = s.rec_seg != nullptr;
     const unsigned long long *bits =
         reinterpret_cast<const unsigned long long *>(s.work_bits) + (tp % 3) * (words + 1);
     const int64_t n_words = has_rec ? words : 0;
@@ -220,9 +216,12 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
     bool aborted = false;
     int64_t done = 0;  // steps whose update has run
+    // input events of step t-1 are in_events[ka, kb); the bound for the next step is fetched a step ahead
+    int64_t ka = 0, kb = s.in_ptr ? s.in_ptr[r.step0] : 0;
     for (int64_t k = 0; k < r.n_steps; ++k) {
         const int64_t t = r.step0 + k;
         PROF_T(c0);
+        const int64_t kn = s.in_ptr ? s.in_ptr[t + 1] : 0;
         // 1. fold the arrivals of slot t-1 and update
         bool spike = false;
         float frac = 0.0f;
@@ -269,7 +268,9 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         if (tid == 0) __hip_atomic_fetch_add(barrier, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         PROF_T(c2);
         // 3. pull the spikes and input events of step t-1 while the barrier fills
-        if (k > 0 && mine > 0) pull_step(s, r, g, t - 1, ring_l, act, scan_l, e0, words);
+        if (k > 0 && mine > 0) pull_step(s, r, g, t - 1, ring_l, act, scan_l, e0, words, ka, kb);
+        ka = kb;
+        kb = kn;
         __syncthreads();
         PROF_T(c3);
         // 4. wait for every workgroup's ballots of step t
@@ -309,7 +310,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     if (!aborted && done > 0) {
         // closing: spikes and inputs of the last step, then fold the last slot
         const int64_t tl = r.step0 + done - 1;
-        if (mine > 0) pull_step(s, r, g, tl, ring_l, act, scan_l, e0, words);
+        if (mine > 0) pull_step(s, r, g, tl, ring_l, act, scan_l, e0, words, ka, kb);
         __syncthreads();
         if (own) {
             float *prev = ring_l + (int)(tl % L) * GLIF3_NREC * span + tid;
