@@ -18,9 +18,13 @@ __device__ __forceinline__ float surrogate(float U, float th, float dampening)
 }
 
 // gz[j*B+b] = sum over out-going synapses (j -> i, w, d, r) of w * lam_ring[(t+d)%L][r][i*B+b]:
-// one wavefront per source neuron and 64-trial tile, lane = trial.  Rows whose
-// every trial has a zero surrogate derivative in this step are skipped.
-__global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, BwdStep q)
+// one wavefront per source neuron and trial tile.  A tile is `bp` trials wide
+// (the batch rounded up to a power of two, at most 64) and the wavefront's 64
+// lanes hold 64/bp synapses side by side, each lane reading one trial of one
+// synapse's adjoint row (bp*4 contiguous bytes per synapse); four such groups
+// are in flight before their products are added.  Rows whose every trial has
+// a zero surrogate derivative in this step are skipped.
+__global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, BwdStep q, int bp)
 {
     const int batch = a.batch;
     const int64_t ne = a.n_neurons * (int64_t)batch;
@@ -28,9 +32,11 @@ __global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, Bw
     const int lane = lane_id();
     const int64_t j = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
     if (j >= a.n_neurons) return;
+    const int per = kWave / bp;  // synapses per wavefront instruction
+    const int sub = lane / bp, b = lane - sub * bp;
     const int tile0 = blockIdx.y * kWave;
-    const bool lane_on = tile0 + lane < batch;
-    const int64_t e = j * batch + tile0 + lane;
+    const bool lane_on = tile0 + b < batch;
+    const int64_t e = j * batch + tile0 + b;
     bool active = false;
     if (lane_on) {
         const uint8_t f = a.save_flags[q.row * ne + e];
@@ -41,30 +47,39 @@ __global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, Bw
         }
     }
     if (__ballot(active) == 0ull) {
-        if (lane_on) a.gz[e] = 0.0f;
+        if (lane_on && sub == 0) a.gz[e] = 0.0f;
         return;
     }
     const int slot0 = (int)(q.t % L);
     const int p0 = a.rec_indptr[j], p1 = a.rec_indptr[j + 1];
     const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.rec_packed);
-    const float *__restrict__ ring = a.lam_ring + tile0 + lane;
+    const float *__restrict__ ring = a.lam_ring + tile0 + b;
+    constexpr int kInFlight = 4;
     float acc = 0.0f;
     for (int base = p0; base < p1; base += kWave) {
         const int p = base + lane;
         uint2 sy = make_uint2(0u, 0u);
         if (p < p1) sy = rows[p];
         const int n_here = min(kWave, p1 - base);
-        for (int l = 0; l < n_here; ++l) {
-            const unsigned tdr = (unsigned)bcast_i((int)sy.x, l);
-            const float w = __uint_as_float((unsigned)bcast_i((int)sy.y, l));
-            int slot = slot0 + (int)(tdr >> 26);
-            slot = slot >= L ? slot - L : slot;
-            const int r = (tdr >> 24) & 3;
-            const int64_t i = tdr & 0xFFFFFFu;
-            if (active) acc += w * ring[(int64_t)(slot * GLIF3_NREC + r) * ne + i * batch];
+        for (int l0 = 0; l0 < n_here; l0 += per * kInFlight) {
+            float w[kInFlight], v[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                const int idx = l0 + u * per + sub;
+                const unsigned tdr = (unsigned)__shfl((int)sy.x, idx & (kWave - 1), kWave);
+                w[u] = __uint_as_float((unsigned)__shfl((int)sy.y, idx & (kWave - 1), kWave));
+                int slot = slot0 + (int)(tdr >> 26);
+                slot = slot >= L ? slot - L : slot;
+                const int r = (tdr >> 24) & 3;
+                const int64_t i = tdr & 0xFFFFFFu;
+                v[u] = (active && idx < n_here) ? ring[(int64_t)(slot * GLIF3_NREC + r) * ne + i * batch] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) acc += w[u] * v[u];
         }
     }
-    if (lane_on) a.gz[e] = acc;
+    for (int off = bp; off < kWave; off <<= 1) acc += __shfl_xor(acc, off, kWave);
+    if (lane_on && sub == 0) a.gz[e] = acc;
 }
 
 // state adjoint of one step, one thread per element; writes the adjoint of
@@ -255,10 +270,12 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
     const unsigned rows_grid = (unsigned)((a.n_neurons + kBlock / kWave - 1) / (kBlock / kWave));
     const unsigned tiles = (unsigned)((a.batch + kWave - 1) / kWave);
     const unsigned elem_grid = (unsigned)((ne + kBlock - 1) / kBlock);
+    int bp = 1;  // trial-tile width: the batch rounded up to a power of two, at most one wavefront
+    while (bp < a.batch && bp < kWave) bp <<= 1;
     for (int64_t k = n_steps - 1; k >= 0; --k) {
         BwdStep q{step0 + k, k};
         if (has_rec)
-            hipLaunchKernelGGL(bwd_gather_kernel, dim3(rows_grid, tiles), dim3(kBlock), 0, st, a, q);
+            hipLaunchKernelGGL(bwd_gather_kernel, dim3(rows_grid, tiles), dim3(kBlock), 0, st, a, q, bp);
         else
             hipLaunchKernelGGL(fill_zero_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a.gz, ne);
         hipLaunchKernelGGL(bwd_state_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q);
