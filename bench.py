@@ -30,9 +30,12 @@ B_PER_EVENT = 18               # 4 index + 4 weight + 1 delay + 1 receptor + 8 r
 
 N_V1, N_IN, MEAN_IN, N_IN_SYN, N_CLASSES = 230924, 17400, 300, 8_000_000, 111
 IN_RATE_HZ, IN_W_SCALE = 5.0, 7.0
-# HBM bytes per simulated step of the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (filled in from the counter runs summarised under profiles/; None = not measured)
-TRAFFIC_BYTES_PER_STEP = None
+# HBM bytes per simulated step of the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE counter
+# runs (summaries under profiles/; one FETCH_SIZE count = 2 KiB, one WRITE_SIZE count = 1 KiB by the
+# 1 GiB copy calibration).  Measured at the default operating point; not re-measured by this script.
+TRAFFIC_BYTES_PER_STEP = {"resident": 4.07e6 + 0.20e6, "per_step": 18.8e6 + 22.0e6}
+TRAFFIC_STATE_UPDATE_1M = 176.2e6 + 51.4e6   # glif3_step_kernel, per launch
+TRAFFIC_PULL_52K_B64 = 455e6 + 53.2e6        # pull_kernel, per launch, pooled over the three rates
 
 
 def build_v1(torch, steps_total, resident="auto"):
@@ -94,7 +97,7 @@ def bench_state_update(torch, steps=1000, warmup=50):
     return {"kernel": "glif3_step_kernel", "workload": "state update N=1048576, per-neuron parameters, 1000 steps",
             "neuron_updates_per_s": n / per, "us_per_launch": per * 1e6,
             "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+                         "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": TRAFFIC_STATE_UPDATE_1M},
             "bytes_per_update": B_PER_UPDATE_PLAIN + 29 * 4}
 
 
@@ -147,7 +150,8 @@ def bench_propagation(torch, steps=200, warmup=20):
                         (t_src.nnz, rate), "events_per_launch": events, "synaptic_events_per_s": events / per,
                         "us_per_launch": per * 1e6,
                         "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS,
-                                     "unit": "GB/s", "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None}})
+                                     "unit": "GB/s", "frac": alg / per / 1e9 / HBM_PEAK_GBS,
+                                     "traffic": TRAFFIC_PULL_52K_B64 if mode == "pull" else None}})
     return out
 
 
@@ -296,8 +300,8 @@ def main():
                    "recurrent_events": rec_ev, "input_events": in_ev, "input_weight_scale": IN_W_SCALE},
         "roofline": {"bound": "hbm", "kernel": "sim_resident_kernel" if resident else "sim_step_kernel",
                      "achieved": alg / per_launch / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": alg / per_launch / 1e9 / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES_PER_STEP * K / launches
-                     if TRAFFIC_BYTES_PER_STEP else None,
+                     "frac": alg / per_launch / 1e9 / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC_BYTES_PER_STEP["resident" if resident else "per_step"] * K / launches,
                      "launches": launches, "algorithmic_bytes_per_launch": alg, "us_per_launch": per_launch * 1e6,
                      "algorithmic_bytes_per_step": alg_step, "us_per_step": dev / K * 1e6},
     }
