@@ -194,7 +194,9 @@ __global__ __launch_bounds__(kBlock) void bwd_rec_grad_kernel(bmtk_glif3_bwd a, 
     }
 }
 
-// input weights: one wavefront per input event, atomics (several trials of one source may fire together)
+// Input weights.  The events of a step are ascending in source*batch+trial, so the trials in
+// which one source fired are adjacent: the wavefront that holds the first event of such a run
+// takes the whole run, which makes it the only writer of that source's row -- no atomics.
 __global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, BwdStep q)
 {
     const int batch = a.batch;
@@ -207,7 +209,11 @@ __global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, 
     for (int64_t k = k0 + blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; k < k1; k += n_waves) {
         const int ev = a.in_events[k];
         const int j = batch == 1 ? ev : (int)((uint32_t)ev / (uint32_t)batch);
-        const int b = ev - j * batch;
+        if (k > k0 && (batch == 1 ? a.in_events[k - 1] : (int)((uint32_t)a.in_events[k - 1] / (uint32_t)batch)) == j)
+            continue;  // not the first event of its source's run
+        int64_t k_end = k + 1;
+        while (k_end < k1 && (batch == 1 ? a.in_events[k_end] : (int)((uint32_t)a.in_events[k_end] / (uint32_t)batch)) == j)
+            ++k_end;
         const int p0 = a.inp_indptr[j], p1 = a.inp_indptr[j + 1];
         for (int p = p0 + lane_id(); p < p1; p += kWave) {
             const uint2 sy = rows[p];
@@ -215,7 +221,10 @@ __global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, 
             slot = slot >= L ? slot - L : slot;
             const int r = (sy.x >> 24) & 3;
             const int64_t i = sy.x & 0xFFFFFFu;
-            atomicAdd(a.d_inp_w + p, a.lam_ring[(int64_t)(slot * GLIF3_NREC + r) * ne + i * batch + b]);
+            const float *cell = a.lam_ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch;
+            float acc = 0.0f;
+            for (int64_t kk = k; kk < k_end; ++kk) acc += cell[a.in_events[kk] - j * batch];
+            a.d_inp_w[p] += acc;
         }
     }
 }
@@ -280,7 +289,7 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
             hipLaunchKernelGGL(fill_zero_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a.gz, ne);
         hipLaunchKernelGGL(bwd_state_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q);
         if (a.d_rec_w) hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
-        if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(64), dim3(kBlock), 0, st, a, q);
+        if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(256), dim3(kBlock), 0, st, a, q);
     }
     BMTK_CHECK_LAUNCH("glif3_simulate_bwd");
     return BMTK_OK;
