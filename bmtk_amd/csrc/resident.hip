@@ -54,14 +54,20 @@ __device__ __forceinline__ unsigned load_agent(const unsigned *p)
 
 // add the weights of one row's synapses that target this workgroup's group,
 // positions [seg_row[g], seg_row[g+1]) of the packed table, to the LDS ring
-// slice.  The first four synapses are fetched together (a segment holds one or
-// two on average), the rest one by one.
+// slice.  Every lane of a wavefront reads a different cache line here, and the
+// address unit serialises such requests, so the number of requests is what
+// costs: the two bounds come in one 8-byte load, and only lanes that really
+// have a k-th synapse issue the k-th load (a segment holds 1.2 on average).
+struct __attribute__((packed, aligned(4))) SegBounds {
+    uint32_t lo, hi;
+};
+
 __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_row, int g,
                                              const bmtk_synapse *__restrict__ tab, float *ring_l, int span, int e0,
                                              int L, int slot0)
 {
-    const uint32_t lo = seg_row[g], hi = seg_row[g + 1];
-    if (hi <= lo) return;
+    const SegBounds sb = *reinterpret_cast<const SegBounds *>(seg_row + g);
+    const uint32_t lo = sb.lo, hi = sb.hi;
     const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(tab);
     auto add = [&](const uint2 sy) {
         int slot = slot0 + (int)(sy.x >> 26);
@@ -70,13 +76,14 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
         const int i = (int)(sy.x & 0xFFFFFFu) - e0;
         atomicAdd(ring_l + (slot * GLIF3_NREC + r) * span + i, __uint_as_float(sy.y));
     };
-    uint2 first[4];
+    uint2 first[3];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) first[u] = rows[min(lo + (uint32_t)u, hi - 1u)];
+    for (int u = 0; u < 3; ++u)
+        if (lo + (uint32_t)u < hi) first[u] = rows[lo + (uint32_t)u];
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < 3; ++u)
         if (lo + (uint32_t)u < hi) add(first[u]);
-    for (uint32_t p = lo + 4u; p < hi; ++p) add(rows[p]);
+    for (uint32_t p = lo + 3u; p < hi; ++p) add(rows[p]);
 }
 
 constexpr int kActCap = 8192;   // active-row list in LDS (entries)
