@@ -1,0 +1,182 @@
+"""Run a SONATA/bmtk PointNet configuration on the GPU.
+
+The three calls of a bmtk run script (examples/point_450glifs/run_pointnet.py),
+
+    configure = pointnet.Config.from_json(config_file)
+    graph = pointnet.PointNetwork.from_config(configure)
+    sim = pointnet.PointSimulator.from_config(configure, graph)
+    sim.run()
+
+with the same meaning for GLIF point networks: build the network from the
+``networks`` section (bmtk/simulator/pointnet/pointnetwork.py:144-232), attach
+the ``inputs`` of type ``spikes`` (modules ``sonata``/``h5`` and ``csv``,
+bmtk/simulator/pointnet/pointsimulator.py:229-262; spike-time rules of
+pointnetwork.py:39-61) and ``current_clamp``, run ``tstop/dt`` steps
+(pointsimulator.py:149-173) and write ``output.spikes_file`` /
+``spikes_file_csv`` in ``output.output_dir`` sorted as ``spikes_sort_order``
+asks (bmtk/simulator/pointnet/modules/record_spikes.py:53-104).
+"""
+import os
+
+import numpy as np
+import pandas as pd
+import torch
+
+from . import sonata
+from .simulator import Glif3Simulator
+from .spike_trains import bin_spike_times
+
+
+class Config(dict):
+    @classmethod
+    def from_json(cls, path):
+        return cls(sonata.load_config(path))
+
+    from_dict = classmethod(lambda cls, d: cls(d))
+
+    def build_env(self):
+        out = self.get("output", {}).get("output_dir")
+        if out:
+            os.makedirs(out, exist_ok=True)
+
+    @property
+    def dt(self):
+        return float(self.get("run", {}).get("dt", 0.001))  # NEST's default resolution is what bmtk falls back to
+
+    @property
+    def tstop(self):
+        return float(self["run"]["tstop"])
+
+
+class PointNetwork(sonata.PointNetwork):
+    @classmethod
+    def from_config(cls, config, dt=None, unsupported="raise"):
+        nw = sonata.load_point_network(config, dt=dt if dt is not None else Config(config).dt,
+                                       unsupported=unsupported)
+        nw.__class__ = cls
+        return nw
+
+
+def _read_input_spikes(entry):
+    module = entry.get("module", "sonata")
+    if module in ("sonata", "h5", "hdf5"):
+        return sonata.read_spikes(entry["input_file"])
+    if module == "csv":
+        return sonata.read_spikes_csv(entry["input_file"])
+    raise NotImplementedError("spikes input module {!r} is not supported".format(module))
+
+
+class PointSimulator:
+    def __init__(self, network, dt, tstop, device=None, resident="auto"):
+        self.net, self.dt, self.tstop = network, float(dt), float(tstop)
+        self.n_steps = int(round(self.tstop / self.dt))
+        self.output = {}
+        self._trains = [None] * network.n_inputs
+        self._i_ext = np.zeros(network.n, np.float64)
+        self._clamps = []
+        self._device, self._resident = device, resident
+        self.spikes = None
+
+    @classmethod
+    def from_config(cls, config, network, dt=None, device=None, resident="auto"):
+        config = Config(config)
+        sim = cls(network, dt if dt is not None else config.dt, config.tstop, device=device, resident=resident)
+        sim.output = dict(config.get("output", {}))
+        for name, entry in config.get("inputs", {}).items():
+            kind = entry.get("input_type")
+            if kind == "spikes":
+                sim.add_spike_inputs(_read_input_spikes(entry), entry.get("node_set"))
+            elif kind == "current_clamp":
+                sim.add_current_clamp(entry)
+            else:
+                raise NotImplementedError("input {!r}: input_type {!r} is not supported".format(name, kind))
+        return sim
+
+    def add_spike_inputs(self, spikes, node_set=None):
+        """Spike trains of virtual populations; a train is only used by the population it is stored under, and
+        ``node_set`` (a population name, or {"population": name}) restricts which populations are taken."""
+        if isinstance(node_set, dict):
+            node_set = node_set.get("population")
+        for pop, entry in spikes.items():
+            if pop not in self.net.virtual or (isinstance(node_set, str) and node_set not in (pop, "all")):
+                continue
+            base = self.net.virtual[pop]
+            ids, ts = np.asarray(entry[0]), np.asarray(entry[1], np.float64)
+            order = np.lexsort((ts, ids))
+            ids, ts = ids[order], ts[order]
+            uniq, start = np.unique(ids, return_index=True)
+            for u, a, b in zip(uniq, start, list(start[1:]) + [ids.size]):
+                row = base + int(u)
+                if row < len(self._trains):
+                    self._trains[row] = ts[a:b]
+
+    def add_current_clamp(self, entry):
+        """A step current on a list of node ids: ``amp`` pA from ``delay`` for ``duration`` ms
+        (bmtk/simulator/pointnet/modules/iclamp.py:8-54, NEST step_current_generator semantics: an amplitude set
+        for time t acts on the update that starts at t + dt)."""
+        ids = entry.get("node_set", {})
+        ids = ids.get("node_id", ids.get("node_ids")) if isinstance(ids, dict) else ids
+        if ids is None or isinstance(ids, str):
+            raise NotImplementedError("current_clamp needs an explicit node id list")
+        amps = np.atleast_1d(np.asarray(entry["amp"], np.float64))
+        delays = np.atleast_1d(np.asarray(entry["delay"], np.float64))
+        durs = np.atleast_1d(np.asarray(entry["duration"], np.float64))
+        for a, t0, dur in zip(amps, delays, durs):
+            self._clamps.append((np.asarray(ids, np.int64), float(a), float(t0), float(t0 + dur)))
+
+    def _segments(self):
+        """Step ranges with a constant external current, and that current."""
+        marks = {0, self.n_steps}
+        for _, _, t0, t1 in self._clamps:
+            for t in (t0, t1):
+                marks.add(min(self.n_steps, max(0, int(round(t / self.dt)) + 1)))
+        marks = sorted(marks)
+        for a, b in zip(marks[:-1], marks[1:]):
+            cur = np.zeros(self.net.n, np.float32)
+            for ids, amp, t0, t1 in self._clamps:
+                if int(round(t0 / self.dt)) + 1 <= a < int(round(t1 / self.dt)) + 1:
+                    cur[ids] += amp
+            yield a, b, cur
+
+    def run(self, record_cap=None):
+        nw = self.net
+        rec, inp = nw.tables()
+        sim = Glif3Simulator(nw.n, nw.par, self.dt, class_id=nw.class_id, rec=rec, inp=inp,
+                             asc_init=nw.asc_init[:, nw.class_id], u_init=nw.u_init[nw.class_id],
+                             i_ext=np.zeros(nw.n, np.float32), device=self._device, resident=self._resident)
+        if inp is not None:
+            sim.set_input_events(*bin_spike_times(self._trains, self.dt, self.n_steps))
+        steps, elems, fracs = [], [], []
+        for a, b, cur in self._segments():
+            sim.i_ext.copy_(torch.as_tensor(cur, device=sim.dev))
+            cap = record_cap or max(1 << 16, (b - a) * nw.n // 8)
+            out = sim.run(b - a, spike_bits=False, record_cap=cap)
+            sim.check()
+            r = out["record"]
+            c = int(r["count"].item())
+            if c > cap:
+                raise RuntimeError("spike record overflow: {} spikes, room for {}".format(c, cap))
+            steps.append(r["step"][:c].cpu().numpy().astype(np.int64))
+            elems.append(r["elem"][:c].cpu().numpy().astype(np.int64))
+            fracs.append(r["frac"][:c].cpu().numpy().astype(np.float64))
+        self.simulator = sim
+        st, el, fr = (np.concatenate(x) for x in (steps, elems, fracs))
+        times = (st + fr) * self.dt  # threshold crossing interpolated inside the step, as glif_psc stamps it
+        order = np.lexsort((el, times))
+        self.spikes = {nw.population: (el[order], times[order])}
+        self._write_outputs()
+        return self.spikes
+
+    def _write_outputs(self):
+        out = self.output
+        if not out:
+            return
+        base = out.get("output_dir", ".")
+        order = out.get("spikes_sort_order", "none")
+        if out.get("spikes_file"):
+            path = out["spikes_file"] if os.path.isabs(out["spikes_file"]) else os.path.join(base, out["spikes_file"])
+            sonata.write_spikes(path, self.spikes, sort_order=order)
+        if out.get("spikes_file_csv"):
+            path = out["spikes_file_csv"]
+            path = path if os.path.isabs(path) else os.path.join(base, path)
+            sonata.write_spikes_csv(path, self.spikes, sort_order=order)

@@ -1,0 +1,273 @@
+"""SONATA files: the HDF5 subset reader/writer, the node/edge loaders and the spike files (CPU only).
+
+The network files under tests/golden/point_450glifs are the data files of the reference's
+examples/point_450glifs (written by h5py).  What pins the reader: facts the example's own tables state
+(populations, node counts per type, the edge-type of every edge), the two redundant indices each edge file
+carries (a wrong offset or a transposed column breaks them), and, where the HDF5 command line tools exist on
+the machine, the HDF5 library's own reading of the same files.  The writer is pinned by that library too
+(h5dump / h5repack read what it wrote) and by the reader.
+"""
+import json
+import os
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+from bmtk_amd import h5lite, network as net, sonata
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+NETDIR = os.path.join(G, "point_450glifs", "network")
+
+
+def _tool(name):
+    for d in (os.environ.get("HDF5_TOOLS_DIR", ""), "/opt/conda/bin"):
+        p = os.path.join(d, name)
+        if d and os.path.exists(p):
+            return p
+    return shutil.which(name)
+
+
+needs_h5dump = pytest.mark.skipif(_tool("h5dump") is None, reason="HDF5 command line tools not installed")
+
+
+def _circuit(dt=0.1):
+    return {"run": {"dt": dt, "tstop": 3000.0},
+            "components": {"point_neuron_models_dir": os.path.join(G, "cell_models"),
+                           "synaptic_models_dir": os.path.join(G, "synaptic_models")},
+            "networks": {"nodes": [{"nodes_file": os.path.join(NETDIR, "v1_nodes.h5"),
+                                    "node_types_file": os.path.join(NETDIR, "v1_node_types.csv")},
+                                   {"nodes_file": os.path.join(NETDIR, "lgn_nodes.h5"),
+                                    "node_types_file": os.path.join(NETDIR, "lgn_node_types.csv")}],
+                         "edges": [{"edges_file": os.path.join(NETDIR, "v1_v1_edges.h5"),
+                                    "edge_types_file": os.path.join(NETDIR, "v1_v1_edge_types.csv")},
+                                   {"edges_file": os.path.join(NETDIR, "lgn_v1_edges.h5"),
+                                    "edge_types_file": os.path.join(NETDIR, "lgn_v1_edge_types.csv")}]}}
+
+
+def _h5dump_values(path, dataset, dtype):
+    out = subprocess.run([_tool("h5dump"), "-d", dataset, "-y", "-w", "65535", path], capture_output=True, text=True,
+                         check=True).stdout
+    start = out.index("DATA {") + 6
+    body = out[start:out.index("}", start)]
+    return np.array([t for t in body.replace("\n", " ").replace(",", " ").split() if t], dtype=dtype)
+
+
+def test_reader_example_structure():
+    with h5lite.File(os.path.join(NETDIR, "v1_v1_edges.h5")) as f:
+        assert int(f.attrs["magic"]) == 0x0A7A and list(f.attrs["version"]) == [0, 1]
+        g = f["/edges/v1_to_v1"]
+        assert g.keys() == ["0", "edge_group_id", "edge_group_index", "edge_type_id", "indices", "source_node_id",
+                            "target_node_id"]
+        assert g["source_node_id"].attrs["node_population"] == "v1"
+        assert g["source_node_id"].dtype == np.dtype("<u8") and g["source_node_id"].shape == (28555,)
+        assert g["0/nsyns"].dtype == np.dtype("<u4")
+        assert "indices/target_to_source/node_id_to_range" in g and "nope" not in g
+        with pytest.raises(KeyError):
+            g["missing"]
+        # edges are written target-major (the builder sorts by target)
+        assert np.all(np.diff(g["target_node_id"][()].astype(np.int64)) >= 0)
+    with h5lite.File(os.path.join(NETDIR, "v1_nodes.h5")) as f:
+        ntid = f["/nodes/v1/node_type_id"][()]
+        # 80,80,80 excitatory + 30,30 inhibitory GLIF cells, 2 x 75 integrate-and-fire cells (v1_node_types.csv order)
+        assert np.array_equal(np.bincount(ntid.astype(np.int64))[100:], [80, 80, 80, 30, 30, 75, 75])
+        assert f["/nodes/v1/0/x"].dtype == np.float64 and f["/nodes/v1/1/x"].shape == (150,)
+    with pytest.raises(h5lite.H5Error):
+        h5lite.File(os.path.join(NETDIR, "v1_node_types.csv"))
+
+
+@needs_h5dump
+@pytest.mark.parametrize("fname,dataset,dtype", [
+    ("v1_v1_edges.h5", "/edges/v1_to_v1/source_node_id", np.uint64),
+    ("v1_v1_edges.h5", "/edges/v1_to_v1/0/nsyns", np.uint32),
+    ("v1_v1_edges.h5", "/edges/v1_to_v1/indices/source_to_target/range_to_edge_id", np.uint64),
+    ("lgn_v1_edges.h5", "/edges/lgn_to_v1/target_node_id", np.uint64),
+    ("v1_nodes.h5", "/nodes/v1/0/rotation_angle_yaxis", np.float64),
+])
+def test_reader_agrees_with_hdf5_library(fname, dataset, dtype):
+    path = os.path.join(NETDIR, fname)
+    want = _h5dump_values(path, dataset, dtype)
+    got = h5lite.File(path)[dataset][()].reshape(-1)
+    if dtype == np.float64:
+        assert np.allclose(got, want, rtol=1e-5)  # h5dump prints 6 significant digits
+    else:
+        assert np.array_equal(got, want)
+
+
+def test_edge_indices_match_edge_lists():
+    cfg = _circuit()
+    for entry in cfg["networks"]["edges"]:
+        for ep in sonata.read_edges(entry["edges_file"], entry["edge_types_file"]).values():
+            assert set(ep.indices) == {"source_to_target", "target_to_source"}
+            ep.check_indices()
+            # and a broken index is noticed
+            lookup, ranges = ep.indices["target_to_source"]
+            bad = ranges.copy()
+            bad[3, 1] += 1
+            ep.indices["target_to_source"] = (lookup, bad)
+            with pytest.raises(ValueError):
+                ep.check_indices()
+
+
+def test_edge_rules_on_example():
+    """weight = nsyns * syn_weight of the edge's type, delay from the type table, receptor from the synaptic-model
+    file (bmtk/simulator/pointnet/sonata_adaptors.py:268-357), stated here straight from the csv and json files."""
+    entry = _circuit()["networks"]["edges"][0]
+    ep = sonata.read_edges(entry["edges_file"], entry["edge_types_file"])["v1_to_v1"]
+    assert ep.source_population == "v1" and ep.target_population == "v1"
+    src, tgt, w, d, r = ep.to_arrays(os.path.join(G, "synaptic_models"), dt=0.1)
+    with h5lite.File(entry["edges_file"]) as f:
+        nsyns = f["/edges/v1_to_v1/0/nsyns"][()].astype(np.float64)
+        etid = f["/edges/v1_to_v1/edge_type_id"][()]
+    table = {}
+    with open(entry["edge_types_file"]) as fh:
+        head = fh.readline().split()
+        for line in fh:
+            row = dict(zip(head, line.split()))
+            with open(os.path.join(G, "synaptic_models", row["dynamics_params"])) as jf:
+                port = json.load(jf).get("receptor_type", 0)
+            table[int(row["edge_type_id"])] = (float(row["syn_weight"]), float(row["delay"]), port)
+    assert np.array_equal(w, np.array([nsyns[i] * table[t][0] for i, t in enumerate(etid)], np.float32))
+    assert np.array_equal(d, np.array([round(table[t][1] / 0.1) for t in etid]))
+    assert np.array_equal(r, np.array([table[t][2] for t in etid]))
+    assert np.array_equal(src, ep.source_node_id) and np.array_equal(tgt, ep.target_node_id)
+    with pytest.raises(net.BadDelay):
+        ep.to_arrays(os.path.join(G, "synaptic_models"), dt=2.5)
+
+
+def test_load_point_network():
+    with pytest.raises(NotImplementedError, match="iaf_psc_alpha"):
+        sonata.load_point_network(_circuit())
+    nw = sonata.load_point_network(_circuit(), unsupported="silence")
+    assert nw.population == "v1" and nw.n == 450 and nw.n_inputs == 100 and nw.virtual == {"lgn": 0}
+    assert list(nw.supported) == [True] * 5 + [False] * 2
+    assert np.array_equal(np.bincount(nw.class_id), [80, 80, 80, 30, 30, 75, 75])
+    # the silenced cells neither receive nor send
+    silent = ~nw.supported[nw.class_id]
+    for e in (nw.rec_edges, nw.inp_edges):
+        assert not silent[e[1]].any()
+    assert not silent[nw.rec_edges[0]].any()
+    rec, inp = nw.tables()
+    net.check_csr(rec, 450, 450, 21)
+    net.check_csr(inp, 100, 450, 21)
+    # class parameters are the converted cell files: E_L of node type 100 (593618144) from its json
+    with open(os.path.join(G, "cell_models", "593618144_glif_lif_asc_psc.json")) as fh:
+        cell = json.load(fh)
+    from bmtk_amd.layout import PAR
+    assert nw.par[PAR["E_L"], 0] == cell["E_L"] and nw.par[PAR["C_M"], 0] == cell["C_m"]
+    # excitatory sources carry positive weights, inhibitory ones negative (v1_v1_edge_types.csv)
+    src_class = nw.class_id[nw.rec_edges[0]]
+    assert np.all(nw.rec_edges[2][src_class <= 2] > 0) and np.all(nw.rec_edges[2][src_class >= 3] < 0)
+
+
+def test_load_config_manifest(tmp_path):
+    (tmp_path / "sub").mkdir()
+    (tmp_path / "circuit.json").write_text(json.dumps({
+        "manifest": {"$BASE_DIR": ".", "$NETWORK_DIR": "$BASE_DIR/network", "$MODELS": "${BASE_DIR}/../models"},
+        "components": {"synaptic_models_dir": "$MODELS/syn"},
+        "networks": {"nodes": [{"nodes_file": "$NETWORK_DIR/n.h5"}]}}))
+    (tmp_path / "sim.json").write_text(json.dumps({
+        "manifest": {"$OUT": "$configdir/output"}, "run": {"dt": 0.1}, "output": {"output_dir": "$OUT"},
+        "network": "circuit.json"}))
+    cfg = sonata.load_config(str(tmp_path / "sim.json"))
+    assert cfg["networks"]["nodes"][0]["nodes_file"] == str(tmp_path / "network" / "n.h5")
+    assert os.path.normpath(cfg["components"]["synaptic_models_dir"]) == str(tmp_path.parent / "models" / "syn")
+    assert cfg["output"]["output_dir"] == str(tmp_path / "output") and cfg["run"]["dt"] == 0.1
+
+
+def test_input_spike_file():
+    sp = sonata.read_spikes(os.path.join(G, "point_450glifs", "inputs", "lgn_spikes.h5"))
+    ids, ts, attrs = sp["lgn"]
+    assert ids.size == 3044 and set(ids) <= set(range(100)) and attrs == {"sorting": "none", "units": "ms"}
+    assert ts.min() > 0 and ts.max() < 3000.0
+    # the file was written node by node: times ascend within a node
+    for node in (0, 57, 99):
+        assert np.all(np.diff(ts[ids == node]) > 0)
+
+
+def _random_spikes(seed=1, n=5000):
+    rng = np.random.default_rng(seed)
+    return rng.integers(0, 300, n), rng.random(n) * 3000.0
+
+
+@pytest.mark.parametrize("order", ["none", "by_time", "by_id", "unknown"])
+def test_spike_file_round_trip(tmp_path, order):
+    ids, ts = _random_spikes()
+    path = str(tmp_path / "out" / "spikes.h5")
+    sonata.write_spikes(path, {"v1": (ids, ts), "empty": (np.zeros(0, int), np.zeros(0))}, sort_order=order)
+    back = sonata.read_spikes(path)
+    assert set(back) == {"v1", "empty"} and back["empty"][0].size == 0
+    rid, rts, attrs = back["v1"]
+    assert attrs["units"] == "ms" and attrs["sorting"] == order
+    if order == "by_time":
+        assert np.all(np.diff(rts) >= 0)
+    elif order == "by_id":
+        assert np.all(np.diff(rid) >= 0) and all(np.all(np.diff(rts[rid == k]) >= 0) for k in (0, 1, 299))
+    else:
+        assert np.array_equal(rid, ids) and np.array_equal(rts, ts)
+    assert sonata.spikes_equal({"v1": (ids, ts)}, {"v1": (rid, rts)})
+    with pytest.raises(ValueError, match="already contains"):
+        sonata.write_spikes(path, {"v1": (ids, ts)}, mode="a")
+    sonata.write_spikes(path, {"lgn": (ids[:10], ts[:10])}, mode="a")
+    assert set(sonata.read_spikes(path)) == {"v1", "empty", "lgn"}
+    csv = str(tmp_path / "spikes.csv")
+    sonata.write_spikes_csv(csv, {"v1": (ids, ts)}, sort_order=order)
+    with open(csv) as fh:
+        assert fh.readline().strip() == "timestamps population node_ids"
+    assert sonata.spikes_equal(sonata.read_spikes_csv(csv), {"v1": (ids, ts)}, err=1e-9)
+
+
+@needs_h5dump
+def test_written_file_is_read_by_hdf5_library(tmp_path):
+    ids, ts = _random_spikes(2, 3000)
+    path = str(tmp_path / "spikes.h5")
+    sonata.write_spikes(path, {"v1": (ids, ts)}, sort_order="by_time")
+    text = subprocess.run([_tool("h5dump"), "-A", path], capture_output=True, text=True, check=True).stdout
+    for needle in ('ATTRIBUTE "magic"', '(0): 2682', 'ATTRIBUTE "sorting"', '"by_time"', 'ATTRIBUTE "units"', '"ms"',
+                   'DATASET "node_ids"', "H5T_STD_U64LE", 'DATASET "timestamps"', "H5T_IEEE_F64LE",
+                   "H5T_CSET_UTF8"):
+        assert needle in text, needle
+    order = np.lexsort((ids, ts))
+    assert np.array_equal(_h5dump_values(path, "/spikes/v1/node_ids", np.uint64), ids[order].astype(np.uint64))
+    # what bmtk itself writes is chunked and gzip-compressed (spikes_file_writers.py:66-68): let the HDF5 library
+    # re-pack our file that way and read it back
+    packed = str(tmp_path / "packed.h5")
+    subprocess.run([_tool("h5repack"), "-f", "SHUF", "-f", "GZIP=4", "-l", "CHUNK=1000", path, packed], check=True)
+    rid, rts, attrs = sonata.read_spikes(packed)["v1"]
+    assert np.array_equal(rid, ids[order]) and np.array_equal(rts, ts[order]) and attrs["sorting"] == "by_time"
+
+
+def test_h5lite_round_trip_types(tmp_path):
+    rng = np.random.default_rng(0)
+    tree = {"a": {"__attrs__": {"note": "täst", "k": np.int64(-3)},
+                  "i8": rng.integers(-100, 100, 17).astype(np.int8), "u16": np.arange(5, dtype=np.uint16),
+                  "f32": (rng.random((3, 4)).astype(np.float32), {"scale": 2.5}),
+                  "names": np.array(["ab", "cde", ""]), "deep": {"x": np.zeros(0, np.float64)}},
+            "flag": np.array([True, False])}
+    path = str(tmp_path / "t.h5")
+    h5lite.write(path, tree, attrs={"version": np.array([0, 1], np.uint32)})
+    with h5lite.File(path) as f:
+        assert f.keys() == ["a", "flag"] and f["a"].attrs == {"note": "täst", "k": -3}
+        assert np.array_equal(f["a/i8"][()], tree["a"]["i8"]) and f["a/i8"].dtype == np.int8
+        assert np.array_equal(f["a/f32"][()], tree["a"]["f32"][0]) and f["a/f32"].attrs["scale"] == 2.5
+        assert list(f["a/names"][()]) == [b"ab", b"cde", b""] and f["/a/deep/x"].shape == (0,)
+        assert np.array_equal(f["a/u16"][1:3], [1, 2])
+    with pytest.raises(h5lite.H5Error):
+        h5lite.write(path, {str(i): np.zeros(1) for i in range(100)})  # more members than one group node holds
+
+
+def test_spike_comparisons():
+    a = {"v1": (np.array([0, 0, 1, 2]), np.array([1.0, 5.0, 2.0, 3.0]))}
+    same = {"v1": (np.array([2, 1, 0, 0]), np.array([3.0, 2.0, 5.0, 1.001]))}
+    # numpy's allclose adds its default relative tolerance of 1e-5 to `err`, in the reference as here
+    assert sonata.spikes_equal(a, same, err=1e-2) and not sonata.spikes_equal(a, same)
+    fewer = {"v1": (np.array([0, 2]), np.array([5.0, 3.0]))}
+    assert not sonata.spikes_equal(a, fewer)
+    assert sonata.spikes_is_subset(fewer, a) and not sonata.spikes_is_subset(a, fewer)
+    assert sonata.spikes_is_subset(a, same, err=1e-2) and not sonata.spikes_is_subset(a, same, err=1e-2, strict=True)
+    moved = {"v1": (np.array([0, 2]), np.array([5.0, 3.5]))}
+    assert not sonata.spikes_is_subset(moved, a)
+    other_pop = {"lgn": a["v1"]}
+    assert not sonata.spikes_equal(a, other_pop) and not sonata.spikes_is_subset(a, other_pop)
+    assert sonata.spikes_is_subset({"v1": (np.zeros(0, int), np.zeros(0))}, a)
