@@ -91,7 +91,7 @@ def test_preconverted_example_cells_have_the_target_keys(golden_dir):
     keys = {"V_m", "V_th", "g", "E_L", "C_m", "t_ref", "V_reset", "asc_init", "asc_decay", "asc_amps", "tau_syn",
             "spike_dependent_threshold", "after_spike_currents", "adapting_threshold"}
     d = os.path.join(golden_dir, "cell_models")
-    files = sorted(os.listdir(d))
+    files = sorted(f for f in os.listdir(d) if f.endswith("_glif_lif_asc_psc.json"))
     assert len(files) == 5
     for f in files:
         cell = json.load(open(os.path.join(d, f)))
