@@ -24,7 +24,7 @@ class Glif3Sim(C.Structure):
         ("n_inputs", c_int64), ("in_ptr", c_void_p), ("in_events", c_void_p),
         ("inp_indptr", c_void_p), ("inp_indices", c_void_p), ("inp_weights", c_void_p),
         ("inp_delays", c_void_p), ("inp_receptors", c_void_p), ("inp_packed", c_void_p), ("i_ext", c_void_p),
-        ("work_bits", c_void_p),
+        ("work_bits", c_void_p), ("delay_offset", c_int32), ("hist_slots", c_int32),
         ("res_span", c_int32), ("res_groups", c_int32), ("rec_seg", c_void_p), ("inp_seg", c_void_p),
         ("res_sync", c_void_p),
         ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),

@@ -20,6 +20,19 @@
 // t+1 and next overwritten in step t+3, which a workgroup can only reach after
 // the barrier of step t+2, i.e. after every workgroup finished reading it.
 //
+// With a delay offset B (tables hold delays shortened by B steps) step t pulls
+// the spikes of step t-1-B from a history of D rows, and a workgroup only has
+// to know that everybody has published step t-B before it starts step t+1: it
+// waits for the barrier of S = min(B, D-3-B, 31) steps ago, so workgroups drift
+// up to S steps apart and the wait is normally over before it begins.  Because
+// of the drift one running count cannot tell who has arrived where: there is a
+// counter per step, 64 of them used in turn (the fastest workgroup is at most
+// 2S+1 < 64 steps ahead of a waiting one), each compared with the number of
+// workgroups times the number of rounds it has served.  Row t%D is
+// overwritten in step t+D; by then its writer has seen every workgroup arrive
+// at the barrier of step t+D-1-S, hence finish the pull of step t+D-2-S, which
+// read the spikes of step t+D-3-S-B >= t.
+//
 // Every wait is bounded: a workgroup that spins too long on the barrier raises
 // the abort word, every other workgroup sees it and all leave the loop, so the
 // grid always drains.
@@ -32,6 +45,8 @@ namespace bmtk {
 
 constexpr int kResBlock = 1024;
 constexpr unsigned kMaxSpin = 4000000u;  // polls of the barrier word before giving up (seconds)
+constexpr int kBarrierWords = 64;        // per-step arrival counters, used round-robin
+constexpr int kMaxSlack = 31;
 
 #ifdef BMTK_RES_PROFILE
 __device__ unsigned long long g_prof[8];
@@ -45,6 +60,7 @@ __device__ unsigned long long g_prof[8];
 struct Resident {
     int64_t step0, n_steps;
     int span, n_groups;
+    int offset, hist, slack;  // B, D, S of the note above
 };
 
 __device__ __forceinline__ unsigned load_agent(const unsigned *p)
@@ -90,22 +106,23 @@ constexpr int kActCap = 8192;   // active-row list in LDS (entries)
 constexpr int kScanWords = 4;   // ballot words per thread and round
 constexpr unsigned kInputTag = 0x80000000u;
 
-// Spikes and input events of step `tp` -> this workgroup's ring slice.
+// Spikes and input events of step `tp`, handed over as if emitted in step
+// `ts` (= tp + delay offset) -> this workgroup's ring slice.
 // Round by round: every thread reads kScanWords ballot words and one input
 // event (independent loads), a workgroup-wide prefix sum packs the rows that
 // fired into one LDS list, then one thread per listed row pulls this
 // workgroup's segment of it.  Must be called by all threads of the workgroup.
-__device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int64_t tp,
+__device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int64_t tp, int64_t ts,
                                           float *ring_l, unsigned *act, unsigned *scan_l, int e0, int64_t words,
                                           int64_t k0, int64_t k1)
 {
     const int tid = threadIdx.x;
     const int L = s.ring_slots;
-    const int slot0 = (int)(tp % L);
+    const int slot0 = (int)(ts % L);
     const int wave = tid / kWave;
     const bool has_rec = s.rec_seg != nullptr;
     const unsigned long long *bits =
-        reinterpret_cast<const unsigned long long *>(s.work_bits) + (tp % 3) * (words + 1);
+        reinterpret_cast<const unsigned long long *>(s.work_bits) + (tp % r.hist) * (words + 1);
     const int64_t n_words = has_rec ? words : 0;
     const int64_t word_rounds = (n_words + (int64_t)kScanWords * kResBlock - 1) / ((int64_t)kScanWords * kResBlock);
     const int64_t event_rounds = (k1 - k0 + kResBlock - 1) / kResBlock;
@@ -202,8 +219,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     const bool own = tid < mine;
     const int64_t e = e0 + tid;
     unsigned *act = reinterpret_cast<unsigned *>(ring_l + s.ring_slots * GLIF3_NREC * r.span);
-    unsigned *barrier = s.res_sync;
     unsigned *abort_word = s.res_sync + 1;
+    unsigned *arrivals = s.res_sync + 2;  // [kBarrierWords]
 
     for (int c = tid; c < L * GLIF3_NREC * span; c += kResBlock) {
         const int dr = c / span, i = c - dr * span;
@@ -223,12 +240,15 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
     bool aborted = false;
     int64_t done = 0;  // steps whose update has run
-    // input events of step t-1 are in_events[ka, kb); the bound for the next step is fetched a step ahead
-    int64_t ka = 0, kb = s.in_ptr ? s.in_ptr[r.step0] : 0;
+    // the input events of the step pulled in step t, u = t-1-B, are in_events[ka, kb); the bound for the
+    // next step is fetched a step ahead.  Steps before 0 have no events (in_ptr[0] = 0).
+    const int B = r.offset;
+    auto in_bound = [&](int64_t i) -> int64_t { return (s.in_ptr && i > 0) ? s.in_ptr[i] : 0; };
+    int64_t ka = 0, kb = in_bound(r.step0 - B);
     for (int64_t k = 0; k < r.n_steps; ++k) {
         const int64_t t = r.step0 + k;
         PROF_T(c0);
-        const int64_t kn = s.in_ptr ? s.in_ptr[t + 1] : 0;
+        const int64_t kn = in_bound(t + 1 - B);
         // 1. fold the arrivals of slot t-1 and update
         bool spike = false;
         float frac = 0.0f;
@@ -247,7 +267,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         const unsigned long long m = __ballot(spike);
         // only the wavefronts that cover this workgroup's span own a ballot word
         if (lane == 0 && tid < span && (e & ~(int64_t)(kWave - 1)) < ne) {
-            __hip_atomic_store(reinterpret_cast<unsigned long long *>(s.work_bits) + (t % 3) * (words + 1) + (e >> 6),
+            __hip_atomic_store(reinterpret_cast<unsigned long long *>(s.work_bits) + (t % r.hist) * (words + 1) + (e >> 6),
                                m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (s.spike_bits) s.spike_bits[k * s.spike_bits_stride + (e >> 6)] = m;
         }
@@ -272,20 +292,26 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         __syncthreads();
         PROF_T(c1);
         // 2. arrive at the barrier of step t (ballots of this workgroup are out)
-        if (tid == 0) __hip_atomic_fetch_add(barrier, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0)
+            __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
         PROF_T(c2);
-        // 3. pull the spikes and input events of step t-1 while the barrier fills
-        if (k > 0 && mine > 0) pull_step(s, r, g, t - 1, ring_l, act, scan_l, e0, words, ka, kb);
+        // 3. pull the spikes and input events of step t-1-B while the barrier fills (the first step of a
+        //    call pulls nothing: the call before it closed with that pull)
+        if (k > 0 && t - 1 - B >= 0 && mine > 0)
+            pull_step(s, r, g, t - 1 - B, t - 1, ring_l, act, scan_l, e0, words, ka, kb);
         ka = kb;
         kb = kn;
         __syncthreads();
         PROF_T(c3);
-        // 4. wait for every workgroup's ballots of step t
+        // 4. wait for every workgroup's ballots of step t-S
         if (tid == 0) {
-            const unsigned target = gridDim.x * (unsigned)(k + 1);
+            const int64_t j = k - r.slack;  // the step (of this call) everybody must have published
+            const unsigned *word = arrivals + ((j < 0 ? 0 : j) & (kBarrierWords - 1));
+            const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
             unsigned spins = 0;
             int ok = 1;
-            while (load_agent(barrier) < target) {
+            while (load_agent(word) < target) {
                 if (load_agent(abort_word) != 0u) {
                     ok = 0;
                     break;
@@ -315,9 +341,9 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     }
 
     if (!aborted && done > 0) {
-        // closing: spikes and inputs of the last step, then fold the last slot
+        // closing: spikes and inputs of the last step (less the delay offset), then fold the last slot
         const int64_t tl = r.step0 + done - 1;
-        if (mine > 0) pull_step(s, r, g, tl, ring_l, act, scan_l, e0, words, ka, kb);
+        if (tl - B >= 0 && mine > 0) pull_step(s, r, g, tl - B, tl, ring_l, act, scan_l, e0, words, ka, kb);
         __syncthreads();
         if (own) {
             float *prev = ring_l + (int)(tl % L) * GLIF3_NREC * span + tid;
@@ -374,7 +400,10 @@ __global__ __launch_bounds__(kBlock) void segment_offsets_kernel(int64_t n_rows,
 
 int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream)
 {
-    Resident r{step0, n_steps, s.res_span, s.res_groups};
+    const int hist = s.hist_slots ? s.hist_slots : 3;
+    int slack = s.delay_offset < hist - 3 - s.delay_offset ? s.delay_offset : hist - 3 - s.delay_offset;
+    slack = slack < kMaxSlack ? slack : kMaxSlack;
+    Resident r{step0, n_steps, s.res_span, s.res_groups, s.delay_offset, hist, slack};
     const size_t lds = (size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) + kActCap * sizeof(int);
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(sim_resident_kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -393,7 +422,7 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
                   n_cu, per_cu);
         return BMTK_E_LAUNCH;
     }
-    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, stream, s.res_sync, 4);
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(128), 0, stream, s.res_sync, 2 + kBarrierWords);
     bmtk_glif3_sim s_copy = s;
     // BMTK_AMD_PLAIN_LAUNCH=1 uses an ordinary launch (co-residency then rests on the occupancy check
     // above and an otherwise idle device); for tools that cannot follow cooperative launches.

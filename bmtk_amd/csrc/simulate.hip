@@ -8,6 +8,9 @@
 //            synapses of every neuron that fired, adding the weights into the
 //            ring slots t..t+D-1 with fp32 atomics;
 //   input    the same for the external events emitted in step t-1.
+// With a delay offset B the tables hold delays shortened by B steps and the
+// deliver/input workgroups of launch t take the spikes and events of step
+// t-1-B from the history instead: same arrival slots, a ring B slots shorter.
 //
 // Folding arrivals one launch late is exact: NEST adds the weights that arrive
 // in step t to y1 at the end of step t (y1 = y1*P11 + s*psc0) and nothing reads
@@ -29,6 +32,8 @@ constexpr int kLdsTableBytes = 48 * 1024;
 
 struct SimLaunch {
     int64_t t;        // step being updated (closing launch: one past the last step)
+    int64_t src;      // step whose spikes and input events are delivered: t - 1 - delay_offset
+    int hist;         // rows of the spike-bit history
     int64_t out_row;  // row of spike_bits to write
     int n_update, n_deliver, n_input;
     int do_update;     // 0 in the closing launch: fold only
@@ -76,11 +81,11 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
     // Delivery workgroups take the lowest block ids so they are dispatched first and
     // their dependent-load chains run under the streaming update, not after it.
     if (bid < q.n_input) {
-        // ---- external input events emitted in step t-1 ----
+        // ---- external input events emitted in step t-1 (t-1-B with a delay offset B) ----
         // (not those of step t: with L = largest delay + 1 slots, a delay of L-1
         //  from step t would land in slot t-1, which this launch is clearing)
         const int slot0 = (int)((q.t - 1) % L);
-        const int64_t k0 = s.in_ptr[q.t - 1], k1 = s.in_ptr[q.t];
+        const int64_t k0 = s.in_ptr[q.src], k1 = s.in_ptr[q.src + 1];
         const int n_waves = q.n_input * kSimWaves;
         const int wave = bid * kSimWaves + threadIdx.x / kWave;
         for (int64_t k = k0 + wave; k < k1; k += n_waves) {
@@ -95,7 +100,7 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
         // ---- spikes of step t-1 ----
         if (!q.deliver_prev) return;
         const int slot0 = (int)((q.t - 1) % L);
-        const uint64_t *__restrict__ bits = s.work_bits + ((q.t - 1) % 3) * (words + 1);
+        const uint64_t *__restrict__ bits = s.work_bits + (q.src % q.hist) * (words + 1);
         const int64_t n_waves = (int64_t)q.n_deliver * kSimWaves;
         const int64_t wave = (int64_t)(bid - q.n_input) * kSimWaves + threadIdx.x / kWave;
         const int64_t per = (words + n_waves - 1) / n_waves;
@@ -181,7 +186,7 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
     const unsigned long long m = __ballot(spike);
     const int64_t wave_base = e & ~(int64_t)(kWave - 1);
     if (lane == 0 && wave_base < ne) {
-        s.work_bits[(q.t % 3) * (words + 1) + (e >> 6)] = m;
+        s.work_bits[(q.t % q.hist) * (words + 1) + (e >> 6)] = m;
         if (s.spike_bits) s.spike_bits[q.out_row * s.spike_bits_stride + (e >> 6)] = m;
     }
     if (s.spike_count && m != 0ull) {
@@ -254,6 +259,10 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     BMTK_REQUIRE(!s.spike_count || (s.spike_step && s.spike_elem && s.spike_cap > 0),
                  "glif3_simulate_fwd: spike record needs spike_step, spike_elem and a positive spike_cap");
     BMTK_REQUIRE(step0 >= 0 && n_steps >= 0, "glif3_simulate_fwd: step0 and n_steps must be non-negative");
+    const int hist = s.hist_slots ? s.hist_slots : 3;
+    BMTK_REQUIRE(s.delay_offset >= 0 && hist >= s.delay_offset + 3,
+                 "glif3_simulate_fwd: hist_slots must be at least delay_offset + 3");
+    BMTK_REQUIRE(!(s.save_v && s.delay_offset), "glif3_simulate_fwd: the per-step record needs delay_offset 0");
     if (n_steps == 0) return BMTK_OK;
     BMTK_REQUIRE((s.save_v == nullptr) == (s.save_flags == nullptr),
                  "glif3_simulate_fwd: save_v and save_flags go together");
@@ -285,11 +294,14 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     for (int64_t k = 0; k <= n_steps; ++k) {
         const bool closing = k == n_steps;
         q.t = step0 + k;
+        q.src = q.t - 1 - s.delay_offset;
+        q.hist = hist;
         q.out_row = k;
         q.do_update = closing ? 0 : 1;
         q.fold_prev = k > 0;
-        q.deliver_prev = (k > 0 && has_rec) ? 1 : 0;
-        q.n_input = k > 0 ? n_input : 0;
+        // the first launch of a call delivers nothing: the closing launch of the call before it did
+        q.deliver_prev = (k > 0 && q.src >= 0 && has_rec) ? 1 : 0;
+        q.n_input = (k > 0 && q.src >= 0) ? n_input : 0;
         const unsigned grid = (unsigned)(q.n_update + q.n_deliver + q.n_input);
         hipLaunchKernelGGL(sim_step_kernel, dim3(grid), dim3(kSimBlock), lds, (hipStream_t)stream, s, q);
     }

@@ -353,15 +353,18 @@ def _build():
                 a.append(src_map[s[mask]]); b.append(n_of[t[mask]]); c.append(ww); d.append(steps[mask])
                 e.append(np.full(int(mask.sum()), rec - 1))
     cat = lambda xs, dt_: np.concatenate(xs).astype(dt_) if xs else np.zeros(0, dt_)
-    max_delay = int(max([1] + [int(x.max()) for x in rd + id_ if x.size]))
-    if max_delay > 62:
-        raise _Errors.BadDelay("delays above 62 steps do not fit the delay ring buffer", "BadDelay")
     n = neuron_ids.size
-    rec = _net.coo_to_csr(cat(rs, np.int64), cat(rt, np.int64), cat(rw, np.float32), cat(rd, np.uint8),
+    rec = _net.coo_to_csr(cat(rs, np.int64), cat(rt, np.int64), cat(rw, np.float32), cat(rd, np.int64),
                           cat(rr, np.uint8), n_rows=n, major="source") if rs else None
-    inp = _net.coo_to_csr(cat(is_, np.int64), cat(it, np.int64), cat(iw, np.float32), cat(id_, np.uint8),
+    inp = _net.coo_to_csr(cat(is_, np.int64), cat(it, np.int64), cat(iw, np.float32), cat(id_, np.int64),
                           cat(ir, np.uint8), n_rows=max(1, gen_ids.size), major="source") if is_ else None
-    sim = Glif3Simulator(n, par, dt, rec=rec, inp=inp, ring_slots=max_delay + 1, asc_init=asc_init, u_init=u_init)
+    try:
+        # delays beyond the 63 steps of the ring are taken up by a delay offset (smallest delay - 1)
+        sim = Glif3Simulator(n, par, dt, rec=rec, inp=inp, asc_init=asc_init, u_init=u_init)
+    except ValueError as err:
+        if "delays span" in str(err):
+            raise _Errors.BadDelay(str(err), "BadDelay")
+        raise
     _S.sim = dict(sim=sim, neuron_ids=neuron_ids, gen_ids=gen_ids, n_of=n_of, steps_done=0)
 
 

@@ -30,7 +30,7 @@ def edge_weights(nsyns, syn_weight):
 
 
 def syn_spec_to_arrays(n_edges, syn_spec, dt):
-    """NEST ``syn_spec`` dict -> (weights f32, delay steps u8, receptor u8 0-based).
+    """NEST ``syn_spec`` dict -> (weights f32, delay steps u8 (int32 beyond 255), receptor u8 0-based).
 
     Scalars are broadcast over the batch; ``receptor_type`` is 1-based as in
     NEST; a delay below the resolution raises ``BadDelay``; delays are rounded
@@ -41,12 +41,11 @@ def syn_spec_to_arrays(n_edges, syn_spec, dt):
         raise BadDelay("synaptic \"delay\" value in edges ({}) is not compatible with simulator "
                        "resolution/\"dt\" ({})".format(np.min(delay_ms), dt))
     steps = np.rint(delay_ms / dt).astype(np.int64)
-    if np.any(steps > 255):
-        raise ValueError("delay of {} steps exceeds the 255-step limit of the ring buffer".format(steps.max()))
     rec = int(syn_spec.get("receptor_type", 1))
     if rec < 1 or rec > NREC:
         raise ValueError("receptor_type {} outside 1..{}".format(rec, NREC))
-    return (w.astype(np.float32), steps.astype(np.uint8), np.full(n_edges, rec - 1, np.uint8))
+    steps = steps.astype(np.uint8 if (steps.size == 0 or steps.max() <= 255) else np.int32)
+    return (w.astype(np.float32), steps, np.full(n_edges, rec - 1, np.uint8))
 
 
 def coo_to_csr(src, tgt, w, d, r, n_rows, major="source"):
@@ -62,8 +61,10 @@ def coo_to_csr(src, tgt, w, d, r, n_rows, major="source"):
     indptr = np.cumsum(indptr)
     if indptr[-1] >= 2 ** 31:
         raise ValueError("more than 2^31-1 synapses in one table")
+    d = np.asarray(d)
+    d = d.astype(np.uint8 if (d.size == 0 or d.max() <= 255) else np.int32)  # long delays keep a wide column
     return (indptr.astype(np.int32), col[order].astype(np.int32), np.asarray(w, np.float32)[order],
-            np.asarray(d, np.uint8)[order], np.asarray(r, np.uint8)[order])
+            d[order], np.asarray(r, np.uint8)[order])
 
 
 def csr_rows(indptr):

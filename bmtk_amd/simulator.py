@@ -22,11 +22,17 @@ class Glif3Simulator:
                 neuron, or per parameter class when ``class_id`` is given
     rec, inp    source-major synapse tables (numpy tuples, see bmtk_amd.network):
                 recurrent (rows = neurons) and external (rows = input sources)
-    ring_slots  slots of the delay ring buffer; default = largest delay + 1
+    ring_slots  slots of the delay ring buffer; default = largest (residual) delay + 1
+    delay_offset  B steps taken off every delay before the tables are built; spikes and input events are
+                then handed to the tables B steps late from a history of spike bits, which gives the same
+                arrivals with a ring B slots shorter.  "auto": 0 while the largest delay is at most 63
+                steps (what the ring and the packed tables hold), else the smallest delay minus one --
+                the case of NEST networks run at a fine resolution (1-2 ms delays at 0.001-0.1 ms steps).
+                The delay columns may then be any integer type; residual delays must stay within 63.
     """
 
     def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
-                 asc_init=None, u_init=None, i_ext=None, device=None, resident="auto"):
+                 asc_init=None, u_init=None, i_ext=None, device=None, resident="auto", delay_offset="auto"):
         self.lib = _lib.load()
         self.dev = device or _dev()
         self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
@@ -44,11 +50,34 @@ class Glif3Simulator:
             raise ValueError("par needs one column per neuron when class_id is not given")
         self.prop = glif3_precompute(par, h)
         self.class_id = None if class_id is None else torch.as_tensor(class_id, device=self.dev)
-        max_delay = 1
+        lo, hi = [], []
         for t in (rec, inp):
             if t is not None and len(t[3]):
-                max_delay = max(max_delay, int(t[3].max()))
-        self.L = int(ring_slots) if ring_slots else max_delay + 1
+                lo.append(int(t[3].min()))
+                hi.append(int(t[3].max()))
+        min_delay, max_delay = (min(lo), max(hi)) if lo else (1, 1)
+        if min_delay < 1:
+            raise ValueError("delays must be at least one step")
+        if delay_offset == "auto":
+            delay_offset = 0 if max_delay <= 63 else min_delay - 1
+        self.delay_offset = int(delay_offset)
+        if not 0 <= self.delay_offset < min_delay:
+            raise ValueError("delay_offset must lie in 0..smallest delay - 1")
+        if max_delay - self.delay_offset > 63:
+            raise ValueError("delays span {}..{} steps: after taking off {} the largest still exceeds the 63 steps "
+                             "the ring buffer holds".format(min_delay, max_delay, self.delay_offset))
+        def narrow(t):
+            return t is None or t[3].dtype == (torch.uint8 if torch.is_tensor(t[3]) else np.uint8)
+
+        if self.delay_offset or not (narrow(rec) and narrow(inp)):
+            def shorten(t):
+                if t is None:
+                    return None
+                d = t[3] - self.delay_offset
+                d = d.to(torch.uint8) if torch.is_tensor(d) else d.astype(np.uint8)
+                return (t[0], t[1], t[2], d, t[4])
+            rec, inp = shorten(rec), shorten(inp)
+        self.L = int(ring_slots) if ring_slots else max_delay - self.delay_offset + 1
         self.rec = self._table(rec, self.n) if rec is not None else None
         self.inp = self._table(inp, None) if inp is not None else None
         self.n_inputs = self.inp.n_rows if self.inp is not None else 0
@@ -61,10 +90,14 @@ class Glif3Simulator:
         self.in_steps = 0
         self.step = 0
         self.words = n_words(self.ne)
-        self.work_bits = torch.zeros(3 * (self.words + 1), dtype=torch.int64, device=self.dev)
+        # history of spike bits: 2B+3 rows let resident workgroups drift B steps apart, B+3 is the least
+        self.hist_slots = 2 * self.delay_offset + 3
+        if self.hist_slots * (self.words + 1) * 8 > 2 ** 30:
+            self.hist_slots = self.delay_offset + 3
+        self.work_bits = torch.zeros(self.hist_slots * (self.words + 1), dtype=torch.int64, device=self.dev)
         if self.n >= 2 ** 24:
             raise ValueError("the packed synapse tables index at most 2^24 neurons")
-        self.res_sync = torch.zeros(4, dtype=torch.int32, device=self.dev)
+        self.res_sync = torch.zeros(80, dtype=torch.int32, device=self.dev)
         self.res_span = self.res_groups = 0
         self.rec_seg = self.inp_seg = None
         self._pending_check = False
@@ -149,6 +182,7 @@ class Glif3Simulator:
             s.inp_packed = _p(self.inp.packed())
         s.i_ext = _p(self.i_ext)
         s.work_bits = _p(self.work_bits)
+        s.delay_offset, s.hist_slots = self.delay_offset, self.hist_slots
         if self.res_span:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
             s.rec_seg, s.inp_seg = _p(self.rec_seg), _p(self.inp_seg)
@@ -178,8 +212,8 @@ class Glif3Simulator:
         s = self._struct(bits, record)
         saved = None
         if save_state:
-            if self.res_span:
-                raise ValueError("save_state needs a simulator built with resident=False")
+            if self.res_span or self.delay_offset:
+                raise ValueError("save_state needs a simulator built with resident=False and delay_offset 0")
             saved = dict(v=torch.empty(n_steps, self.ne, device=self.dev),
                          flags=torch.empty(n_steps, self.ne, dtype=torch.uint8, device=self.dev), step0=self.step)
             s.save_v, s.save_flags = _p(saved["v"]), _p(saved["flags"])

@@ -515,17 +515,15 @@ class PointNetwork:
         self.virtual, self.n_inputs = virtual, n_inputs
 
     def tables(self):
-        """-> (rec, inp) source-major synapse tables; delays are still whole steps (int64) and may exceed what a
-        ring buffer of a given size takes — the simulator checks."""
+        """-> (rec, inp) source-major synapse tables; the delay column is uint8 when every delay fits, int32
+        otherwise (a Glif3Simulator takes such tables with a delay offset)."""
         out = []
         for edges, rows in ((self.rec_edges, self.n), (self.inp_edges, self.n_inputs)):
             if edges is None:
                 out.append(None)
                 continue
             src, tgt, w, d, r = edges
-            if d.size and d.max() > 255:
-                raise ValueError("a delay of {} steps does not fit the 8-bit delay column".format(d.max()))
-            out.append(net.coo_to_csr(src, tgt, w, d.astype(np.uint8), r, rows, "source"))
+            out.append(net.coo_to_csr(src, tgt, w, d, r, rows, "source"))
         return out
 
 

@@ -48,8 +48,8 @@ class Glif3Bptt:
     built with ``resident=False``."""
 
     def __init__(self, sim, dampening=0.3):
-        if sim.res_span:
-            raise ValueError("the backward pass needs a simulator built with resident=False")
+        if sim.res_span or sim.delay_offset:
+            raise ValueError("the backward pass needs a simulator built with resident=False and delay_offset 0")
         self.sim, self.dampening = sim, float(dampening)
         self.lib = _lib.load()
         dev, ne = sim.dev, sim.ne

@@ -172,7 +172,17 @@ typedef struct bmtk_glif3_sim {
     const uint8_t *inp_delays, *inp_receptors;
     const bmtk_synapse *inp_packed; /* required when in_ptr is set */
     const float *i_ext;          /* [ne] constant external current or NULL */
-    uint64_t *work_bits;         /* scratch, 3*(ceil(ne/64)+1) words: spike bits of the last steps */
+    uint64_t *work_bits;         /* history of spike bits, hist_slots rows of ceil(ne/64)+1 words: the spikes
+                                  * of step t live in row t % hist_slots.  Zero it before the first run and
+                                  * leave it alone between runs that continue one another. */
+    /* Long delays.  NEST networks have a minimum delay, often far above one step (1-2 ms at a 0.001-0.1 ms
+     * resolution).  With delay_offset = B every delay stored in the two tables is the true delay minus B steps
+     * (still >= 1) and the spikes and input events of step u are handed to the tables B steps late, from the
+     * history, so the ring only has to span the residual delays.  Results are identical to B = 0 with the true
+     * delays.  In resident mode workgroups may then run up to min(B, hist_slots - 3 - B) steps apart before
+     * one waits for another (at most 31) (what NEST's min_delay communication interval does between ranks). */
+    int32_t delay_offset;        /* B >= 0 */
+    int32_t hist_slots;          /* rows of work_bits, at least delay_offset + 3; 0 stands for 3 */
     /* Resident mode (optional, batch 1 only; res_span == 0 disables it): the
      * network is split into res_groups = ceil(ne/res_span) workgroups that keep
      * their elements' state in registers and their slice of the ring in LDS for
@@ -183,7 +193,7 @@ typedef struct bmtk_glif3_sim {
     int32_t res_groups;
     const uint32_t *rec_seg;     /* [neurons][res_groups+1] */
     const uint32_t *inp_seg;     /* [inputs][res_groups+1] */
-    uint32_t *res_sync;          /* 4 words of scratch: barrier counter, abort flag; zeroed by the call.
+    uint32_t *res_sync;          /* 80 words of scratch: abort flag, per-step arrival counters; zeroed by the call.
                                   * After the run, word 1 != 0 means the grid barrier timed out and the
                                   * results are invalid. */
     /* outputs */
@@ -216,7 +226,8 @@ typedef struct bmtk_glif3_sim {
  * move no membrane potential before step t+1: the update of step t+1 folds the
  * arrivals of slot t into y1 first (same two roundings as adding them at the
  * end of step t), so slot t need only be complete when launch t+1 starts.  The
- * closing launch delivers the spikes and input events of the last step and folds the last
+ * closing launch delivers the spikes and input events of the last step (with delay_offset = B: of
+ * step last-B; the B younger steps stay in the history for a run that continues) and folds the last
  * slot, after which state and ring are what a step-by-step evaluation gives.
  * Enqueues n_steps+1 launches on `stream` and returns.
  *

@@ -156,11 +156,18 @@ def step(st, prop, h, batch=1, class_id=None, syn=None, i_ext=None, want_frac=Fa
     return z, frac
 
 
+def _wide(csr):
+    """The C side reads delays as int32 (any number of steps); tables carry uint8 or wider columns."""
+    if csr is None or csr[0] is None:
+        return csr
+    return (csr[0], csr[1], csr[2], np.ascontiguousarray(csr[3], np.int32), csr[4])
+
+
 def deliver_events(active_e, batch, csr, ring, n_tgt, step_idx):
     """Event-driven delivery through a source-major CSR (indptr, indices=targets,
-    weights f32, delays u8, receptors u8) into ring[L][NREC][n_tgt*batch]."""
+    weights f32, delays in steps, receptors u8) into ring[L][NREC][n_tgt*batch]."""
     sfx, _ = _real(ring.dtype)
-    indptr, indices, weights, delays, receptors = csr
+    indptr, indices, weights, delays, receptors = _wide(csr)
     active_e = np.ascontiguousarray(active_e, np.int32)
     getattr(lib(), "csr_deliver_events" + sfx)(
         C.c_int64(active_e.size), _ptr(active_e), C.c_int32(batch), _ptr(indptr), _ptr(indices), _ptr(weights),
@@ -170,7 +177,7 @@ def deliver_events(active_e, batch, csr, ring, n_tgt, step_idx):
 def gather_rows(z, batch, csr, ring, n_tgt, step_idx):
     """Row-by-row sums over a target-major CSR (indices=sources), stored order."""
     sfx, _ = _real(ring.dtype)
-    indptr, indices, weights, delays, receptors = csr
+    indptr, indices, weights, delays, receptors = _wide(csr)
     z = np.ascontiguousarray(z, np.uint8)
     getattr(lib(), "csr_gather_rows" + sfx)(
         C.c_int64(n_tgt), C.c_int32(batch), _ptr(z), _ptr(indptr), _ptr(indices), _ptr(weights),
@@ -194,8 +201,8 @@ def simulate(st, prop, h, n_steps, batch=1, class_id=None, ring=None, rec=None, 
     s_elem = np.zeros(spike_cap, np.int32)
     s_frac = np.zeros(spike_cap, dtype)
     ras = np.zeros((n_steps, ne), np.uint8) if raster else None
-    rec = rec or (None,) * 5
-    inp = inp or (None,) * 5
+    rec = _wide(rec) or (None,) * 5
+    inp = _wide(inp) or (None,) * 5
     if in_ptr is not None:
         in_ptr = np.ascontiguousarray(in_ptr, np.int64)
         in_events = np.ascontiguousarray(in_events, np.int32)

@@ -119,7 +119,7 @@ void FN(glif3_step)(int64_t n_neurons, int32_t batch,
  */
 void FN(csr_deliver_events)(int64_t n_active, const int32_t *active_e, int32_t batch,
                             const int32_t *indptr, const int32_t *indices, const float *weights,
-                            const uint8_t *delays, const uint8_t *receptors,
+                            const int32_t *delays, const uint8_t *receptors,
                             REAL *ring, int32_t L, int64_t n_tgt, int64_t step)
 {
     const int64_t ne = n_tgt * (int64_t)batch;
@@ -153,7 +153,7 @@ void FN(csr_deliver_events)(int64_t n_active, const int32_t *active_e, int32_t b
  */
 void FN(csr_gather_rows)(int64_t n_tgt, int32_t batch, const uint8_t *z,
                          const int32_t *indptr, const int32_t *indices, const float *weights,
-                         const uint8_t *delays, const uint8_t *receptors,
+                         const int32_t *delays, const uint8_t *receptors,
                          REAL *ring, int32_t L, int64_t step)
 {
     const int64_t ne = n_tgt * (int64_t)batch;
@@ -186,10 +186,10 @@ int64_t FN(glif3_simulate)(int64_t n_neurons, int32_t batch, int64_t n_steps, in
                            const REAL *prop, int64_t prop_stride, const int32_t *class_id, REAL h,
                            REAL *ring, int32_t L,
                            const int32_t *r_indptr, const int32_t *r_indices, const float *r_weights,
-                           const uint8_t *r_delays, const uint8_t *r_receptors,
+                           const int32_t *r_delays, const uint8_t *r_receptors,
                            const int64_t *in_ptr, const int32_t *in_events,
                            const int32_t *i_indptr, const int32_t *i_indices, const float *i_weights,
-                           const uint8_t *i_delays, const uint8_t *i_receptors,
+                           const int32_t *i_delays, const uint8_t *i_receptors,
                            const REAL *i_ext,
                            int32_t *spk_step, int32_t *spk_elem, REAL *spk_frac, int64_t spk_cap,
                            uint8_t *raster)

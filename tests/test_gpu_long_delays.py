@@ -1,0 +1,130 @@
+"""Delays far above the 63 steps of the ring buffer: the delay offset.
+
+NEST networks run at fine resolutions (bmtk's examples: 0.001-0.01 ms with 1-2 ms delays, i.e. 100-2000 steps).
+The simulator takes the smallest delay minus one off every delay and hands spikes to the tables that many steps
+late from a history of spike bits.  That must be invisible: same raster and state as the oracle run with the
+true delays and a ring as long as the longest of them.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import glif3_oracle as orc
+from bmtk_amd import synthetic
+from bmtk_amd.glif_utils import convert_aibs2nest, params_table
+from bmtk_amd.simulator import Glif3Simulator
+
+pytestmark = pytest.mark.gpu
+
+
+def _exact(csr, extra_delay):
+    """Weights rounded to multiples of 1/4 pA (sums exact in fp32 whatever the order) and delays lengthened."""
+    indptr, indices, w, d, r = csr
+    return (indptr, indices, (np.round(w * 4.0) / 4.0 + np.sign(w) * 0.25).astype(np.float32),
+            d.astype(np.int32) + extra_delay, r)
+
+
+def _network(extra_delay, seed=9, steps=1000):
+    cfg = synthetic.small_glif3_network(n=3000, n_in=500, steps=steps, seed=seed, in_w_scale=3.0, in_fanout=300,
+                                        p_conn=0.03, w_scale=1.5)
+    cfg["rec_src"] = _exact(cfg["rec_src"], extra_delay)
+    cfg["inp_src"] = _exact(cfg["inp_src"], extra_delay)
+    return cfg
+
+
+def _oracle(cfg, dtype=np.float32):
+    orc.set_threads(1)
+    prop = orc.precompute(cfg["par"], cfg["h"])
+    st = orc.new_state(cfg["n"], 1, dtype)
+    L = int(max(cfg["rec_src"][3].max(), cfg["inp_src"][3].max())) + 1
+    ring = np.zeros((L, 4, cfg["n"]), dtype)
+    out = orc.simulate(st, prop, cfg["h"], cfg["steps"], class_id=cfg["class_id"], ring=ring, rec=cfg["rec_src"],
+                       inp=cfg["inp_src"], in_ptr=cfg["in_ptr"], in_events=cfg["in_events"], raster=True)
+    return out, st
+
+
+@pytest.mark.parametrize("resident", [False, True])
+@pytest.mark.parametrize("extra", [100, 300])
+def test_long_delays_equal_the_oracle_with_true_delays(extra, resident):
+    """True delays extra+1 .. extra+4 steps.  Bit-identical raster and state after 1000 steps run as 400 + 600
+    (the history has to carry the undelivered spikes across the two calls), on both drivers; dozens of resident
+    workgroups drift up to `extra` steps apart in between."""
+    cfg = _network(extra)
+    want, st = _oracle(cfg)
+    assert want["count"] > 2000
+    sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                         inp=cfg["inp_src"], resident=resident)
+    assert sim.delay_offset == extra and sim.L == 5 and bool(sim.res_span) == resident
+    assert sim.hist_slots == 2 * extra + 3
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    a = sim.run(400)
+    b = sim.run(600)
+    sim.check()
+    ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
+    np.testing.assert_array_equal(ras, want["raster"])
+    got = sim.state.to_numpy()
+    for k in ("V", "asc", "ref", "y2"):
+        np.testing.assert_array_equal(got[k], st[k], err_msg=k)
+
+
+@pytest.mark.parametrize("resident", [False, True])
+def test_offset_choice_does_not_change_results(resident):
+    """Delays 4..7 steps fit the ring as they are; taking 0, 2 or 3 steps off must give the same run."""
+    cfg = _network(3, seed=4, steps=600)
+    runs = []
+    for offset in (0, 2, 3):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], resident=resident, delay_offset=offset)
+        assert sim.delay_offset == offset and sim.L == 8 - offset
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        out = sim.run(600)
+        sim.check()
+        runs.append((sim.raster(out["bits"]).cpu().numpy(), sim.state.to_numpy()))
+    assert runs[0][0].sum() > 1500
+    for ras, st in runs[1:]:
+        np.testing.assert_array_equal(ras, runs[0][0])
+        for k in ("V", "asc", "ref", "y2"):
+            np.testing.assert_array_equal(st[k], runs[0][1][k], err_msg=k)
+
+
+def test_delay_spread_beyond_the_ring_is_refused():
+    cfg = _network(0)
+    indptr, indices, w, d, r = cfg["rec_src"]
+    d = d.copy()
+    d[0] = 200
+    with pytest.raises(ValueError, match="delays span"):
+        Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=(indptr, indices, w, d, r))
+    with pytest.raises(ValueError, match="delay_offset"):
+        Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"], delay_offset=1)
+
+
+@pytest.mark.parametrize("h,atol", [(0.01, 2e-3), (0.001, 2e-2)])
+def test_known_answer_at_fine_resolution(golden_dir, h, atol):
+    """The reference's known-answer protocol at the resolution its own test sets (0.001 ms; the 1 ms delay is
+    then 1000 steps) and at 0.01 ms: 14.46548367 ms / 14.77547828 ms
+    (bmtk/tests/simulator/pointnet/test_glif_utils.py:16-44, which allows 1.0 ms).  fp32 state over 50,000 steps
+    of 0.001 ms keeps the spike within 0.02 ms."""
+    kat = json.load(open(os.path.join(golden_dir, "glif_kat.json")))
+    pr = kat["protocol"]
+    for model, exp in kat["expected"].items():
+        aibs = json.load(open(os.path.join(golden_dir, exp["file"])))
+        _, cell = convert_aibs2nest(model, aibs)
+        par, asc_init, u_init = params_table([cell])
+        d = int(round(pr["delay_ms"] / h))
+        inp = (np.array([0, 1], np.int32), np.array([0], np.int32), np.array([pr["spike_weight_pA"]], np.float32),
+               np.array([d], np.int32), np.array([pr["receptor_type"] - 1], np.uint8))
+        n_steps = int(round(pr["tstop_ms"] / h))
+        stamps = np.rint(np.array(pr["spike_times_ms"]) / h).astype(np.int64)
+        in_ptr = np.zeros(n_steps + 1, np.int64)
+        np.add.at(in_ptr, stamps, 1)
+        sim = Glif3Simulator(1, par, h, inp=inp, asc_init=asc_init, u_init=u_init, resident=True)
+        assert sim.delay_offset == d - 1
+        sim.set_input_events(np.cumsum(in_ptr), np.zeros(len(stamps), np.int32))
+        rec = sim.run(n_steps, spike_bits=False, record_cap=16)["record"]
+        sim.check()
+        c = int(rec["count"].item())
+        assert c == len(exp["times"])
+        t = (rec["step"][:c].cpu().numpy() + rec["frac"][:c].cpu().numpy().astype(np.float64)) * h
+        np.testing.assert_allclose(t, exp["times"], atol=atol, rtol=0)

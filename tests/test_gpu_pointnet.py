@@ -140,3 +140,20 @@ def test_current_clamp_segments(tmp_path):
         want |= set(zip(out["step"].tolist(), out["elem"].tolist()))
     got = set(zip(np.floor(ts / dt + 1e-9).astype(int).tolist(), ids.tolist()))
     assert len(got & want) / max(1, len(got | want)) >= 0.999
+
+
+def test_example_at_its_own_resolution(tmp_path):
+    """The example's configured resolution, dt = 0.001 ms: its 2 ms delays are 2000 steps, far beyond the ring,
+    so the run rests on the delay offset (1999 steps) and a ring of 2 slots.  200 ms = 200,000 steps, resident
+    kernel; spike for spike equal to the fp32 oracle run with the true delays and a 2001-slot ring."""
+    dt, tstop = 0.001, 200.0
+    conf = pointnet.Config.from_json(_write_configs(str(tmp_path), dt, tstop))
+    graph = pointnet.PointNetwork.from_config(conf, unsupported="silence")
+    assert graph.rec_edges[3].min() == graph.rec_edges[3].max() == 2000
+    sim = pointnet.PointSimulator.from_config(conf, graph, resident=True)
+    ids, ts = sim.run()["v1"]
+    assert sim.simulator.delay_offset == 1999 and sim.simulator.L == 2 and sim.n_steps == 200000
+    want = _oracle_spikes(graph, dt, sim.n_steps, sim._trains, np.float32)
+    assert want["count"] > 1000
+    got = _pairs(np.floor(ts / dt + 1e-9).astype(int), ids)
+    assert got == _pairs(want["step"], want["elem"])
