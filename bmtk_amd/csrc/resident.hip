@@ -61,6 +61,7 @@ struct Resident {
     int64_t step0, n_steps;
     int span, n_groups;
     int offset, hist, slack;  // B, D, S of the note above
+    int check;                // the arrival counters are looked at every `check` steps (1 when S = 0)
 };
 
 __device__ __forceinline__ unsigned load_agent(const unsigned *p)
@@ -197,6 +198,8 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
     }
 }
 
+// kLate: the run has slack (S > 0), see the loop body
+template <bool kLate>
 __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim s, Resident r)
 {
     extern __shared__ float ring_l[];  // [L*4][span], then the active-row list
@@ -284,17 +287,26 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
             }
         }
         done = k + 1;
-        // Every wavefront waits until its own ballot store (a write-through, device-coherent
-        // store) has been acknowledged, then the workgroup meets; only after that does the
-        // barrier count move.  No L2 write-back is needed: nothing else written inside the
-        // loop is read by another workgroup before the kernel ends.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __syncthreads();
-        PROF_T(c1);
-        // 2. arrive at the barrier of step t (ballots of this workgroup are out)
-        if (tid == 0)
-            __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+        // With no slack (S = 0) the arrival is signalled before the pull so that the barrier fills while
+        // the pull runs.  With slack nobody is waiting for this step yet: the arrival moves behind the pull,
+        // which saves a workgroup barrier and the wait for the ballot store, and the counters are only
+        // looked at every `check` steps.
+        constexpr bool late = kLate;
+        const int check = late ? r.check : 1;
+        if (!late) {
+            // Every wavefront waits until its own ballot store (a write-through, device-coherent
+            // store) has been acknowledged, then the workgroup meets; only after that does the
+            // barrier count move.  No L2 write-back is needed: nothing else written inside the
+            // loop is read by another workgroup before the kernel ends.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+            PROF_T(c1);
+            // 2. arrive at the barrier of step t (ballots of this workgroup are out)
+            if (tid == 0)
+                __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            PROF_ADD(0, c0, c1);
+        }
         PROF_T(c2);
         // 3. pull the spikes and input events of step t-1-B while the barrier fills (the first step of a
         //    call pulls nothing: the call before it closed with that pull)
@@ -302,11 +314,18 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
             pull_step(s, r, g, t - 1 - B, t - 1, ring_l, act, scan_l, e0, words, ka, kb);
         ka = kb;
         kb = kn;
+        if (late) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         PROF_T(c3);
-        // 4. wait for every workgroup's ballots of step t-S
+        if (late && tid == 0)
+            __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        // 4. every `check` steps (each step without slack) wait until every workgroup has published
+        //    step k - S + (check - 1): enough for the steps up to the next look
+        if (late && k % check != check - 1 && k + 1 < r.n_steps) continue;
         if (tid == 0) {
-            const int64_t j = k - r.slack;  // the step (of this call) everybody must have published
+            int64_t j = late ? k - r.slack + (check - 1) : k;  // step of this call everybody must have published
+            j = j < k ? j : k;
             const unsigned *word = arrivals + ((j < 0 ? 0 : j) & (kBarrierWords - 1));
             const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
             unsigned spins = 0;
@@ -330,8 +349,6 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         }
         __syncthreads();
         PROF_T(c4);
-        PROF_ADD(0, c0, c1);
-        PROF_ADD(1, c1, c2);
         PROF_ADD(2, c2, c3);
         PROF_ADD(3, c3, c4);
         if (!go_on) {
@@ -403,10 +420,11 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     const int hist = s.hist_slots ? s.hist_slots : 3;
     int slack = s.delay_offset < hist - 3 - s.delay_offset ? s.delay_offset : hist - 3 - s.delay_offset;
     slack = slack < kMaxSlack ? slack : kMaxSlack;
-    Resident r{step0, n_steps, s.res_span, s.res_groups, s.delay_offset, hist, slack};
+    Resident r{step0, n_steps, s.res_span, s.res_groups, s.delay_offset, hist, slack, slack / 2 + 1};
     const size_t lds = (size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) + kActCap * sizeof(int);
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(sim_resident_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    const void *kernel = slack > 0 ? reinterpret_cast<const void *>(sim_resident_kernel<true>)
+                                   : reinterpret_cast<const void *>(sim_resident_kernel<false>);
+    hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) {
         set_error("glif3_simulate_fwd: resident mode needs %zu bytes of LDS: %s", lds, hipGetErrorString(err));
         return BMTK_E_LAUNCH;
@@ -416,7 +434,10 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     int dev = 0, n_cu = 0, per_cu = 0;
     (void)hipGetDevice(&dev);
     (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
-    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, sim_resident_kernel, kResBlock, lds);
+    if (slack > 0)
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, sim_resident_kernel<true>, kResBlock, lds);
+    else
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, sim_resident_kernel<false>, kResBlock, lds);
     if ((int64_t)per_cu * n_cu < (int64_t)grid) {
         set_error("glif3_simulate_fwd: %u resident workgroups do not fit the device (%d compute units x %d)", grid,
                   n_cu, per_cu);
@@ -428,12 +449,14 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     // above and an otherwise idle device); for tools that cannot follow cooperative launches.
     const char *plain = getenv("BMTK_AMD_PLAIN_LAUNCH");
     if (plain && plain[0] == '1') {
-        hipLaunchKernelGGL(sim_resident_kernel, dim3(grid), dim3(kResBlock), lds, stream, s_copy, r);
+        if (slack > 0)
+            hipLaunchKernelGGL(sim_resident_kernel<true>, dim3(grid), dim3(kResBlock), lds, stream, s_copy, r);
+        else
+            hipLaunchKernelGGL(sim_resident_kernel<false>, dim3(grid), dim3(kResBlock), lds, stream, s_copy, r);
         err = hipGetLastError();
     } else {
         void *args[] = {&s_copy, &r};
-        err = hipLaunchCooperativeKernel(reinterpret_cast<const void *>(sim_resident_kernel), dim3(grid),
-                                         dim3(kResBlock), args, lds, stream);
+        err = hipLaunchCooperativeKernel(kernel, dim3(grid), dim3(kResBlock), args, lds, stream);
     }
     if (err != hipSuccess) {
         set_error("glif3_simulate_fwd: launch of %u resident workgroups failed: %s", grid, hipGetErrorString(err));
