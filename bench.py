@@ -101,6 +101,37 @@ def bench_state_update(torch, steps=1000, warmup=50):
             "bytes_per_update": B_PER_UPDATE_PLAIN + 29 * 4}
 
 
+def bench_compaction(torch, steps=200, warmup=20):
+    """Spike compaction at the propagation workload's size: 51,978 neurons x 64 trials = 3.3 M elements at
+    5 Hz x 1 ms, from byte flags and from spike-bit words.  Algorithmic bytes: the scan reads 1 B (1 bit) per
+    element and writes 4 B per spike."""
+    from bmtk_amd import ops
+    n = 51978 * 64
+    g = torch.Generator(device="cuda").manual_seed(7)
+    z = (torch.rand(n, device="cuda", generator=g) < 5e-3).to(torch.uint8)
+    words = (n + 63) // 64
+    pad = torch.zeros(words * 64, dtype=torch.uint8, device="cuda")
+    pad[:n] = z
+    weights = (2 ** torch.arange(64, device="cuda", dtype=torch.int64))
+    bits = (pad.view(words, 64).to(torch.int64) * weights).sum(1)  # bit 63 wraps into the sign: intended
+    bits = torch.cat([bits, bits.new_zeros(1)])
+    comp = ops.SpikeCompactor(n)
+    out = []
+    for name, src, scan_bytes in (("flags", z, n), ("bits", bits, n // 8)):
+        for _ in range(warmup):
+            comp(src)
+        wall, dev = time_region(torch, lambda: [comp(src) for _ in range(steps)])
+        per = dev / steps
+        count = int(comp.count.item())
+        alg = scan_bytes + 4 * count
+        out.append({"kernel": "compact_count/scan/write (%s)" % name,
+                    "workload": "compaction of %d elements, %d spikes" % (n, count),
+                    "elements_per_s": n / per, "us_per_call": per * 1e6,
+                    "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None}})
+    return out
+
+
 def bench_propagation(torch, steps=200, warmup=20):
     """Isolated spike propagation: 51,978 neurons, Poisson(1000) in-degree
     (~52 M synapses), batch 64, Bernoulli spikes at 1, 5 and 20 Hz."""
@@ -306,7 +337,8 @@ def main():
                      "algorithmic_bytes_per_step": alg_step, "us_per_step": dev / K * 1e6},
     }
     if not args.no_kernels:
-        line["kernels"] = [bench_state_update(torch)] + bench_propagation(torch) + [bench_bptt(torch)]
+        line["kernels"] = ([bench_state_update(torch)] + bench_compaction(torch) + bench_propagation(torch) +
+                           [bench_bptt(torch)])
     if args.cpu_steps > 0:
         line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, min(args.cpu_steps, W + K))
     print(json.dumps(line))
