@@ -32,7 +32,8 @@ def _rel(got, want):
     return float(np.max(np.abs(got - want)) / max(np.max(np.abs(want)), 1e-30))
 
 
-@pytest.mark.parametrize("batch,seed,loss_kind", [(1, 2, "per_step"), (3, 4, "per_step"), (1, 5, "rates"), (4, 6, "rates")])
+@pytest.mark.parametrize("batch,seed,loss_kind", [(1, 2, "per_step"), (3, 4, "per_step"), (1, 5, "rates"), (4, 6, "rates"),
+                                                  (8, 8, "per_step"), (32, 9, "rates")])  # multiples of 4: four trials per lane
 def test_weight_gradients_match_autograd(batch, seed, loss_kind):
     cfg = _net(batch, seed)
     n, T, h = cfg["n"], cfg["steps"], cfg["h"]
