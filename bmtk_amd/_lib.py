@@ -27,6 +27,9 @@ class Glif3Sim(C.Structure):
         ("work_bits", c_void_p), ("delay_offset", c_int32), ("hist_slots", c_int32),
         ("res_span", c_int32), ("res_groups", c_int32), ("rec_seg", c_void_p), ("inp_seg", c_void_p),
         ("res_sync", c_void_p),
+        ("pull_indptr", c_void_p), ("pull_packed", c_void_p), ("pull_syn", c_void_p), ("pull_work", c_void_p),
+        ("pull_inp_indptr", c_void_p), ("pull_inp_packed", c_void_p), ("pull_inp_syn", c_void_p),
+        ("pull_inp_work", c_void_p), ("in_hist", c_void_p), ("in_hist_stride", c_int64),
         ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
         ("save_v", c_void_p), ("save_flags", c_void_p),
         ("spike_step", c_void_p), ("spike_elem", c_void_p), ("spike_frac", c_void_p),

@@ -109,7 +109,7 @@ constexpr unsigned kInputTag = 0x80000000u;
 
 // Spikes and input events of step `tp`, handed over as if emitted in step
 // `ts` (= tp + delay offset) -> this workgroup's ring slice.
-// Round by round: every thread reads kScanWords ballot words and one input
+// Pass by pass: every thread reads kScanWords ballot words and one input
 // event (independent loads), a workgroup-wide prefix sum packs the rows that
 // fired into one LDS list, then one thread per listed row pulls this
 // workgroup's segment of it.  Must be called by all threads of the workgroup.

@@ -40,6 +40,8 @@ struct SimLaunch {
     int fold_prev;     // slot t-1 holds arrivals not yet folded into y1
     int deliver_prev;  // work_bits buffer (t-1)%3 holds spikes not yet delivered
     int lds_table;     // propagator table staged in LDS
+    int pull;          // pull_syn holds the recurrent arrivals of step t-1, to be folded with slot t-1
+    int pull_inp;      // pull_inp_syn holds the input arrivals of step t-1
 };
 
 // walk one row of a packed table, four 64-synapse chunks in flight at a time
@@ -148,7 +150,9 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
                 for (int k = 0; k < GLIF3_NREC; ++k) {
                     const float psc0 = q.lds_table ? table[col * GLIF3_NPROP + GLIF3_PSC0_0 + k]
                                                    : s.prop[(GLIF3_PSC0_0 + k) * s.prop_stride + col];
-                    const float a = prev[k * ne];
+                    float a = prev[k * ne];
+                    if (q.pull) a = a + s.pull_syn[k * ne + e];
+                    if (q.pull_inp) a = a + s.pull_inp_syn[k * ne + e];
                     prev[k * ne] = 0.0f;
                     s.y1[k * ne + e] = s.y1[k * ne + e] + a * psc0;
                 }
@@ -164,7 +168,9 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
             if (q.fold_prev) {
 #pragma unroll
                 for (int k = 0; k < GLIF3_NREC; ++k) {
-                    const float a = prev[k * ne];
+                    float a = prev[k * ne];
+                    if (q.pull) a = a + s.pull_syn[k * ne + e];
+                    if (q.pull_inp) a = a + s.pull_inp_syn[k * ne + e];
                     prev[k * ne] = 0.0f;
                     st.y1[k] = st.y1[k] + a * p.psc0[k];
                 }
@@ -202,6 +208,24 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
             if (s.spike_frac) s.spike_frac[idx] = frac;
         }
     }
+}
+
+// one row of the input-event history: bit (source*batch+trial) for every event of the step
+__global__ __launch_bounds__(kBlock) void input_bits_kernel(const int64_t *__restrict__ in_ptr,
+                                                            const int32_t *__restrict__ in_events, int64_t step,
+                                                            unsigned long long *__restrict__ row)
+{
+    const int64_t k0 = in_ptr[step], k1 = in_ptr[step + 1];
+    for (int64_t k = k0 + (int64_t)blockIdx.x * kBlock + threadIdx.x; k < k1; k += (int64_t)gridDim.x * kBlock) {
+        const int e = in_events[k];
+        atomicOr(row + (e >> 6), 1ull << (e & 63));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void zero_row_kernel(unsigned long long *__restrict__ row, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) row[i] = 0ull;
 }
 
 __global__ __launch_bounds__(kBlock) void pack_kernel(int64_t nnz, const int32_t *__restrict__ indices,
@@ -260,7 +284,7 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
                  "glif3_simulate_fwd: spike record needs spike_step, spike_elem and a positive spike_cap");
     BMTK_REQUIRE(step0 >= 0 && n_steps >= 0, "glif3_simulate_fwd: step0 and n_steps must be non-negative");
     const int hist = s.hist_slots ? s.hist_slots : 3;
-    BMTK_REQUIRE(s.delay_offset >= 0 && hist >= s.delay_offset + 3,
+    BMTK_REQUIRE(s.delay_offset >= 0 && (hist >= s.delay_offset + 3 || (s.pull_packed && s.res_span == 0)),
                  "glif3_simulate_fwd: hist_slots must be at least delay_offset + 3");
     BMTK_REQUIRE(!(s.save_v && s.delay_offset), "glif3_simulate_fwd: the per-step record needs delay_offset 0");
     if (n_steps == 0) return BMTK_OK;
@@ -283,11 +307,26 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     }
 
     const int64_t words = (ne + 63) / 64;
+    const bool pull = has_rec && s.pull_packed != nullptr;
+    if (pull) {
+        BMTK_REQUIRE(s.pull_indptr && s.pull_syn && s.pull_work,
+                     "glif3_simulate_fwd: the pull form needs pull_indptr, pull_syn and pull_work");
+        BMTK_REQUIRE(s.delay_offset == 0 && hist == s.ring_slots,
+                     "glif3_simulate_fwd: the pull form needs delay_offset 0 and hist_slots == ring_slots");
+    }
+    const bool pull_inp = pull && has_inp && s.pull_inp_packed != nullptr;
+    if (pull_inp) {
+        BMTK_REQUIRE(s.pull_inp_indptr && s.pull_inp_syn && s.pull_inp_work && s.in_hist,
+                     "glif3_simulate_fwd: the pull form of the inputs needs pull_inp_indptr, pull_inp_syn, "
+                     "pull_inp_work and in_hist");
+        BMTK_REQUIRE(s.in_hist_stride >= (s.n_inputs * (int64_t)s.batch + 63) / 64 + 1,
+                     "glif3_simulate_fwd: in_hist_stride must hold ceil(n_inputs*batch/64)+1 words");
+    }
     SimLaunch q{};
     q.n_update = (int)((ne + kSimBlock - 1) / kSimBlock);
     const int64_t max_deliver = (words + kSimWaves - 1) / kSimWaves;  // at least one word per wavefront
-    q.n_deliver = has_rec ? (int)(max_deliver < 128 ? max_deliver : 128) : 0;
-    const int n_input = has_inp ? 64 : 0;
+    q.n_deliver = (has_rec && !pull) ? (int)(max_deliver < 128 ? max_deliver : 128) : 0;
+    const int n_input = (has_inp && !pull_inp) ? 64 : 0;
     const size_t table_bytes = (size_t)s.prop_stride * GLIF3_NPROP * sizeof(float);
     q.lds_table = (s.class_id && table_bytes <= (size_t)kLdsTableBytes) ? 1 : 0;
     const size_t lds = q.lds_table ? table_bytes : 0;
@@ -300,7 +339,33 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
         q.do_update = closing ? 0 : 1;
         q.fold_prev = k > 0;
         // the first launch of a call delivers nothing: the closing launch of the call before it did
-        q.deliver_prev = (k > 0 && q.src >= 0 && has_rec) ? 1 : 0;
+        q.deliver_prev = (k > 0 && q.src >= 0 && has_rec && !pull) ? 1 : 0;
+        q.pull = (pull && k > 0) ? 1 : 0;
+        if (q.pull) {
+            // everything that arrives in step t-1 over recurrent synapses, from the spikes of steps <= t-2
+            const int rc = bmtk_csr_propagate_pull(s.work_bits, words + 1, s.ring_slots, s.n_neurons, s.batch,
+                                                   s.pull_indptr, s.pull_packed, s.pull_syn, s.n_neurons, q.t - 1,
+                                                   s.pull_work, stream);
+            if (rc != BMTK_OK) return rc;
+        }
+        q.pull_inp = 0;
+        if (pull_inp && q.t >= 1) {
+            // the events of step t-1 become row (t-1) % L of the input history; what arrives in step t-1 is then
+            // summed from the rows of the steps before it
+            unsigned long long *row = reinterpret_cast<unsigned long long *>(s.in_hist) +
+                                      ((q.t - 1) % s.ring_slots) * s.in_hist_stride;
+            hipLaunchKernelGGL(zero_row_kernel, dim3((unsigned)((s.in_hist_stride + kBlock - 1) / kBlock)),
+                               dim3(kBlock), 0, (hipStream_t)stream, row, s.in_hist_stride);
+            hipLaunchKernelGGL(input_bits_kernel, dim3(16), dim3(kBlock), 0, (hipStream_t)stream, s.in_ptr,
+                               s.in_events, q.t - 1, row);
+            if (k > 0) {
+                const int rc = bmtk_csr_propagate_pull(s.in_hist, s.in_hist_stride, s.ring_slots, s.n_inputs, s.batch,
+                                                       s.pull_inp_indptr, s.pull_inp_packed, s.pull_inp_syn,
+                                                       s.n_neurons, q.t - 1, s.pull_inp_work, stream);
+                if (rc != BMTK_OK) return rc;
+                q.pull_inp = 1;
+            }
+        }
         q.n_input = (k > 0 && q.src >= 0) ? n_input : 0;
         const unsigned grid = (unsigned)(q.n_update + q.n_deliver + q.n_input);
         hipLaunchKernelGGL(sim_step_kernel, dim3(grid), dim3(kSimBlock), lds, (hipStream_t)stream, s, q);

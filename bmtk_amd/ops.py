@@ -210,6 +210,20 @@ class SynapseTable:
                             self.delays[order].contiguous(), self.receptors[order].contiguous(),
                             n_rows=self.n_rows, max_row=self.max_row)
 
+    def transposed(self, n_cols):
+        """source-major <-> target-major on the device, keeping the (row, column, position) order
+        (what ``bmtk_amd.network.csr_transpose`` does on the host)."""
+        dev = self.indices.device
+        rows = torch.repeat_interleave(torch.arange(self.n_rows, device=dev, dtype=torch.int32),
+                                       (self.indptr[1:] - self.indptr[:-1]).long())
+        order = torch.sort(self.indices.long(), stable=True).indices
+        counts = torch.bincount(self.indices.long(), minlength=n_cols)
+        indptr = torch.zeros(n_cols + 1, dtype=torch.int32, device=dev)
+        indptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+        return SynapseTable(indptr, rows[order].contiguous(), self.weights[order].contiguous(),
+                            self.delays[order].contiguous(), self.receptors[order].contiguous(), n_rows=n_cols,
+                            max_row=int(counts.max().item()) if counts.numel() else 0)
+
     def segment_offsets(self, span, n_groups):
         """uint32 [n_rows, n_groups+1] offsets of the first synapse per row whose index is >= g*span
         (stored in an int32 tensor).  Raises if a row is not sorted by index."""

@@ -23,6 +23,11 @@ class Glif3Simulator:
     rec, inp    source-major synapse tables (numpy tuples, see bmtk_amd.network):
                 recurrent (rows = neurons) and external (rows = input sources)
     ring_slots  slots of the delay ring buffer; default = largest (residual) delay + 1
+    pull        launch-per-step mode only: sum the recurrent arrivals of a step in one pass over a target-major
+                copy of the table from the spike-bit history, instead of pushing them into the ring with global
+                atomics as spikes occur -- the faster form for batched runs.  "auto": batch >= 8 (and delay_offset
+                0, network small enough for the activity map in LDS).  Recurrent arrivals still ahead at the end
+                of a run then live in the history, and ``ring`` holds the input arrivals only.
     delay_offset  B steps taken off every delay before the tables are built; spikes and input events are
                 then handed to the tables B steps late from a history of spike bits, which gives the same
                 arrivals with a ring B slots shorter.  "auto": 0 while the largest delay is at most 63
@@ -32,7 +37,8 @@ class Glif3Simulator:
     """
 
     def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
-                 asc_init=None, u_init=None, i_ext=None, device=None, resident="auto", delay_offset="auto"):
+                 asc_init=None, u_init=None, i_ext=None, device=None, resident="auto", delay_offset="auto",
+                 pull="auto"):
         self.lib = _lib.load()
         self.dev = device or _dev()
         self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
@@ -103,6 +109,28 @@ class Glif3Simulator:
         self._pending_check = False
         if resident:
             self._setup_resident(required=(resident is True))
+        self.pull_table = self.pull_syn = self.pull_work = None
+        self.pull_inp_table = self.pull_inp_syn = self.pull_inp_work = self.in_hist = None
+        can_pull = (self.rec is not None and not self.res_span and self.delay_offset == 0
+                    and self.L * ((self.n + 31) // 32) * 4 + 16 * 1024 <= 64 * 1024)
+        if pull is True and not can_pull:
+            raise ValueError("the pull form needs a recurrent table, launch-per-step mode, delay_offset 0 and "
+                             "ring_slots * n_neurons / 8 bytes of LDS (at most 48 KB)")
+        if can_pull and (pull is True or (pull == "auto" and self.batch >= 8)):
+            self.pull_table = self.rec.transposed(self.n)
+            self.pull_syn = torch.zeros(NREC, self.ne, device=self.dev)
+            need = self.lib.bmtk_csr_propagate_pull_workspace_bytes(self.L, self.n)
+            self.pull_work = torch.zeros(need // 4 + 1, dtype=torch.int32, device=self.dev)
+            # the history must hold one row per ring slot, row t % L = spikes of step t
+            self.hist_slots = self.L
+            self.work_bits = torch.zeros(self.hist_slots * (self.words + 1), dtype=torch.int64, device=self.dev)
+            if self.inp is not None and self.L * ((self.n_inputs + 31) // 32) * 4 + 16 * 1024 <= 64 * 1024:
+                self.pull_inp_table = self.inp.transposed(self.n)
+                self.pull_inp_syn = torch.zeros(NREC, self.ne, device=self.dev)
+                need = self.lib.bmtk_csr_propagate_pull_workspace_bytes(self.L, self.n_inputs)
+                self.pull_inp_work = torch.zeros(need // 4 + 1, dtype=torch.int32, device=self.dev)
+                self.in_hist_stride = n_words(self.n_inputs * self.batch) + 1
+                self.in_hist = torch.zeros(self.L * self.in_hist_stride, dtype=torch.int64, device=self.dev)
 
     def _setup_resident(self, required):
         """Resident mode keeps state in registers and the ring in LDS for a whole
@@ -183,6 +211,13 @@ class Glif3Simulator:
         s.i_ext = _p(self.i_ext)
         s.work_bits = _p(self.work_bits)
         s.delay_offset, s.hist_slots = self.delay_offset, self.hist_slots
+        if self.pull_table is not None:
+            s.pull_indptr, s.pull_packed = _p(self.pull_table.indptr), _p(self.pull_table.packed())
+            s.pull_syn, s.pull_work = _p(self.pull_syn), _p(self.pull_work)
+            if self.pull_inp_table is not None and self.in_ptr is not None:
+                s.pull_inp_indptr, s.pull_inp_packed = _p(self.pull_inp_table.indptr), _p(self.pull_inp_table.packed())
+                s.pull_inp_syn, s.pull_inp_work = _p(self.pull_inp_syn), _p(self.pull_inp_work)
+                s.in_hist, s.in_hist_stride = _p(self.in_hist), self.in_hist_stride
         if self.res_span:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
             s.rec_seg, s.inp_seg = _p(self.rec_seg), _p(self.inp_seg)

@@ -196,6 +196,25 @@ typedef struct bmtk_glif3_sim {
     uint32_t *res_sync;          /* 80 words of scratch: abort flag, per-step arrival counters; zeroed by the call.
                                   * After the run, word 1 != 0 means the grid barrier timed out and the
                                   * results are invalid. */
+    /* Pull form of the recurrent delivery for batched runs (optional; launch-per-step mode with delay_offset 0
+     * and hist_slots == ring_slots): a TARGET-major packed copy of the recurrent table.  The recurrent arrivals
+     * of step t-1 are then summed in one pass over that table from the spike-bit history
+     * (bmtk_csr_propagate_pull) before the launch of step t, instead of being pushed into the ring with global
+     * atomics as the spikes occur.  Recurrent arrivals still ahead at the end of a call then live in the
+     * history (work_bits), not in `ring`, which holds the input arrivals only. */
+    const int32_t *pull_indptr;      /* [n_neurons + 1] */
+    const bmtk_synapse *pull_packed; /* rows = targets, index field = source */
+    float *pull_syn;                 /* [4][ne] scratch */
+    void *pull_work;                 /* bmtk_csr_propagate_pull_workspace_bytes(ring_slots, n_neurons) bytes */
+    /* The same for the external inputs (optional, only together with the above): a target-major packed copy of
+     * the input table and a history of input-event bits, row t % ring_slots = the events of step t as bits of
+     * element ids source*batch+trial; the driver fills the rows from in_ptr/in_events as it goes. */
+    const int32_t *pull_inp_indptr;      /* [n_neurons + 1] */
+    const bmtk_synapse *pull_inp_packed; /* rows = targets, index field = input source */
+    float *pull_inp_syn;                 /* [4][ne] scratch */
+    void *pull_inp_work;                 /* bmtk_csr_propagate_pull_workspace_bytes(ring_slots, n_inputs) bytes */
+    uint64_t *in_hist;                   /* [ring_slots][in_hist_stride], zeroed before the first run */
+    int64_t in_hist_stride;              /* >= ceil(n_inputs*batch/64) + 1 */
     /* outputs */
     uint64_t *spike_bits;        /* [n_steps][words] spike bits per step, words = ceil(ne/64); or NULL.
                                   * Row k belongs to step step0+k of the call that wrote it. */

@@ -250,3 +250,32 @@ def ops_popcount(bits):
     import torch
     x = bits.reshape(-1)
     return sum(int(((x >> s) & 1).sum()) for s in range(64))
+
+
+@pytest.mark.parametrize("batch", [3, 32, 64])
+def test_pull_form_of_the_per_step_driver(batch):
+    """Batched runs sum the recurrent arrivals of a step in one pass over a target-major copy of the table
+    (no global atomics).  With exact weights the run must equal the fp32 oracle bit for bit -- raster and state,
+    after 150 + 250 steps as two calls (the history carries the spikes still under way across the calls) -- and
+    so must the run that pushes arrivals into the ring."""
+    cfg = synthetic.small_glif3_network(n=700, n_in=300, steps=400, seed=12, in_w_scale=3.0, in_fanout=100,
+                                        p_conn=0.05, w_scale=1.5, batch=batch)
+    cfg["rec_src"] = _integer_weights(cfg["rec_src"])
+    cfg["inp_src"] = _integer_weights(cfg["inp_src"])
+    want, st, _ = _oracle_run(cfg, np.float32, batch=batch)
+    assert want["count"] > 1000 * batch // 4
+    for pull in (True, False):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], ring_slots=cfg["L"], resident=False, pull=pull)
+        assert (sim.pull_table is not None) == pull
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        a = sim.run(150)
+        b = sim.run(250)
+        ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
+        np.testing.assert_array_equal(ras, want["raster"])
+        got = sim.state.to_numpy()
+        for k in ("V", "asc", "y1", "y2", "ref"):
+            np.testing.assert_array_equal(got[k], st[k], err_msg=k)
+    auto = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
+                          resident=False)
+    assert (auto.pull_table is not None) == (batch >= 8)
