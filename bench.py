@@ -224,7 +224,8 @@ def bench_bptt(torch, steps=600):
     deg = (sim.rec.indptr[1:] - sim.rec.indptr[:-1]).long()
     spikes = res["counts"].view(n, batch).sum(1)
     events = int((spikes.long() * deg).sum().item())
-    return {"kernel": "sim_step_kernel + bwd_gather_kernel + bwd_state_kernel + bwd_rec_grad_kernel",
+    return {"kernel": "sim_step_kernel + pull_kernel (forward), bwd_gather4_kernel + bwd_state_kernel + bwd_rec_grad_kernel + "
+                      "bwd_inp_grad_kernel (backward)",
             "workload": "BPTT step N=51978 nnz=%d inputs=17400 batch=32 steps=%d" % (sim.rec.nnz, steps),
             "seconds_per_training_step": t_f + t_b, "forward_s": t_f, "backward_s": t_b,
             "mean_rate_hz": float(res["counts"].float().mean().item()) / steps * 1e3,
@@ -277,6 +278,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--cpu-steps", type=int, default=3000, help="steps of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the isolated-kernel measurements")
+    ap.add_argument("--kernels", default="state,compaction,propagation,bptt",
+                    help="which isolated-kernel measurements to run (comma-separated)")
     ap.add_argument("--per-step", action="store_true", help="force one launch per step instead of resident mode")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy 10 times (reference for scaling the FETCH_SIZE / "
@@ -337,8 +340,14 @@ def main():
                      "algorithmic_bytes_per_step": alg_step, "us_per_step": dev / K * 1e6},
     }
     if not args.no_kernels:
-        line["kernels"] = ([bench_state_update(torch)] + bench_compaction(torch) + bench_propagation(torch) +
-                           [bench_bptt(torch)])
+        want = set(args.kernels.split(","))
+        unknown = want - {"state", "compaction", "propagation", "bptt"}
+        if unknown:
+            sys.exit("bench.py: unknown --kernels entries: %s" % ", ".join(sorted(unknown)))
+        line["kernels"] = (([bench_state_update(torch)] if "state" in want else []) +
+                           (bench_compaction(torch) if "compaction" in want else []) +
+                           (bench_propagation(torch) if "propagation" in want else []) +
+                           ([bench_bptt(torch)] if "bptt" in want else []))
     if args.cpu_steps > 0:
         line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, min(args.cpu_steps, W + K))
     print(json.dumps(line))
