@@ -52,17 +52,23 @@ __device__ __forceinline__ unsigned long long bcast_u64(unsigned long long v, in
     return ((unsigned long long)hi << 32) | lo;
 }
 
-// inclusive prefix sum over the 64 lanes
+// inclusive prefix sum over the 64 lanes, with data-parallel-primitive moves (no LDS round trips): sums of 4
+// by three one-lane shifts within a row of 16, then shifts by 4 and 8 confined to the lanes that have such a
+// neighbour, then the last lane of row 0 (2) is added to row 1 (3) and lane 31 to the upper half
+#define BMTK_DPP(src, ctrl, row_mask, bank_mask) \
+    ((unsigned)__builtin_amdgcn_update_dpp(0, (int)(src), (ctrl), (row_mask), (bank_mask), false))
 __device__ __forceinline__ unsigned wave_inclusive_scan(unsigned v)
 {
-    const int lane = lane_id();
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const unsigned o = __shfl_up(v, off, kWave);
-        if (lane >= off) v += o;
-    }
-    return v;
+    unsigned t = v + BMTK_DPP(v, 0x111, 0xF, 0xF);  // row_shr:1
+    t += BMTK_DPP(v, 0x112, 0xF, 0xF);              // row_shr:2
+    t += BMTK_DPP(v, 0x113, 0xF, 0xF);              // row_shr:3
+    t += BMTK_DPP(t, 0x114, 0xF, 0xE);              // row_shr:4, lanes 4..15 of each row
+    t += BMTK_DPP(t, 0x118, 0xF, 0xC);              // row_shr:8, lanes 8..15
+    t += BMTK_DPP(t, 0x142, 0xA, 0xF);              // row_bcast:15 into rows 1 and 3
+    t += BMTK_DPP(t, 0x143, 0xC, 0xF);              // row_bcast:31 into rows 2 and 3
+    return t;
 }
+#undef BMTK_DPP
 
 // exclusive prefix sum over the 256 threads of a workgroup; *total gets the block sum
 __device__ __forceinline__ unsigned block_exclusive_scan(unsigned v, unsigned *total)

@@ -148,13 +148,10 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
         if (lane_id() == kWave - 1) scan_l[wave] = inc;
         __syncthreads();
         PROF_T(p1);
-        unsigned base = 0, total = 0;
-#pragma unroll
-        for (int q = 0; q < kResBlock / kWave; ++q) {
-            const unsigned x = scan_l[q];
-            if (q < wave) base += x;
-            total += x;
-        }
+        // prefix over the 16 wavefront sums: one LDS read per lane and one more scan instead of 16 reads
+        const unsigned part = wave_inclusive_scan(lane_id() < kResBlock / kWave ? scan_l[lane_id()] : 0u);
+        const unsigned total = (unsigned)bcast_i((int)part, kResBlock / kWave - 1);
+        const unsigned base = wave > 0 ? (unsigned)__shfl((int)part, wave - 1, kWave) : 0u;
         const bool listed = total <= (unsigned)kActCap;
         unsigned pos = base + inc - cnt;
 #pragma unroll
