@@ -311,8 +311,12 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
             pull_step(s, r, g, t - 1 - B, t - 1, ring_l, act, scan_l, e0, words, ka, kb);
         ka = kb;
         kb = kn;
-        if (late) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __syncthreads();
+        if (late) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+        }
+        // (without slack no workgroup barrier is needed here: pull_step ends with one, and the word thread 0
+        //  writes below was last read before the barrier that precedes the arrival)
         PROF_T(c3);
         if (late && tid == 0)
             __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
