@@ -152,26 +152,33 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
         const unsigned part = wave_inclusive_scan(lane_id() < kResBlock / kWave ? scan_l[lane_id()] : 0u);
         const unsigned total = (unsigned)bcast_i((int)part, kResBlock / kWave - 1);
         const unsigned base = wave > 0 ? (unsigned)__shfl((int)part, wave - 1, kWave) : 0u;
-        const bool listed = total <= (unsigned)kActCap;
-        unsigned pos = base + inc - cnt;
+        const bool listed = total <= (unsigned)kActCap;  // workgroup-uniform
+        if (listed) {
+            unsigned pos = base + inc - cnt;
 #pragma unroll
-        for (int u = 0; u < kScanWords; ++u) {
-            unsigned long long x = v[u];
-            const int64_t j0 = (w0 + (int64_t)u * kResBlock + tid) << 6;
-            while (x) {
-                const int bit = __ffsll((long long)x) - 1;
-                x &= x - 1ull;
-                if (listed)
-                    act[pos++] = (unsigned)(j0 + bit);
-                else  // more rows than the list holds: pull directly, unbalanced but correct
+            for (int u = 0; u < kScanWords; ++u) {
+                unsigned long long x = v[u];
+                const unsigned j0 = (unsigned)((w0 + (int64_t)u * kResBlock + tid) << 6);
+                while (x) {
+                    const int bit = __ffsll((long long)x) - 1;
+                    x &= x - 1ull;
+                    act[pos++] = j0 + (unsigned)bit;
+                }
+            }
+            if (has_event) act[pos] = event_row | kInputTag;
+        } else {
+            // more rows than the list holds: every thread pulls what it found itself, unbalanced but correct
+            for (int u = 0; u < kScanWords; ++u) {
+                unsigned long long x = v[u];
+                const int64_t j0 = (w0 + (int64_t)u * kResBlock + tid) << 6;
+                while (x) {
+                    const int bit = __ffsll((long long)x) - 1;
+                    x &= x - 1ull;
                     pull_segment(s.rec_seg + (j0 + bit) * (r.n_groups + 1), g, s.rec_packed, ring_l, r.span, e0, L,
                                  slot0);
+                }
             }
-        }
-        if (has_event) {
-            if (listed)
-                act[pos++] = event_row | kInputTag;
-            else
+            if (has_event)
                 pull_segment(s.inp_seg + (int64_t)event_row * (r.n_groups + 1), g, s.inp_packed, ring_l, r.span, e0,
                              L, slot0);
         }
@@ -179,12 +186,14 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
         PROF_T(p2);
         if (listed) {
             for (unsigned a = tid; a < total; a += kResBlock) {
+                // one code path for both kinds of rows: a wavefront nearly always holds some of each, and a
+                // branch would make it walk the two chains of dependent loads one after the other
                 const unsigned entry = act[a];
                 const int64_t row = entry & ~kInputTag;
-                if (entry & kInputTag)
-                    pull_segment(s.inp_seg + row * (r.n_groups + 1), g, s.inp_packed, ring_l, r.span, e0, L, slot0);
-                else
-                    pull_segment(s.rec_seg + row * (r.n_groups + 1), g, s.rec_packed, ring_l, r.span, e0, L, slot0);
+                const bool is_input = (entry & kInputTag) != 0u;
+                const uint32_t *seg = is_input ? s.inp_seg : s.rec_seg;
+                const bmtk_synapse *tab = is_input ? s.inp_packed : s.rec_packed;
+                pull_segment(seg + row * (r.n_groups + 1), g, tab, ring_l, r.span, e0, L, slot0);
             }
         }
         __syncthreads();
