@@ -52,6 +52,8 @@ class Glif3Bwd(C.Structure):
     ]
 
 
+ABI_VERSION = 3  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
     "bmtk_amd_abi_version": (c_int32, []),
@@ -102,6 +104,9 @@ def load(build_if_missing=True):
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = res, args
+    if lib.bmtk_amd_abi_version() != ABI_VERSION:
+        raise LibraryMissing("{} has ABI version {}, these bindings are for {}; rebuild it".format(
+            LIB_PATH, lib.bmtk_amd_abi_version(), ABI_VERSION))
     if lib.bmtk_glif3_sim_sizeof() != C.sizeof(Glif3Sim) or lib.bmtk_glif3_bwd_sizeof() != C.sizeof(Glif3Bwd):
         raise LibraryMissing("{} was built from a different include/bmtk_amd.h (struct size {} vs {}); rebuild it"
                              .format(LIB_PATH, lib.bmtk_glif3_sim_sizeof(), C.sizeof(Glif3Sim)))

@@ -313,7 +313,7 @@ using namespace bmtk;
 
 extern "C" {
 
-int bmtk_amd_abi_version(void) { return 1; }
+int bmtk_amd_abi_version(void) { return BMTK_AMD_ABI_VERSION; }
 
 const char *bmtk_amd_last_error(void) { return g_error; }
 

@@ -47,6 +47,9 @@ extern "C" {
 #define BMTK_E_LAUNCH (-2) /* HIP reported an error for the launch */
 #define BMTK_E_DEVICE (-3) /* no usable gfx950 device */
 
+/* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
+ * library was built with. */
+#define BMTK_AMD_ABI_VERSION 3
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */

@@ -25,7 +25,9 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), name
     assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
-    assert lib.bmtk_amd_abi_version() >= 1
+    declared = int(re.search(r"#define BMTK_AMD_ABI_VERSION (\d+)",
+                             open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()).group(1))
+    assert lib.bmtk_amd_abi_version() == declared == _lib.ABI_VERSION
 
 
 @pytest.mark.parametrize("cname,mirror,sizeof", [("bmtk_glif3_sim", "Glif3Sim", "bmtk_glif3_sim_sizeof"),
