@@ -27,8 +27,11 @@ def test_bad_delay_and_receptor():
         net.syn_spec_to_arrays(1, {"weight": 1.0, "delay": 1.0, "receptor_type": 5}, dt=0.1)
     with pytest.raises(ValueError):
         net.syn_spec_to_arrays(1, {"weight": 1.0, "delay": 1.0, "receptor_type": 0}, dt=0.1)
-    with pytest.raises(ValueError):
-        net.syn_spec_to_arrays(1, {"weight": 1.0, "delay": 300.0}, dt=1.0)
+    # delays beyond 255 steps keep a wide column (the simulator takes them with a delay offset)
+    w, d, r = net.syn_spec_to_arrays(2, {"weight": 1.0, "delay": 300.0}, dt=1.0)
+    assert d.dtype == np.int32 and list(d) == [300, 300]
+    w, d, r = net.syn_spec_to_arrays(2, {"weight": 1.0, "delay": 3.0}, dt=1.0)
+    assert d.dtype == np.uint8 and list(d) == [3, 3]
 
 
 def test_check_csr_rejects_what_a_kernel_would_trip_over():
