@@ -1,0 +1,75 @@
+"""Randomly shaped small networks through every forward driver.
+
+Sizes that are not multiples of a wavefront, a single neuron, rows without synapses, no inputs at all, odd
+batches, one-step and six-step delays, long delays, parameter classes or per-neuron parameters: with weights that
+are multiples of 1/4 pA (sums exact in fp32, whatever their order) every driver must reproduce the fp32 oracle's
+raster and state bit for bit.
+"""
+import numpy as np
+import pytest
+
+from oracle import glif3_oracle as orc
+from bmtk_amd import synthetic
+from bmtk_amd.simulator import Glif3Simulator
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.choice([1, 2, 63, 64, 65, 130, 333, 900]))
+    n_in = int(rng.choice([0, 1, 7, 40]))
+    batch = int(rng.choice([1, 1, 1, 2, 5, 8, 16]))
+    max_delay = int(rng.choice([1, 2, 4, 6]))
+    extra = int(rng.choice([0, 0, 0, 70]))
+    classes = int(rng.choice([0, 0, 3])) or None
+    steps = 150
+    cfg = synthetic.small_glif3_network(n=n, n_in=n_in, steps=steps, seed=seed, p_conn=float(rng.choice([0.0, 0.05, 0.5])),
+                                        in_rate=60.0, in_fanout=max(1, min(n, 20)), max_delay=max_delay,
+                                        n_classes=classes, batch=batch, w_scale=6.0, in_w_scale=40.0)
+    for key in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = cfg[key]
+        cfg[key] = (indptr, indices, (np.round(w * 4.0) / 4.0 + np.sign(w) * 0.25).astype(np.float32),
+                    d.astype(np.int32) + extra, r)
+    cfg["extra"] = extra
+    # a constant current per element, strong enough for a good part of the cells to fire without any input
+    cfg["i_ext"] = rng.uniform(0.0, 600.0, n * batch).astype(np.float32)
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_every_driver_equals_the_oracle(seed):
+    cfg = _case(seed)
+    n, batch, steps = cfg["n"], cfg["batch"], cfg["steps"]
+    has_rec = cfg["rec_src"][1].size > 0
+    has_inp = cfg["n_in"] > 0
+    rec = cfg["rec_src"] if has_rec else None
+    inp = cfg["inp_src"] if has_inp else None
+    L = int(max([1] + [int(t[3].max()) for t in (rec, inp) if t is not None])) + 1
+    orc.set_threads(1)
+    prop = orc.precompute(cfg["par"], cfg["h"])
+    st = orc.new_state(n, batch, np.float32)
+    ring = np.zeros((L, 4, n * batch), np.float32)
+    want = orc.simulate(st, prop, cfg["h"], steps, batch=batch, class_id=cfg["class_id"], ring=ring, rec=rec, inp=inp,
+                        in_ptr=cfg["in_ptr"] if has_inp else None, in_events=cfg["in_events"] if has_inp else None,
+                        i_ext=cfg["i_ext"], raster=True)
+    assert want["count"] > 0
+    drivers = [dict(resident=False, pull=False)]
+    if has_rec and cfg["extra"] == 0:
+        drivers.append(dict(resident=False, pull=True))
+    if batch == 1:
+        drivers.append(dict(resident=True))
+    for kw in drivers:
+        sim = Glif3Simulator(n, cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=rec, inp=inp,
+                             i_ext=cfg["i_ext"], **kw)
+        assert sim.delay_offset == (cfg["extra"] if (has_rec or has_inp) and cfg["extra"] else 0)
+        if has_inp:
+            sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        a = sim.run(60)
+        b = sim.run(steps - 60)
+        sim.check()
+        ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
+        np.testing.assert_array_equal(ras, want["raster"], err_msg=str(kw))
+        got = sim.state.to_numpy()
+        for k in ("V", "asc", "y2", "ref"):
+            np.testing.assert_array_equal(got[k], st[k], err_msg="%s %s" % (k, kw))
