@@ -42,13 +42,16 @@ struct SimLaunch {
     int lds_table;     // propagator table staged in LDS
     int pull;          // pull_syn holds the recurrent arrivals of step t-1, to be folded with slot t-1
     int pull_inp;      // pull_inp_syn holds the input arrivals of step t-1
+    int idx_bits;      // width of the index field of the packed tables (24 in the standard packing)
 };
 
 // walk one row of a packed table, four 64-synapse chunks in flight at a time
 __device__ __forceinline__ void deliver_row_packed(const int32_t *__restrict__ indptr,
                                                    const bmtk_synapse *__restrict__ syn, int j, int b, int batch,
-                                                   float *__restrict__ ring, int L, int slot0, int64_t ne)
+                                                   float *__restrict__ ring, int L, int slot0, int64_t ne,
+                                                   int idx_bits)
 {
+    const unsigned idx_mask = (1u << idx_bits) - 1u;
     const int p0 = indptr[j], p1 = indptr[j + 1];
     if (p1 <= p0) return;
     const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(syn);
@@ -60,10 +63,10 @@ __device__ __forceinline__ void deliver_row_packed(const int32_t *__restrict__ i
         for (int u = 0; u < 4; ++u) {
             if (base + u * kWave < p1) {
                 const unsigned tdr = s[u].x;
-                int slot = slot0 + (int)(tdr >> 26);
+                int slot = slot0 + (int)(tdr >> (idx_bits + 2));
                 slot = slot >= L ? slot - L : slot;
-                const int r = (tdr >> 24) & 3;
-                const int64_t i = tdr & 0xFFFFFFu;
+                const int r = (tdr >> idx_bits) & 3;
+                const int64_t i = tdr & idx_mask;
                 atomicAdd(ring + ((int64_t)(slot * GLIF3_NREC + r) * ne + i * batch + b), __uint_as_float(s[u].y));
             }
         }
@@ -93,7 +96,7 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
         for (int64_t k = k0 + wave; k < k1; k += n_waves) {
             const int e = s.in_events[k];
             const int j = batch == 1 ? e : (int)((uint32_t)e / (uint32_t)batch);
-            deliver_row_packed(s.inp_indptr, s.inp_packed, j, e - j * batch, batch, s.ring, L, slot0, ne);
+            deliver_row_packed(s.inp_indptr, s.inp_packed, j, e - j * batch, batch, s.ring, L, slot0, ne, q.idx_bits);
         }
         return;
     }
@@ -121,7 +124,7 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
                     vl &= vl - 1ull;
                     const int es = (int)(e0 + bit);
                     const int j = batch == 1 ? es : (int)((uint32_t)es / (uint32_t)batch);
-                    deliver_row_packed(s.rec_indptr, s.rec_packed, j, es - j * batch, batch, s.ring, L, slot0, ne);
+                    deliver_row_packed(s.rec_indptr, s.rec_packed, j, es - j * batch, batch, s.ring, L, slot0, ne, q.idx_bits);
                 }
             }
         }
@@ -242,9 +245,36 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(int64_t nnz, const int32_t
     packed[p] = o;
 }
 
+__global__ __launch_bounds__(kBlock) void pack_wide_kernel(int64_t nnz, const int32_t *__restrict__ indices,
+                                                           const float *__restrict__ weights,
+                                                           const int32_t *__restrict__ delays,
+                                                           const uint8_t *__restrict__ receptors, int idx_bits,
+                                                           bmtk_synapse *__restrict__ packed)
+{
+    const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (p >= nnz) return;
+    bmtk_synapse o;
+    o.tdr = (uint32_t)indices[p] | ((uint32_t)receptors[p] << idx_bits) | ((uint32_t)delays[p] << (idx_bits + 2));
+    o.weight = weights[p];
+    packed[p] = o;
+}
+
 }  // namespace bmtk
 
 using namespace bmtk;
+
+extern "C" int bmtk_csr_pack_wide(int64_t nnz, const int32_t *indices, const float *weights, const int32_t *delays,
+                                  const uint8_t *receptors, int32_t delay_bits, bmtk_synapse *packed, void *stream)
+{
+    BMTK_REQUIRE(nnz >= 0 && nnz < (1ll << 31), "csr_pack_wide: nnz must lie in 0..2^31-1");
+    BMTK_REQUIRE(delay_bits >= 6 && delay_bits <= 14, "csr_pack_wide: delay_bits must lie in 6..14");
+    if (nnz == 0) return BMTK_OK;
+    BMTK_REQUIRE(indices && weights && delays && receptors && packed, "csr_pack_wide: pointers must be non-null");
+    hipLaunchKernelGGL(pack_wide_kernel, dim3((unsigned)((nnz + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, nnz, indices, weights, delays, receptors, 30 - delay_bits, packed);
+    BMTK_CHECK_LAUNCH("csr_pack_wide");
+    return BMTK_OK;
+}
 
 extern "C" int bmtk_csr_pack(int64_t nnz, const int32_t *indices, const float *weights, const uint8_t *delays,
                              const uint8_t *receptors, bmtk_synapse *packed, void *stream)
@@ -265,9 +295,14 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     BMTK_REQUIRE(s.n_neurons > 0 && s.batch > 0, "glif3_simulate_fwd: n_neurons and batch must be positive");
     const int64_t ne = s.n_neurons * (int64_t)s.batch;
     BMTK_REQUIRE(ne < (1ll << 31), "glif3_simulate_fwd: n_neurons*batch must stay below 2^31");
-    BMTK_REQUIRE(s.n_neurons < (1ll << 24), "glif3_simulate_fwd: the packed tables index at most 2^24 neurons");
-    BMTK_REQUIRE(s.ring_slots > 1 && s.ring_slots <= 64,
-                 "glif3_simulate_fwd: ring_slots must exceed the largest delay and stay within 2..64");
+    const int delay_bits = s.delay_bits ? s.delay_bits : 6;
+    BMTK_REQUIRE(delay_bits >= 6 && delay_bits <= 14, "glif3_simulate_fwd: delay_bits must be 0 or lie in 6..14");
+    BMTK_REQUIRE(delay_bits == 6 || (s.res_span == 0 && s.pull_packed == nullptr),
+                 "glif3_simulate_fwd: wide delay fields are read by the launch-per-step driver without the pull form only");
+    BMTK_REQUIRE(s.n_neurons < (1ll << (30 - delay_bits)) && (s.in_ptr == nullptr || s.n_inputs < (1ll << 24)),
+                 "glif3_simulate_fwd: more neurons than the index field of the packed tables holds");
+    BMTK_REQUIRE(s.ring_slots > 1 && s.ring_slots <= (1 << delay_bits),
+                 "glif3_simulate_fwd: ring_slots must exceed the largest delay and stay within 2..2^delay_bits");
     BMTK_REQUIRE(s.h > 0.0f, "glif3_simulate_fwd: resolution h must be positive");
     BMTK_REQUIRE(s.V && s.asc && s.y1 && s.y2 && s.ref && s.prop && s.ring && s.work_bits,
                  "glif3_simulate_fwd: state, prop, ring and work_bits pointers must be non-null");
@@ -335,6 +370,7 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
         q.t = step0 + k;
         q.src = q.t - 1 - s.delay_offset;
         q.hist = hist;
+        q.idx_bits = 30 - delay_bits;
         q.out_row = k;
         q.do_update = closing ? 0 : 1;
         q.fold_prev = k > 0;

@@ -191,13 +191,21 @@ class SynapseTable:
         return self._max_delay
 
     def packed(self):
-        """The table as 8-byte {index | receptor<<24 | delay<<26, weight} records (built once)."""
+        """The table as 8-byte {index | receptor<<24 | delay<<26, weight} records (built once); with
+        ``delay_bits`` above 6 (set by the simulator for delay spreads beyond 63 steps) the delay field is that
+        wide and the index field correspondingly narrower."""
         if getattr(self, "_packed", None) is None:
-            if self.max_delay() >= 64:
-                raise ValueError("packed tables hold delays below 64 steps")
+            bits = getattr(self, "delay_bits", 6)
+            if self.max_delay() >= (1 << bits):
+                raise ValueError("packed tables hold delays below {} steps".format(1 << bits))
             lib = _lib.load()
             out = torch.empty(max(self.nnz, 1), 2, dtype=torch.int32, device=self.indices.device)
-            _lib.check(lib.bmtk_csr_pack(self.nnz, *self.pointers()[1:], _p(out), _stream()))
+            if bits == 6:
+                _lib.check(lib.bmtk_csr_pack(self.nnz, *self.pointers()[1:], _p(out), _stream()))
+            else:
+                _lib.check(lib.bmtk_csr_pack_wide(self.nnz, _p(self.indices), _p(self.weights),
+                                                  _p(self.delays.to(torch.int32).contiguous()), _p(self.receptors),
+                                                  bits, _p(out), _stream()))
             self._packed = out
         return self._packed
 
@@ -239,7 +247,8 @@ class SynapseTable:
     def pointers(self):
         nnz = self.nnz
         return (_p(self.indptr, torch.int32, self.n_rows + 1, "indptr"), _p(self.indices, torch.int32, nnz, "indices"),
-                _p(self.weights, torch.float32, nnz, "weights"), _p(self.delays, torch.uint8, nnz, "delays"),
+                _p(self.weights, torch.float32, nnz, "weights"),
+                _p(self.delays, torch.uint8, nnz, "delays") if self.delays.dtype == torch.uint8 else None,
                 _p(self.receptors, torch.uint8, nnz, "receptors"))
 
 

@@ -69,23 +69,41 @@ class Glif3Simulator:
         self.delay_offset = int(delay_offset)
         if not 0 <= self.delay_offset < min_delay:
             raise ValueError("delay_offset must lie in 0..smallest delay - 1")
-        if max_delay - self.delay_offset > 63:
-            raise ValueError("delays span {}..{} steps: after taking off {} the largest still exceeds the 63 steps "
-                             "the ring buffer holds".format(min_delay, max_delay, self.delay_offset))
+        # residual delays beyond 63 steps: a wider delay field and a longer ring, which only the launch-per-step
+        # driver (without the pull form) handles
+        residual = max_delay - self.delay_offset
+        self.delay_bits = 6 if residual <= 63 else max(7, int(residual).bit_length())
+        if self.delay_bits > 6:
+            ring_bytes = (residual + 1) * NREC * self.ne * 4
+            if (self.delay_bits > 14 or self.n >= 2 ** (30 - self.delay_bits) or ring_bytes > 8 << 30
+                    or resident is True or pull is True):
+                raise ValueError("delays span {}..{} steps: after taking off {} the largest still exceeds the 63 steps "
+                                 "the ring buffer of the resident and pull forms holds, or what the wide form takes "
+                                 "({} ring bytes, {} neurons)".format(min_delay, max_delay, self.delay_offset,
+                                                                      ring_bytes, self.n))
+            resident = pull = False
+        wide = self.delay_bits > 6
+
         def narrow(t):
             return t is None or t[3].dtype == (torch.uint8 if torch.is_tensor(t[3]) else np.uint8)
 
-        if self.delay_offset or not (narrow(rec) and narrow(inp)):
+        if self.delay_offset or wide or not (narrow(rec) and narrow(inp)):
             def shorten(t):
                 if t is None:
                     return None
                 d = t[3] - self.delay_offset
-                d = d.to(torch.uint8) if torch.is_tensor(d) else d.astype(np.uint8)
+                if torch.is_tensor(d):
+                    d = d.to(torch.int32 if wide else torch.uint8)
+                else:
+                    d = d.astype(np.int32 if wide else np.uint8)
                 return (t[0], t[1], t[2], d, t[4])
             rec, inp = shorten(rec), shorten(inp)
         self.L = int(ring_slots) if ring_slots else max_delay - self.delay_offset + 1
         self.rec = self._table(rec, self.n) if rec is not None else None
         self.inp = self._table(inp, None) if inp is not None else None
+        for t in (self.rec, self.inp):
+            if t is not None:
+                t.delay_bits = self.delay_bits
         self.n_inputs = self.inp.n_rows if self.inp is not None else 0
         self.state = Glif3State.zeros(self.n, self.batch, asc_init=asc_init, u_init=u_init, device=self.dev)
         self.ring = torch.zeros(self.L, NREC, self.ne, device=self.dev)
@@ -210,7 +228,7 @@ class Glif3Simulator:
             s.inp_packed = _p(self.inp.packed())
         s.i_ext = _p(self.i_ext)
         s.work_bits = _p(self.work_bits)
-        s.delay_offset, s.hist_slots = self.delay_offset, self.hist_slots
+        s.delay_offset, s.hist_slots, s.delay_bits = self.delay_offset, self.hist_slots, self.delay_bits
         if self.pull_table is not None:
             s.pull_indptr, s.pull_packed = _p(self.pull_table.indptr), _p(self.pull_table.packed())
             s.pull_syn, s.pull_work = _p(self.pull_syn), _p(self.pull_work)

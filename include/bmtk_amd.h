@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 3
+#define BMTK_AMD_ABI_VERSION 4
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -141,6 +141,13 @@ int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_stride, int
 int bmtk_csr_pack(int64_t nnz, const int32_t *indices, const float *weights, const uint8_t *delays,
                   const uint8_t *receptors, bmtk_synapse *packed, void *stream);
 
+/* The same with a wider delay field, for delay spreads beyond 63 steps: tdr = index | receptor << (30 - delay_bits)
+ * | delay << (32 - delay_bits), delay_bits in 6..14, index < 2^(30 - delay_bits), delay < 2^delay_bits (int32
+ * input).  Only the launch-per-step driver without the pull form reads such tables (bmtk_glif3_sim.delay_bits);
+ * its ring then has up to 2^delay_bits slots in device memory. */
+int bmtk_csr_pack_wide(int64_t nnz, const int32_t *indices, const float *weights, const int32_t *delays,
+                       const uint8_t *receptors, int32_t delay_bits, bmtk_synapse *packed, void *stream);
+
 /* Per-row segment offsets of a SOURCE-MAJOR table whose rows are sorted by
  * target: seg[row*(n_groups+1) + g] = position of the first synapse of the row
  * whose target is >= g*span (g = 0..n_groups; the last entry is the row end).
@@ -186,6 +193,10 @@ typedef struct bmtk_glif3_sim {
      * one waits for another (at most 31) (what NEST's min_delay communication interval does between ranks). */
     int32_t delay_offset;        /* B >= 0 */
     int32_t hist_slots;          /* rows of work_bits, at least delay_offset + 3; 0 stands for 3 */
+    int32_t delay_bits;          /* width of the delay field of rec_packed / inp_packed: 0 or 6 = the standard
+                                  * packing; 7..14 = bmtk_csr_pack_wide tables (launch-per-step mode without the
+                                  * pull form only), ring_slots may then reach 2^delay_bits */
+    int32_t _pad2;
     /* Resident mode (optional, batch 1 only; res_span == 0 disables it): the
      * network is split into res_groups = ceil(ne/res_span) workgroups that keep
      * their elements' state in registers and their slice of the ring in LDS for

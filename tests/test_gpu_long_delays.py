@@ -89,15 +89,33 @@ def test_offset_choice_does_not_change_results(resident):
             np.testing.assert_array_equal(st[k], runs[0][1][k], err_msg=k)
 
 
-def test_delay_spread_beyond_the_ring_is_refused():
-    cfg = _network(0)
-    indptr, indices, w, d, r = cfg["rec_src"]
-    d = d.copy()
-    d[0] = 200
-    with pytest.raises(ValueError, match="delays span"):
-        Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=(indptr, indices, w, d, r))
+def test_delay_spread_beyond_63_steps():
+    """Delays scattered over 81..400 steps (bmtk's point_neuropixels example mixes 0.8, 1.5 and 2.0 ms at a
+    0.001 ms resolution): the offset takes off 80, the remaining spread needs a 9-bit delay field and a ring of
+    321 slots, which the launch-per-step driver handles; the resident and pull forms refuse."""
+    cfg = _network(0, seed=5, steps=900)
+    rng = np.random.default_rng(3)
+    for key in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = cfg[key]
+        cfg[key] = (indptr, indices, w, rng.integers(81, 401, d.size).astype(np.int32), r)
+    want, st = _oracle(cfg)
+    assert want["count"] > 2000
+    sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                         inp=cfg["inp_src"])
+    assert sim.delay_offset == 80 and sim.delay_bits == 9 and sim.L <= 321 and not sim.res_span
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    a = sim.run(500)
+    b = sim.run(400)
+    ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
+    np.testing.assert_array_equal(ras, want["raster"])
+    got = sim.state.to_numpy()
+    for k in ("V", "asc", "ref", "y2"):
+        np.testing.assert_array_equal(got[k], st[k], err_msg=k)
+    for kw in (dict(resident=True), dict(resident=False, pull=True)):
+        with pytest.raises(ValueError, match="delays span"):
+            Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"], **kw)
     with pytest.raises(ValueError, match="delay_offset"):
-        Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"], delay_offset=1)
+        Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"], delay_offset=500)
 
 
 @pytest.mark.parametrize("h,atol", [(0.01, 2e-3), (0.001, 2e-2)])
