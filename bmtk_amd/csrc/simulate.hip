@@ -321,7 +321,6 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     const int hist = s.hist_slots ? s.hist_slots : 3;
     BMTK_REQUIRE(s.delay_offset >= 0 && (hist >= s.delay_offset + 3 || (s.pull_packed && s.res_span == 0)),
                  "glif3_simulate_fwd: hist_slots must be at least delay_offset + 3");
-    BMTK_REQUIRE(!(s.save_v && s.delay_offset), "glif3_simulate_fwd: the per-step record needs delay_offset 0");
     if (n_steps == 0) return BMTK_OK;
     BMTK_REQUIRE((s.save_v == nullptr) == (s.save_flags == nullptr),
                  "glif3_simulate_fwd: save_v and save_flags go together");

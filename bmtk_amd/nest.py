@@ -26,6 +26,7 @@ import numpy as np
 
 from . import network as _net
 from .glif_utils import params_table
+from .layout import PAR as _PAR
 
 __version__ = "3.3-bmtk_amd"
 
@@ -102,8 +103,9 @@ def _ids_of(nodes):
 
 
 _NEURON, _GENERATOR, _RECORDER, _CURRENT = "glif_psc", "spike_generator", "spike_recorder", "step_current_generator"
+_MULTIMETER = "multimeter"
 _MODELS = {"glif_psc": _NEURON, "spike_generator": _GENERATOR, "spike_recorder": _RECORDER,
-           "spike_detector": _RECORDER, "step_current_generator": _CURRENT}
+           "spike_detector": _RECORDER, "step_current_generator": _CURRENT, "multimeter": _MULTIMETER}
 
 
 class _State(object):
@@ -115,6 +117,8 @@ class _State(object):
         self.edges = []         # (src ids, tgt ids, weights f64, delay ms f64, receptor 1-based)
         self.rec_links = []     # (neuron ids, recorder id)
         self.cur_links = []     # (generator id, neuron ids)
+        self.mm_links = []      # (multimeter id, neuron ids)
+        self.mm_events = {}     # multimeter id -> (senders, times, V_m)
         self.sim = None         # built Glif3Simulator and its id maps
         self.events = {}        # recorder id -> (senders, times)
 
@@ -184,6 +188,8 @@ def Create(model, n=1, params=None):
         p = dict(p or {})
         if kind == _NEURON:
             _check_neuron(p)
+        if kind == _MULTIMETER:
+            _check_multimeter(p)
         _S.kind.append(kind)
         _S.params.append(p)
     nodes = NodeCollection(range(first, first + n))
@@ -212,8 +218,26 @@ def _check_neuron(p):
     p.update(full)
 
 
+def _check_multimeter(p):
+    """What bmtk's membrane reports ask of a multimeter (bmtk/simulator/pointnet/modules/multimeter_reporter.py:
+    21-46,113-115): V_m of a list of cells, every ``interval`` ms between ``start`` and ``stop``, to an ascii file."""
+    names = p.get("record_from", ["V_m"])
+    names = [names] if isinstance(names, str) else list(names)
+    if names != ["V_m"]:
+        raise _Errors.BadProperty("the GPU path's multimeter records V_m only, not {}".format(names))
+    p["record_from"] = names
+    p.setdefault("interval", 1.0)
+    p.setdefault("start", 0.0)
+    p.setdefault("stop", float("inf"))
+
+
 def _set_one(node, params):
     kind = _S.kind[node - 1]
+    if kind == _MULTIMETER and "interval" in params:
+        dt = _S.status["resolution"]
+        k = float(params["interval"]) / dt
+        if k < 1.0 - 1e-9 or abs(k - round(k)) > 1e-6:
+            raise _Errors.BadProperty("the sampling interval must be a multiple of the resolution")
     if kind == _GENERATOR and "spike_times" in params:
         st = np.array(params["spike_times"], np.float64)
         if st.size and (np.any(st <= 0.0) or np.any(np.diff(st) < 0)):
@@ -237,7 +261,7 @@ def SetStatus(nodes, params, val=None):
     ids = _ids_of(nodes)
     plist = params if isinstance(params, (list, tuple)) else [params] * len(ids)
     for node, p in zip(ids, plist):
-        if _S.sim is not None and _S.kind[node - 1] != _RECORDER:
+        if _S.sim is not None and _S.kind[node - 1] not in (_RECORDER, _MULTIMETER):
             raise NESTError("node parameters cannot change after the first Simulate")
         _set_one(node, dict(p))
 
@@ -250,6 +274,10 @@ def GetStatus(nodes, keys=None):
         if _S.kind[node - 1] == _RECORDER:
             senders, times = _S.events.get(node, (np.zeros(0, np.int64), np.zeros(0)))
             d["events"] = {"senders": senders, "times": times}
+            d["n_events"] = len(times)
+        if _S.kind[node - 1] == _MULTIMETER:
+            senders, times, vm = _S.mm_events.get(node, (np.zeros(0, np.int64), np.zeros(0), np.zeros(0)))
+            d["events"] = {"senders": senders, "times": times, "V_m": vm}
             d["n_events"] = len(times)
         out.append(d if keys is None else d[keys] if isinstance(keys, str) else tuple(d[k] for k in keys))
     return tuple(out)
@@ -267,6 +295,12 @@ def Connect(pre, post, conn_spec=None, syn_spec=None):
             raise NESTError("only neurons can be connected to a spike recorder")
         for r in tgt:
             _S.rec_links.append((np.array(src, np.int64), r))
+        return
+    if kinds_src == {_MULTIMETER}:
+        if kinds_tgt != {_NEURON}:
+            raise NESTError("a multimeter connects to neurons")
+        for m in src:
+            _S.mm_links.append((m, np.array(tgt, np.int64)))
         return
     if kinds_src == {_CURRENT}:
         if kinds_tgt != {_NEURON}:
@@ -317,7 +351,7 @@ def GetConnections(source=None, target=None):
         out.extend(zip(s.tolist(), t.tolist()))
     for ids, r in _S.rec_links:
         out.extend((int(i), r) for i in ids)
-    for g, ids in _S.cur_links:
+    for g, ids in _S.cur_links + _S.mm_links:
         out.extend((g, int(i)) for i in ids)
     return out
 
@@ -360,12 +394,15 @@ def _build():
                           cat(ir, np.uint8), n_rows=max(1, gen_ids.size), major="source") if is_ else None
     try:
         # delays beyond the 63 steps of the ring are taken up by a delay offset (smallest delay - 1)
-        sim = Glif3Simulator(n, par, dt, rec=rec, inp=inp, asc_init=asc_init, u_init=u_init)
+        # a membrane record is kept by the launch-per-step driver only
+        sim = Glif3Simulator(n, par, dt, rec=rec, inp=inp, asc_init=asc_init, u_init=u_init,
+                             **(dict(resident=False, pull=False) if _S.mm_links else {}))
     except ValueError as err:
         if "delays span" in str(err):
             raise _Errors.BadDelay(str(err), "BadDelay")
         raise
-    _S.sim = dict(sim=sim, neuron_ids=neuron_ids, gen_ids=gen_ids, n_of=n_of, steps_done=0)
+    _S.sim = dict(sim=sim, neuron_ids=neuron_ids, gen_ids=gen_ids, n_of=n_of, steps_done=0,
+                  e_l=par[_PAR["E_L"]].copy())
 
 
 def _current_at(step):
@@ -413,14 +450,34 @@ def Simulate(t_ms):
             k = int(round((tt + dt) / dt))
             if step0 < k < step0 + n_steps:
                 bounds.add(k)
+    if _S.mm_links:  # the per-step membrane record is taken in pieces of bounded size
+        piece = max(1, (1 << 26) // max(1, sim.ne))
+        for k in range(step0 + piece, step0 + n_steps, piece):
+            bounds.add(k)
     bounds = sorted(bounds)
     want_record = bool(_S.rec_links)
     senders, times = [], []
+    mm_rows = {m: ([], [], []) for m, _ in _S.mm_links}
     for a, b in zip(bounds[:-1], bounds[1:]):
         if _S.cur_links:
             sim.i_ext = torch.as_tensor(_current_at(a), device=sim.dev)
         cap = int(min(max(4096, (b - a) * sim.ne), 1 << 26)) if want_record else 0
-        out = sim.run(b - a, spike_bits=False, record_cap=cap)
+        out = sim.run(b - a, spike_bits=False, record_cap=cap, save_state=bool(_S.mm_links))
+        for m, ids in _S.mm_links:
+            # NEST samples at the end of a step: row k of the record is the potential at time (a + k + 1) * dt
+            p = _S.params[m - 1]
+            every = int(round(float(p["interval"]) / dt))
+            stamps = np.arange(a + 1, b + 1)
+            keep = (stamps % every == 0) & (stamps * dt > float(p["start"]) + 1e-9) & \
+                   (stamps * dt <= float(p["stop"]) + 1e-9)
+            if keep.any():
+                cols = torch.as_tensor(s["n_of"][ids], device=sim.dev)
+                rows = torch.as_tensor(np.flatnonzero(keep), device=sim.dev)
+                v = out["saved"]["v"].view(b - a, sim.ne)[rows][:, cols].cpu().numpy().astype(np.float64)
+                v += s["e_l"][s["n_of"][ids]][None, :]
+                mm_rows[m][0].append(np.tile(ids, int(keep.sum())))
+                mm_rows[m][1].append(np.repeat(stamps[keep] * dt, ids.size))
+                mm_rows[m][2].append(v.reshape(-1))
         if want_record:
             rec = out["record"]
             sim.check()
@@ -437,6 +494,12 @@ def Simulate(t_ms):
             senders.append(s["neuron_ids"][el[order]])
     s["steps_done"] = step0 + n_steps
     _S.status["biological_time"] = s["steps_done"] * dt
+    for m, (a_s, a_t, a_v) in mm_rows.items():
+        if a_s:
+            new = (np.concatenate(a_s), np.concatenate(a_t), np.concatenate(a_v))
+            old = _S.mm_events.get(m, (np.zeros(0, np.int64), np.zeros(0), np.zeros(0)))
+            _S.mm_events[m] = tuple(np.concatenate([o, n_]) for o, n_ in zip(old, new))
+            _write_ascii(m, new[0], new[1], new[2])
     if want_record:
         all_s, all_t = np.concatenate(senders), np.concatenate(times)
         for ids, r in _S.rec_links:
@@ -446,22 +509,27 @@ def Simulate(t_ms):
             _write_ascii(r, all_s[keep], all_t[keep])
 
 
-def _write_ascii(recorder, senders, times):
+def _write_ascii(recorder, senders, times, values=None):
     """NEST 3 ``record_to: 'ascii'`` file, the form bmtk reads back
     (bmtk/simulator/pointnet/modules/record_spikes.py:76-82): '#' comment
     lines, a tab-separated header ``sender time_ms``, one row per spike."""
     p = _S.params[recorder - 1]
     if p.get("record_to") != "ascii" and not p.get("to_file", False):
         return
-    label = p.get("label") or "spike_recorder"
+    label = p.get("label") or _S.kind[recorder - 1]
     path = os.path.join(_S.status.get("data_path", "") or "", "{}-{}-0.dat".format(label, recorder))
     new = not os.path.exists(path) or (_S.status.get("overwrite_files") and recorder not in _written)
     _written.add(recorder)
     with open(path, "w" if new else "a") as f:
         if new:
-            f.write("# NEST version: {}\n# RecordingBackendASCII version: 2\nsender\ttime_ms\n".format(__version__))
-        for sdr, t in zip(senders, times):
-            f.write("{}\t{:.3f}\n".format(int(sdr), t))
+            f.write("# NEST version: {}\n# RecordingBackendASCII version: 2\nsender\ttime_ms{}\n".format(
+                __version__, "" if values is None else "\tV_m"))
+        if values is None:
+            for sdr, t in zip(senders, times):
+                f.write("{}\t{:.3f}\n".format(int(sdr), t))
+        else:
+            for sdr, t, v in zip(senders, times, values):
+                f.write("{}\t{:.3f}\t{:.6f}\n".format(int(sdr), t, v))
 
 
 _written = set()

@@ -265,8 +265,8 @@ class Glif3Simulator:
         s = self._struct(bits, record)
         saved = None
         if save_state:
-            if self.res_span or self.delay_offset:
-                raise ValueError("save_state needs a simulator built with resident=False and delay_offset 0")
+            if self.res_span:
+                raise ValueError("save_state needs a simulator built with resident=False")
             saved = dict(v=torch.empty(n_steps, self.ne, device=self.dev),
                          flags=torch.empty(n_steps, self.ne, dtype=torch.uint8, device=self.dev), step0=self.step)
             s.save_v, s.save_flags = _p(saved["v"]), _p(saved["flags"])

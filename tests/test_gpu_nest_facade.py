@@ -173,3 +173,61 @@ def test_small_network_through_the_front_end_matches_the_oracle(golden_dir, tmp_
     df = pd.read_csv(dat[0], index_col=False, sep='\t', comment='#')
     assert list(df.columns) == ['sender', 'time_ms'] and len(df) == want["count"]
     np.testing.assert_allclose(np.sort(df['time_ms'].values), np.sort(want_t), atol=dt * 2e-2 + 1e-3)
+
+
+def test_multimeter_records_membrane_potential(golden_dir, tmp_path):
+    """What bmtk's membrane report asks of NEST (bmtk/simulator/pointnet/modules/multimeter_reporter.py:36-46,
+    113-115): a multimeter on V_m with an interval, a start and a stop, written as an ascii file with the columns
+    sender, time_ms, V_m.  The trace must follow the fp64 oracle stepped one step at a time: the sample stamped t is
+    the potential at the end of the step that ends at t."""
+    import pandas as pd
+    from oracle import glif3_oracle as orc
+    from bmtk_amd.glif_utils import params_table
+    from bmtk_amd.spike_trains import bin_spike_times
+    from bmtk_amd.layout import PAR
+    cells = [json.load(open(os.path.join(golden_dir, "cell_models", f)))
+             for f in ("318808427_glif_lif_asc_psc.json", "478958894_glif_lif_asc_psc.json")]
+    dt, T = 0.1, 40.0
+    nest.ResetKernel()
+    nest.SetKernelStatus({"resolution": dt, "data_path": str(tmp_path), "overwrite_files": True})
+    a = nest.Create('glif_psc', 1, cells[0])
+    b = nest.Create('glif_psc', 1, cells[1])
+    gen = nest.Create('spike_generator', 1, {'spike_times': [3.0, 5.0, 6.0, 7.5, 9.0, 11.0, 12.0, 20.0]})
+    nest.Connect(gen, a + b, syn_spec={'weight': 400.0, 'delay': 1.0, 'receptor_type': 1})
+    mm = nest.Create('multimeter', params={'start': 2.0, 'stop': 30.0, 'record_to': 'ascii', 'record_from': ['V_m'],
+                                           'label': 'membrane'})
+    nest.SetStatus(mm, 'interval', 0.5)
+    nest.Connect(mm, a + b)
+    with pytest.raises(nest.kernel.NESTErrors.BadProperty):
+        nest.Create('multimeter', params={'record_from': ['I_syn']})
+    with pytest.raises(nest.kernel.NESTErrors.BadProperty):
+        nest.SetStatus(mm, 'interval', 0.25)
+    nest.Simulate(T / 2)
+    nest.Simulate(T / 2)
+    ev = nest.GetStatus(mm, 'events')[0]
+    times = np.arange(2.5, 30.0 + 1e-9, 0.5)
+    assert ev['times'].size == 2 * times.size
+    np.testing.assert_allclose(ev['times'][0::2], times, atol=1e-9)
+    assert list(ev['senders'][:2]) == a.tolist() + b.tolist()
+    # the oracle, one step at a time
+    par, asc_init, u_init = params_table(cells)
+    prop = orc.precompute(par, dt)
+    steps = int(round(T / dt))
+    d = int(round(1.0 / dt))
+    inp = (np.array([0, 2], np.int32), np.array([0, 1], np.int32), np.array([400.0, 400.0], np.float32),
+           np.array([d, d], np.uint8), np.zeros(2, np.uint8))
+    in_ptr, in_ev = bin_spike_times([np.array([3.0, 5.0, 6.0, 7.5, 9.0, 11.0, 12.0, 20.0])], dt, steps)
+    st = orc.new_state(2, 1, np.float64, asc_init=asc_init, u_init=u_init)
+    ring = np.zeros((d + 1, 4, 2))
+    trace = np.zeros((steps, 2))
+    for k in range(steps):
+        orc.simulate(st, prop, dt, 1, ring=ring, inp=inp, in_ptr=in_ptr, in_events=in_ev, step0=k)
+        trace[k] = st["V"] + par[PAR["E_L"]]
+    rows = np.rint(times / dt).astype(int) - 1
+    want = trace[rows]
+    got = ev['V_m'].reshape(-1, 2)
+    assert np.abs(want).max() > 50 and np.ptp(want[:, 0]) > 5.0  # the cell is depolarised and fires in the window
+    np.testing.assert_allclose(got, want, atol=2e-3)
+    df = pd.read_csv(os.path.join(str(tmp_path), "membrane-{}-0.dat".format(mm.tolist()[0])), sep='\t', comment='#')
+    assert list(df.columns) == ['sender', 'time_ms', 'V_m'] and len(df) == 2 * times.size
+    np.testing.assert_allclose(df['V_m'].to_numpy(), ev['V_m'], atol=1e-6)
