@@ -23,6 +23,7 @@ returns a numpy array, `.attrs` a dict, groups iterate over member names.
 """
 from __future__ import annotations
 
+import mmap
 import struct
 import zlib
 
@@ -81,7 +82,7 @@ def _parse_datatype(buf, off):
         q = p + used
         names = []
         for _ in range(n):
-            end = buf.index(b"\0", q)
+            end = buf.find(b"\0", q)
             names.append(bytes(buf[q:end]))
             q += ((end - q) // 8 + 1) * 8 if (cls_ver >> 4) < 3 else end - q + 1
         q += n * base.size
@@ -92,7 +93,7 @@ def _parse_datatype(buf, off):
         q = p
         fields = []
         for _ in range(n):
-            end = buf.index(b"\0", q)
+            end = buf.find(b"\0", q)
             name = bytes(buf[q:end]).decode()
             if version < 3:
                 q += ((end - q) // 8 + 1) * 8
@@ -215,7 +216,7 @@ def _decode(f, dt, shape, raw):
         if shape == ():
             return vals[0]
         return np.array(vals, dtype=object).reshape(shape)
-    arr = np.frombuffer(raw, dtype=dt.dtype, count=count).reshape(shape)
+    arr = np.frombuffer(raw, dtype=dt.dtype, count=count).reshape(shape).copy()  # detach from the mapping
     if dt.is_bool:
         arr = arr.astype(bool)
     if dt.dtype.kind == "S" and shape == ():
@@ -286,7 +287,7 @@ class Dataset(_Node):
             addr = _u(buf, d + 2, 8)
             if addr == UNDEF:
                 return bytes(nbytes)
-            return bytes(buf[addr:addr + nbytes])
+            return memoryview(buf)[addr:addr + nbytes]  # no copy: the file is memory-mapped
         if cls == 2:
             rank = buf[d + 2]
             btree = _u(buf, d + 3, 8)
@@ -394,7 +395,7 @@ class Group(_Node):
                     for i in range(n):
                         e = addr + 8 + 40 * i
                         noff, oaddr = _u(buf, e, 8), _u(buf, e + 8, 8)
-                        end = buf.index(b"\0", hdata + noff)
+                        end = buf.find(b"\0", hdata + noff)
                         links[bytes(buf[hdata + noff:end]).decode()] = oaddr
                     return
                 if buf[addr:addr + 4] != b"TREE" or buf[addr + 4] != 0:
@@ -464,14 +465,19 @@ class Group(_Node):
 
 
 class File(Group):
-    """Read-only view of an HDF5 file held in memory (SONATA files are read whole by the reference too)."""
+    """Read-only view of a memory-mapped HDF5 file: a data set is read from disk when it is asked for, so a
+    multi-gigabyte edge file costs the memory of the arrays taken from it and no more."""
 
     def __init__(self, path, mode="r"):
         if mode != "r":
             raise H5Error("File() reads; use h5lite.write() to create a file")
-        with open(path, "rb") as fh:
-            self.buf = fh.read()
         self.path = str(path)
+        self._fh = open(path, "rb")
+        try:
+            self.buf = mmap.mmap(self._fh.fileno(), 0, access=mmap.ACCESS_READ)
+        except ValueError:
+            self._fh.close()
+            raise H5Error(f"{path}: not an HDF5 file")
         buf = self.buf
         base = 0
         while buf[base:base + 8] != SIGNATURE:
@@ -521,7 +527,11 @@ class File(Group):
         return self._gheaps[addr][index]
 
     def close(self):
-        pass
+        try:
+            self.buf.close()
+        except (BufferError, ValueError):
+            pass  # a view is still alive; the mapping goes with it
+        self._fh.close()
 
     def __enter__(self):
         return self

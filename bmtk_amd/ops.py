@@ -165,6 +165,32 @@ class SynapseTable:
         return cls(*t, n_rows=indptr.size - 1, max_row=int(deg.max()) if deg.size else 0)
 
     @classmethod
+    def from_edges(cls, src, tgt, w, d, r, n_rows, n_cols, device=None):
+        """Edge list (host arrays or device tensors) -> source-major table, rows ordered by (row, column,
+        original position), built on the device: what ``bmtk_amd.network.coo_to_csr`` does on the host, without
+        its sort of tens of millions of keys on one CPU core."""
+        dev = device or _dev()
+        src = torch.as_tensor(np.ascontiguousarray(src) if not torch.is_tensor(src) else src, device=dev).long()
+        tgt = torch.as_tensor(np.ascontiguousarray(tgt) if not torch.is_tensor(tgt) else tgt, device=dev).long()
+        if src.numel() and (int(src.min()) < 0 or int(src.max()) >= n_rows or int(tgt.min()) < 0
+                            or int(tgt.max()) >= n_cols):
+            raise ValueError("edge endpoints outside 0..{} / 0..{}".format(n_rows - 1, n_cols - 1))
+        order = torch.sort(src * n_cols + tgt, stable=True).indices
+        counts = torch.bincount(src, minlength=n_rows)
+        indptr = torch.zeros(n_rows + 1, dtype=torch.int32, device=dev)
+        indptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+
+        def col(a, dtype):
+            a = torch.as_tensor(np.ascontiguousarray(a) if not torch.is_tensor(a) else a, device=dev)
+            return a.to(dtype)[order].contiguous()
+
+        d = torch.as_tensor(np.ascontiguousarray(d) if not torch.is_tensor(d) else d, device=dev)
+        wide = bool(d.numel()) and int(d.max()) > 255
+        return cls(indptr, tgt[order].to(torch.int32).contiguous(), col(w, torch.float32),
+                   d.to(torch.int32 if wide else torch.uint8)[order].contiguous(), col(r, torch.uint8),
+                   n_rows=n_rows, max_row=int(counts.max().item()) if counts.numel() else 0)
+
+    @classmethod
     def from_device(cls, csr, n_rows, n_cols, ring_slots):
         """Adopt device tensors after the same checks ``network.check_csr`` makes on the host."""
         indptr, indices, w, d, r = (t.contiguous() for t in csr)

@@ -19,7 +19,6 @@ asks (bmtk/simulator/pointnet/modules/record_spikes.py:53-104).
 import os
 
 import numpy as np
-import pandas as pd
 import torch
 
 from . import sonata
@@ -140,7 +139,7 @@ class PointSimulator:
 
     def run(self, record_cap=None):
         nw = self.net
-        rec, inp = nw.tables()
+        rec, inp = nw.device_tables(self._device)
         sim = Glif3Simulator(nw.n, nw.par, self.dt, class_id=nw.class_id, rec=rec, inp=inp,
                              asc_init=nw.asc_init[:, nw.class_id], u_init=nw.u_init[nw.class_id],
                              i_ext=np.zeros(nw.n, np.float32), device=self._device, resident=self._resident)

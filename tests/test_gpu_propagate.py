@@ -172,3 +172,20 @@ def test_pull_matches_oracle(batch, p):
         assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-2 * m + 1e-30)) < 1e-5
         assert np.all(got[m == 0] == 0)
     assert np.abs(want).max() > 0
+
+
+def test_table_from_edges_on_the_device_equals_the_host_build():
+    from bmtk_amd import network as net
+    rng = np.random.default_rng(5)
+    n_rows, n_cols, nnz = 300, 450, 20000
+    src, tgt = rng.integers(0, n_rows, nnz), rng.integers(0, n_cols, nnz)
+    w = rng.normal(size=nnz).astype(np.float32)
+    r = rng.integers(0, 4, nnz).astype(np.uint8)
+    for d in (rng.integers(1, 6, nnz), rng.integers(100, 1000, nnz)):
+        want = net.coo_to_csr(src, tgt, w, d, r, n_rows, "source")
+        got = ops.SynapseTable.from_edges(src, tgt, w, d, r, n_rows, n_cols)
+        for a, b in zip(want, (got.indptr, got.indices, got.weights, got.delays, got.receptors)):
+            np.testing.assert_array_equal(a, b.cpu().numpy())
+            assert a.dtype == b.cpu().numpy().dtype
+    with pytest.raises(ValueError):
+        ops.SynapseTable.from_edges(src, tgt + n_cols, w, d, r, n_rows, n_cols)
