@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import glif3_oracle as orc
-from bmtk_amd import synthetic
+from bmtk_amd import network as net, synthetic
 from bmtk_amd.glif_utils import convert_aibs2nest, params_table
 from bmtk_amd.simulator import Glif3Simulator
 from gpu_util import rel_err
@@ -279,3 +279,43 @@ def test_pull_form_of_the_per_step_driver(batch):
     auto = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
                           resident=False)
     assert (auto.pull_table is not None) == (batch >= 8)
+
+
+def test_resident_pull_with_more_fired_rows_than_its_list_holds():
+    """20,000 identical neurons driven by the same current fire in the same steps: 20,000 fired rows in one step
+    exceed the 8192 entries of the resident kernel's LDS list, so its workgroups fall back to pulling what each
+    thread found itself.  Raster and state must still equal the fp32 oracle bit for bit."""
+    n, steps = 20000, 60
+    rng = np.random.default_rng(21)
+    par = synthetic.random_cells(rng, 1)
+    class_id = np.zeros(n, np.int32)
+    nnz = 10 * n
+    src, tgt = rng.integers(0, n, nnz), rng.integers(0, n, nnz)
+    w = (rng.integers(1, 20, nnz) * 0.25).astype(np.float32)
+    rec = net.coo_to_csr(src, tgt, w, rng.integers(1, 4, nnz), rng.integers(0, 4, nnz).astype(np.uint8), n, "source")
+    i_ext = np.full(n, 900.0, np.float32)
+    # and 5000 input sources that all fire in steps 5, 6 and 30: several passes of 1024 events per workgroup
+    n_in = 5000
+    isrc, itgt = np.repeat(np.arange(n_in), 4), rng.integers(0, n, 4 * n_in)
+    inp = net.coo_to_csr(isrc, itgt, (rng.integers(1, 40, 4 * n_in) * 0.25).astype(np.float32),
+                         rng.integers(1, 4, 4 * n_in), np.zeros(4 * n_in, np.uint8), n_in, "source")
+    in_ptr = np.zeros(steps + 1, np.int64)
+    for k in (5, 6, 30):
+        in_ptr[k + 1:] += n_in
+    in_events = np.tile(np.arange(n_in, dtype=np.int32), 3)
+    prop = orc.precompute(par, 1.0)
+    st = orc.new_state(n, 1, np.float32)
+    ring = np.zeros((4, 4, n), np.float32)
+    orc.set_threads(1)
+    want = orc.simulate(st, prop, 1.0, steps, class_id=class_id, ring=ring, rec=rec, inp=inp, in_ptr=in_ptr,
+                        in_events=in_events, i_ext=i_ext, raster=True)
+    per_step = want["raster"].sum(1)
+    assert per_step.max() > 8192  # the case this test is about
+    sim = Glif3Simulator(n, par, 1.0, class_id=class_id, rec=rec, inp=inp, i_ext=i_ext, resident=True)
+    sim.set_input_events(in_ptr, in_events)
+    out = sim.run(steps)
+    sim.check()
+    np.testing.assert_array_equal(sim.raster(out["bits"]).cpu().numpy(), want["raster"])
+    got = sim.state.to_numpy()
+    for k in ("V", "asc", "y1", "y2", "ref"):
+        np.testing.assert_array_equal(got[k], st[k], err_msg=k)
