@@ -25,7 +25,7 @@ class Glif3Sim(C.Structure):
         ("inp_indptr", c_void_p), ("inp_indices", c_void_p), ("inp_weights", c_void_p),
         ("inp_delays", c_void_p), ("inp_receptors", c_void_p), ("inp_packed", c_void_p), ("i_ext", c_void_p),
         ("work_bits", c_void_p), ("delay_offset", c_int32), ("hist_slots", c_int32),
-        ("delay_bits", c_int32), ("_pad2", c_int32),
+        ("delay_bits", c_int32), ("res_spin_limit", C.c_uint32),
         ("res_span", c_int32), ("res_groups", c_int32), ("rec_seg", c_void_p), ("inp_seg", c_void_p),
         ("res_sync", c_void_p),
         ("pull_indptr", c_void_p), ("pull_packed", c_void_p), ("pull_syn", c_void_p), ("pull_work", c_void_p),
@@ -53,7 +53,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 4  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 5  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {

@@ -348,7 +348,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
                     ok = 0;
                     break;
                 }
-                if (++spins > kMaxSpin) {
+                if (++spins > (s.res_spin_limit ? s.res_spin_limit : kMaxSpin)) {
                     __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     ok = 0;
                     break;

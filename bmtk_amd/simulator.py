@@ -125,6 +125,7 @@ class Glif3Simulator:
         self.res_span = self.res_groups = 0
         self.rec_seg = self.inp_seg = None
         self._pending_check = False
+        self.spin_limit = 0  # resident mode: polls of the grid barrier before giving up (0 = built-in limit)
         if resident:
             self._setup_resident(required=(resident is True))
         self.pull_table = self.pull_syn = self.pull_work = None
@@ -238,6 +239,7 @@ class Glif3Simulator:
                 s.in_hist, s.in_hist_stride = _p(self.in_hist), self.in_hist_stride
         if self.res_span:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
+            s.res_spin_limit = int(self.spin_limit)
             s.rec_seg, s.inp_seg = _p(self.rec_seg), _p(self.inp_seg)
         if bits is not None:
             s.spike_bits, s.spike_bits_stride = _p(bits), bits.shape[1]

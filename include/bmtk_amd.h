@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 4
+#define BMTK_AMD_ABI_VERSION 5
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -196,7 +196,8 @@ typedef struct bmtk_glif3_sim {
     int32_t delay_bits;          /* width of the delay field of rec_packed / inp_packed: 0 or 6 = the standard
                                   * packing; 7..14 = bmtk_csr_pack_wide tables (launch-per-step mode without the
                                   * pull form only), ring_slots may then reach 2^delay_bits */
-    int32_t _pad2;
+    uint32_t res_spin_limit;     /* resident mode: polls of the grid barrier before a workgroup gives up and raises
+                                  * the abort word (0 = the built-in limit, a few seconds) */
     /* Resident mode (optional, batch 1 only; res_span == 0 disables it): the
      * network is split into res_groups = ceil(ne/res_span) workgroups that keep
      * their elements' state in registers and their slice of the ring in LDS for

@@ -319,3 +319,22 @@ def test_resident_pull_with_more_fired_rows_than_its_list_holds():
     got = sim.state.to_numpy()
     for k in ("V", "asc", "y1", "y2", "ref"):
         np.testing.assert_array_equal(got[k], st[k], err_msg=k)
+
+
+def test_resident_barrier_gives_up_cleanly():
+    """Failure handling of the grid barrier, forced from the host: with a spin limit of one poll some workgroup
+    finds the barrier unfinished, raises the abort word, every workgroup leaves its loop and the kernel ends
+    normally; check() then reports the run as invalid.  A following run with the normal limit works."""
+    cfg = synthetic.small_glif3_network(n=3000, n_in=500, steps=300, seed=8, in_w_scale=3.0, in_fanout=300,
+                                        p_conn=0.03, w_scale=1.5)
+    sim = _gpu_sim(cfg, resident=True)
+    assert sim.res_groups > 8
+    sim.spin_limit = 1
+    sim.run(300)
+    with pytest.raises(RuntimeError, match="barrier"):
+        sim.check()
+    want, _, _ = _oracle_run(cfg, np.float64)
+    sim = _gpu_sim(cfg, resident=True)
+    out = sim.run(300)
+    sim.check()
+    assert (sim.raster(out["bits"]).cpu().numpy() == want["raster"][:300]).mean() >= 0.999
