@@ -14,7 +14,10 @@ bmtk/simulator/pointnet/pointsimulator.py:229-262; spike-time rules of
 pointnetwork.py:39-61) and ``current_clamp``, run ``tstop/dt`` steps
 (pointsimulator.py:149-173) and write ``output.spikes_file`` /
 ``spikes_file_csv`` in ``output.output_dir`` sorted as ``spikes_sort_order``
-asks (bmtk/simulator/pointnet/modules/record_spikes.py:53-104).
+asks (bmtk/simulator/pointnet/modules/record_spikes.py:53-104).  ``reports``
+entries of module ``multimeter_report`` / ``membrane_report`` for ``V_m``
+become SONATA cell-variable files
+(bmtk/simulator/pointnet/modules/multimeter_reporter.py:64-140).
 """
 import os
 
@@ -75,6 +78,7 @@ class PointSimulator:
         self._clamps = []
         self._device, self._resident = device, resident
         self.spikes = None
+        self.reports = {}  # name -> dict(node_ids, interval, tstart, tstop, file)
 
     @classmethod
     def from_config(cls, config, network, dt=None, device=None, resident="auto"):
@@ -89,7 +93,36 @@ class PointSimulator:
                 sim.add_current_clamp(entry)
             else:
                 raise NotImplementedError("input {!r}: input_type {!r} is not supported".format(name, kind))
+        for name, entry in config.get("reports", {}).items():
+            sim.add_report(name, entry)
         return sim
+
+    def add_report(self, name, entry):
+        """A membrane potential report: ``cells`` (a node id list, or {"population":…, "node_id": […]}; absent or
+        "all" = every node), ``variable_name`` V_m, optional ``file_name``, ``tstart``, ``tstop``, ``dt``
+        (sampling interval, a multiple of the resolution)."""
+        module = entry.get("module", "multimeter_report")
+        if module not in ("multimeter_report", "membrane_report"):
+            raise NotImplementedError("report {!r}: module {!r} is not supported".format(name, module))
+        var = entry.get("variable_name", "V_m")
+        var = var[0] if isinstance(var, (list, tuple)) and len(var) == 1 else var
+        if var != "V_m":
+            raise NotImplementedError("report {!r}: only V_m is recorded, not {!r}".format(name, var))
+        cells = entry.get("cells", "all")
+        if isinstance(cells, dict):
+            if cells.get("population", self.net.population) != self.net.population:
+                raise ValueError("report {!r}: population {!r} is not simulated".format(name, cells["population"]))
+            cells = cells.get("node_id", cells.get("node_ids", "all"))
+        ids = np.arange(self.net.n) if isinstance(cells, str) else np.asarray(cells, np.int64)
+        if ids.size and (ids.min() < 0 or ids.max() >= self.net.n):
+            raise ValueError("report {!r}: node id outside 0..{}".format(name, self.net.n - 1))
+        interval = float(entry.get("dt") or self.dt)
+        every = interval / self.dt
+        if every < 1 - 1e-9 or abs(every - round(every)) > 1e-6:
+            raise ValueError("report {!r}: the sampling interval must be a multiple of the resolution".format(name))
+        self.reports[name] = dict(node_ids=ids, every=int(round(every)), tstart=float(entry.get("tstart") or 0.0),
+                                  tstop=float(entry.get("tstop") or self.tstop),
+                                  file=entry.get("file_name") or name + ".h5", rows=[])
 
     def add_spike_inputs(self, spikes, node_set=None):
         """Spike trains of virtual populations; a train is only used by the population it is stored under, and
@@ -142,15 +175,33 @@ class PointSimulator:
         rec, inp = nw.device_tables(self._device)
         sim = Glif3Simulator(nw.n, nw.par, self.dt, class_id=nw.class_id, rec=rec, inp=inp,
                              asc_init=nw.asc_init[:, nw.class_id], u_init=nw.u_init[nw.class_id],
-                             i_ext=np.zeros(nw.n, np.float32), device=self._device, resident=self._resident)
+                             i_ext=np.zeros(nw.n, np.float32), device=self._device,
+                             **(dict(resident=False, pull=False) if self.reports else dict(resident=self._resident)))
         if inp is not None:
             sim.set_input_events(*bin_spike_times(self._trains, self.dt, self.n_steps))
         steps, elems, fracs = [], [], []
+        from .layout import PAR
+        e_l = nw.par[PAR["E_L"]][nw.class_id]
+        pieces = []
         for a, b, cur in self._segments():
+            # a membrane record is taken in pieces of bounded size
+            piece = max(1, (1 << 26) // nw.n) if self.reports else b - a
+            pieces += [(k, min(k + piece, b), cur) for k in range(a, b, piece)]
+        for a, b, cur in pieces:
             sim.i_ext.copy_(torch.as_tensor(cur, device=sim.dev))
             cap = record_cap or max(1 << 16, (b - a) * nw.n // 8)
-            out = sim.run(b - a, spike_bits=False, record_cap=cap)
+            out = sim.run(b - a, spike_bits=False, record_cap=cap, save_state=bool(self.reports))
             sim.check()
+            for rep in self.reports.values():
+                # the sample stamped t is the potential at the end of the step that ends at t
+                stamps = np.arange(a + 1, b + 1)
+                keep = (stamps % rep["every"] == 0) & (stamps * self.dt > rep["tstart"] + 1e-9) & \
+                       (stamps * self.dt <= rep["tstop"] + 1e-9)
+                if keep.any():
+                    rows = torch.as_tensor(np.flatnonzero(keep), device=sim.dev)
+                    cols = torch.as_tensor(rep["node_ids"], device=sim.dev)
+                    v = out["saved"]["v"].view(b - a, nw.n)[rows][:, cols].cpu().numpy().astype(np.float64)
+                    rep["rows"].append((stamps[keep] * self.dt, v + e_l[rep["node_ids"]][None, :]))
             r = out["record"]
             c = int(r["count"].item())
             if c > cap:
@@ -168,9 +219,18 @@ class PointSimulator:
 
     def _write_outputs(self):
         out = self.output
+        base = out.get("output_dir", ".")
+        for rep in self.reports.values():
+            if rep["rows"]:
+                times = np.concatenate([r[0] for r in rep["rows"]])
+                data = np.concatenate([r[1] for r in rep["rows"]])
+                interval = rep["every"] * self.dt
+                path = rep["file"] if os.path.isabs(rep["file"]) else os.path.join(base, rep["file"])
+                sonata.write_membrane_report(path, self.net.population, rep["node_ids"], data, float(times[0]),
+                                             float(times[-1]) + interval, interval)
+                rep["times"], rep["data"], rep["rows"] = times, data, []
         if not out:
             return
-        base = out.get("output_dir", ".")
         order = out.get("spikes_sort_order", "none")
         if out.get("spikes_file"):
             path = out["spikes_file"] if os.path.isabs(out["spikes_file"]) else os.path.join(base, out["spikes_file"])

@@ -425,6 +425,42 @@ def read_spikes(path, populations=None):
     return out
 
 
+def write_membrane_report(path, population, node_ids, data, tstart, tstop, dt, variable="V_m", units="mV"):
+    """A SONATA cell-variable report with one element per node, the layout bmtk's ``CompartmentReport`` writes for
+    PointNet membrane reports (bmtk/utils/reports/compartment/compartment_writer.py:175-227,456-516):
+    ``/report/<population>/data`` float64 [steps][nodes] with attributes ``variable`` and ``units``, and
+    ``/report/<population>/mapping/{node_ids, element_ids, element_pos, index_pointer, time}`` with
+    ``time = [tstart, tstop, dt]``, steps = (tstop - tstart) / dt."""
+    node_ids = np.asarray(node_ids, np.uint64)
+    data = np.asarray(data, np.float64)
+    if data.ndim != 2 or data.shape[1] != node_ids.size:
+        raise ValueError("data must be [steps, nodes]")
+    n = node_ids.size
+    tree = {"report": {population: {
+        "data": (data, {"variable": variable, "units": units}),
+        "mapping": {"node_ids": node_ids, "element_ids": np.zeros(n, np.uint64), "element_pos": np.zeros(n, np.float64),
+                    "index_pointer": np.arange(n + 1, dtype=np.uint64),
+                    "time": np.array([tstart, tstop, dt], np.float64)}}}}
+    os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+    h5lite.write(path, tree, attrs={"magic": np.uint32(MAGIC_VAL), "version": np.array(VERSION, np.uint32)})
+
+
+def read_membrane_report(path, population=None):
+    """-> (node_ids int64 [nodes], times float64 [steps] (the end of each sampled step), data float64 [steps][nodes],
+    attributes of the data set)."""
+    with h5lite.File(path) as h5:
+        root = h5["/report"]
+        pop = population or root.keys()[0]
+        g = root[pop]
+        data = np.asarray(g["data"][()], np.float64)
+        t0, t1, dt = (float(x) for x in g["mapping/time"][()])
+        ptr = np.asarray(g["mapping/index_pointer"][()], np.int64)
+        if not np.array_equal(np.diff(ptr), np.ones(ptr.size - 1, np.int64)):
+            raise NotImplementedError("reports with several elements per node are not supported")
+        return (np.asarray(g["mapping/node_ids"][()], np.int64), t0 + dt * np.arange(data.shape[0]), data,
+                dict(g["data"].attrs))
+
+
 def write_spikes_csv(path, spikes, sort_order="none"):
     """Space-separated ``timestamps population node_ids`` with a header line (spikes_file_writers.py:115-126)."""
     frames = []

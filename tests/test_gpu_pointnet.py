@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 
 from oracle import glif3_oracle as orc
-from bmtk_amd import ops, pointnet, sonata
+from bmtk_amd import h5lite, ops, pointnet, sonata
 from bmtk_amd.spike_trains import bin_spike_times
 
 pytestmark = pytest.mark.gpu
@@ -157,3 +157,43 @@ def test_example_at_its_own_resolution(tmp_path):
     assert want["count"] > 1000
     got = _pairs(np.floor(ts / dt + 1e-9).astype(int), ids)
     assert got == _pairs(want["step"], want["elem"])
+
+
+def test_membrane_report(tmp_path):
+    """A ``reports`` entry as in examples/point_120cells/config.simulation.json: V_m of five cells, here every
+    0.5 ms.  The file has bmtk's cell-variable layout and its trace follows the fp64 oracle stepped one step at a
+    time, while the trajectories have not separated (first 60 ms)."""
+    dt, tstop = 0.1, 100.0
+    cfg_path = _write_configs(str(tmp_path), dt, tstop)
+    conf = pointnet.Config.from_json(cfg_path)
+    cells = [0, 85, 170, 250, 299]
+    conf["reports"] = {"membrane_potential": {"cells": {"population": "v1", "node_id": cells}, "variable_name": "V_m",
+                                              "module": "multimeter_report", "sections": "soma", "dt": 0.5}}
+    graph = pointnet.PointNetwork.from_config(conf, unsupported="silence")
+    sim = pointnet.PointSimulator.from_config(conf, graph)
+    sim.run()
+    ids, times, data, attrs = sonata.read_membrane_report(str(tmp_path / "output" / "membrane_potential.h5"))
+    assert list(ids) == cells and attrs == {"variable": "V_m", "units": "mV"}
+    np.testing.assert_allclose(times, np.arange(0.5, tstop + 1e-9, 0.5), atol=1e-9)
+    assert data.shape == (times.size, len(cells))
+    with h5lite.File(str(tmp_path / "output" / "membrane_potential.h5")) as f:
+        assert list(f["/report/v1/mapping/time"][()]) == [0.5, tstop + 0.5, 0.5]
+        assert list(f["/report/v1/mapping/index_pointer"][()]) == [0, 1, 2, 3, 4, 5]
+    # the oracle, stepped
+    from bmtk_amd.layout import PAR
+    rec, inp = graph.tables()
+    prop = orc.precompute(graph.par, dt)
+    st = orc.new_state(graph.n, 1, np.float64, asc_init=graph.asc_init[:, graph.class_id],
+                       u_init=graph.u_init[graph.class_id])
+    ring = np.zeros((21, 4, graph.n))
+    n_early = 600
+    in_ptr, in_ev = bin_spike_times(sim._trains, dt, n_early)
+    e_l = graph.par[PAR["E_L"]][graph.class_id]
+    want = np.zeros((n_early // 5, len(cells)))
+    for k in range(n_early):
+        orc.simulate(st, prop, dt, 1, class_id=graph.class_id, ring=ring, rec=rec, inp=inp, in_ptr=in_ptr,
+                     in_events=in_ev, step0=k)
+        if (k + 1) % 5 == 0:
+            want[(k + 1) // 5 - 1] = (st["V"] + e_l)[cells]
+    assert np.ptp(want) > 10.0
+    np.testing.assert_allclose(data[:n_early // 5], want, atol=5e-3)
