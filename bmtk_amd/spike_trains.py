@@ -94,6 +94,29 @@ class PoissonSpikeGenerator(object):
                            "population": rows_p, "node_ids": np.concatenate(rows_n) if rows_n else []})
         return df if with_population_col else df.drop(columns="population")
 
+    def _as_spikes(self):
+        out = {}
+        for p in self.populations:
+            ids = self.node_ids(p)
+            ts = [self.get_times(n, p) for n in ids]
+            out[p] = (np.concatenate([np.full(t.size, n, np.int64) for n, t in zip(ids, ts)]) if ids
+                      else np.zeros(0, np.int64), np.concatenate(ts) if ts else np.zeros(0))
+        return out
+
+    def to_sonata(self, path, mode="w", sort_order="none", **kwargs):
+        """``/spikes/<population>/{node_ids,timestamps}`` as bmtk/utils/reports/spike_trains/spike_trains_api.py:147-158
+        writes them; the file is stored uncompressed whatever ``compression`` asks."""
+        from . import sonata
+        sonata.write_spikes(path, self._as_spikes(), sort_order=getattr(sort_order, "value", sort_order),
+                            units=self.units, mode=mode)
+
+    def to_csv(self, path, mode="w", sort_order="none", **kwargs):
+        """Space-separated ``timestamps population node_ids`` (spike_trains_api.py:160-169)."""
+        from . import sonata
+        if mode != "w":
+            raise NotImplementedError("to_csv only writes a new file")
+        sonata.write_spikes_csv(path, self._as_spikes(), sort_order=getattr(sort_order, "value", sort_order))
+
     # -- generators --------------------------------------------------------
     def add(self, node_ids, firing_rate, population=None, times=(0.0, 1.0), abs_ref=0, tau_ref=0):
         """``firing_rate`` in Hz (scalar, or an array paired with ``times``), ``times`` in seconds."""
@@ -101,6 +124,11 @@ class PoissonSpikeGenerator(object):
             raise ValueError("Refractory period time constant (sec) cannot be negative.")
         if abs_ref < 0:
             raise ValueError("Absolute refractory period (sec) cannot be negative.")
+        if isinstance(node_ids, str):
+            # a nodes file: the ids of ``population`` in it (bmtk/utils/sonata/utils.py:111-115)
+            from . import h5lite
+            with h5lite.File(node_ids) as h5:
+                node_ids = np.asarray(h5["/nodes/{}/node_id".format(population)][()], np.int64)
         if np.isscalar(node_ids):
             node_ids = [node_ids]
         if np.isscalar(firing_rate):

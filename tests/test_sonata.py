@@ -271,3 +271,24 @@ def test_spike_comparisons():
     other_pop = {"lgn": a["v1"]}
     assert not sonata.spikes_equal(a, other_pop) and not sonata.spikes_is_subset(a, other_pop)
     assert sonata.spikes_is_subset({"v1": (np.zeros(0, int), np.zeros(0))}, a)
+
+
+def test_poisson_generator_files(tmp_path):
+    """The calls of examples/point_450glifs/create_inputs.py: ids from a nodes file, trains to SONATA and csv."""
+    from bmtk_amd.spike_trains import PoissonSpikeGenerator
+    nodes = os.path.join(NETDIR, "lgn_nodes.h5")
+    psg = PoissonSpikeGenerator(population="lgn", seed=7)
+    psg.add(node_ids=nodes, firing_rate=15.0, times=(0.0, 0.5), population="lgn")
+    with h5lite.File(nodes) as h5:
+        want_ids = np.asarray(h5["/nodes/lgn/node_id"][()])
+    assert psg.node_ids("lgn") == sorted(want_ids.tolist()) or set(psg.node_ids("lgn")) <= set(want_ids.tolist())
+    h5p, csvp = str(tmp_path / "in.h5"), str(tmp_path / "in.csv")
+    psg.to_sonata(h5p, sort_order="by_id")
+    psg.to_csv(csvp)
+    ids, ts, attrs = sonata.read_spikes(h5p)["lgn"]
+    assert attrs["sorting"] == "by_id" and np.all(np.diff(ids) >= 0)
+    assert ids.size == psg.n_spikes("lgn") and ts.min() >= 0 and ts.max() <= 500.0
+    for n in (int(ids[0]), int(ids[-1])):
+        assert np.array_equal(np.sort(ts[ids == n]), np.sort(psg.get_times(n, "lgn")))
+    cid, cts = sonata.read_spikes_csv(csvp)["lgn"][:2]
+    assert sonata.spikes_equal({"lgn": (ids, ts)}, {"lgn": (cid, cts)})
