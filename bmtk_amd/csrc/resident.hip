@@ -51,7 +51,7 @@ constexpr int kMaxSlack = 31;
 #ifdef BMTK_RES_PROFILE
 __device__ unsigned long long g_prof[8];
 #define PROF_T(var) const long long var = wall_clock64()
-#define PROF_ADD(i, a, b) if (threadIdx.x == 0 && blockIdx.x == 0) g_prof[i] += (unsigned long long)((b) - (a))
+#define PROF_ADD(i, a, b) if (threadIdx.x == 0 && blockIdx.x == 0) atomicAdd(&g_prof[i], (unsigned long long)((b) - (a)))
 #else
 #define PROF_T(var)
 #define PROF_ADD(i, a, b)
@@ -257,9 +257,15 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     const int B = r.offset;
     auto in_bound = [&](int64_t i) -> int64_t { return (s.in_ptr && i > 0) ? s.in_ptr[i] : 0; };
     int64_t ka = 0, kb = in_bound(r.step0 - B);
+#ifdef BMTK_RES_PROFILE
+    long long prof_prev = 0, prof_c1 = 0;
+#endif
     for (int64_t k = 0; k < r.n_steps; ++k) {
         const int64_t t = r.step0 + k;
         PROF_T(c0);
+#ifdef BMTK_RES_PROFILE
+        if (k > 0) PROF_ADD(1, prof_prev, c0);
+#endif
         const int64_t kn = in_bound(t + 1 - B);
         // 1. fold the arrivals of slot t-1 and update
         bool spike = false;
@@ -315,8 +321,14 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
                 __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
             PROF_ADD(0, c0, c1);
+#ifdef BMTK_RES_PROFILE
+            prof_c1 = c1;
+#endif
         }
         PROF_T(c2);
+#ifdef BMTK_RES_PROFILE
+        if (!kLate) PROF_ADD(7, prof_c1, c2);
+#endif
         // 3. pull the spikes and input events of step t-1-B while the barrier fills (the first step of a
         //    call pulls nothing: the call before it closed with that pull)
         if (k > 0 && t - 1 - B >= 0 && mine > 0)
@@ -364,6 +376,9 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         PROF_T(c4);
         PROF_ADD(2, c2, c3);
         PROF_ADD(3, c3, c4);
+#ifdef BMTK_RES_PROFILE
+        prof_prev = c4;
+#endif
         if (!go_on) {
             aborted = true;
             break;
