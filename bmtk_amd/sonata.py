@@ -381,9 +381,15 @@ def write_spikes(path, spikes, sort_order="none", units="ms", mode="w"):
         raise ValueError("mode must be 'w' or 'a'")
     tree = {}
     if mode == "a" and os.path.exists(path):
+        # the file is rewritten with what it held; population groups without data are kept too
+        with h5lite.File(path) as h5:
+            held = [k for k in h5["/spikes"].keys() if isinstance(h5["/spikes"][k], h5lite.Group)] \
+                if "/spikes" in h5 else []
+        tree = {pop: {} for pop in held}
         for pop, (ids, ts, attrs) in read_spikes(path).items():
-            tree[pop] = {"__attrs__": {k: v for k, v in attrs.items() if k == "sorting"},
-                         "timestamps": (ts, {"units": attrs.get("units", "ms")}), "node_ids": ids}
+            if pop in tree:
+                tree[pop] = {"__attrs__": {k: v for k, v in attrs.items() if k == "sorting" and v != "unknown"},
+                             "timestamps": (ts, {"units": "ms"}), "node_ids": np.asarray(ids, np.uint64)}
     for pop, (ids, ts) in spikes.items():
         if pop in tree:
             raise ValueError("sonata file {} already contains a spikes group {}, skiping(use option mode=\"w\" to "

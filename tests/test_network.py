@@ -48,3 +48,22 @@ def test_check_csr_rejects_what_a_kernel_would_trip_over():
         net.check_csr((indptr, indices, w[:1], d, r), 2, 2, 3)
     with pytest.raises(ValueError):
         net.coo_to_csr([5], [0], [1.0], [1], [0], n_rows=2, major="source")
+
+
+@pytest.mark.parametrize("dt", [0.001, 1.0, 5.0, 10.0])
+def test_multimeter_at_any_resolution(dt, tmp_path):
+    """bmtk/tests/simulator/pointnet/test_multimeter_report.py:10-28: the calls MultimeterMod.initialize makes
+    (bmtk/simulator/pointnet/modules/multimeter_reporter.py:103-115) go through at small and large steps."""
+    from bmtk_amd import nest
+    nest.ResetKernel()
+    nest.SetKernelStatus({"resolution": dt, "overwrite_files": True, "print_time": False})
+    cells = nest.Create("glif_psc", 4, {})
+    mm = nest.Create("multimeter", params={"start": 0.0, "stop": 100.0, "record_to": "ascii",
+                                            "record_from": ["V_m"], "label": str(tmp_path / "__bmtk_nest_test")})
+    nest.SetStatus(mm, "interval", dt)
+    nest.Connect(mm, cells)
+    assert nest.GetStatus(mm, "interval")[0] == dt
+    assert nest.GetKernelStatus("min_delay") == dt
+    with pytest.raises(nest.kernel.NESTError):
+        nest.SetStatus(mm, "interval", dt * 0.5)  # not a multiple of the resolution
+    nest.ResetKernel()

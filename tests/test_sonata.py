@@ -292,3 +292,79 @@ def test_poisson_generator_files(tmp_path):
         assert np.array_equal(np.sort(ts[ids == n]), np.sort(psg.get_times(n, "lgn")))
     cid, cts = sonata.read_spikes_csv(csvp)["lgn"][:2]
     assert sonata.spikes_equal({"lgn": (ids, ts)}, {"lgn": (cid, cts)})
+
+
+def _magic():
+    return {"magic": np.uint32(sonata.MAGIC_VAL), "version": np.array(sonata.VERSION, np.uint32)}
+
+
+def test_write_no_spikes(tmp_path):
+    """A run without a single spike still writes a valid file with an empty /spikes group
+    (bmtk/tests/utils/reports/spike_trains/test_sonata_adaptor.py:103-116)."""
+    path = str(tmp_path / "none.h5")
+    sonata.write_spikes(path, {})
+    with h5lite.File(path) as h5:
+        assert int(h5.attrs["magic"]) == sonata.MAGIC_VAL and len(h5.attrs["version"]) == 2
+        assert "/spikes" in h5 and len(h5["/spikes"].keys()) == 0
+    assert sonata.read_spikes(path) == {}
+    # a population that never fired
+    sonata.write_spikes(path, {"V1": (np.zeros(0, np.int64), np.zeros(0))}, sort_order="by_time")
+    ids, ts, attrs = sonata.read_spikes(path)["V1"]
+    assert ids.size == 0 and ts.size == 0 and attrs["sorting"] == "by_time"
+
+
+def test_append_keeps_other_populations_and_refuses_an_existing_one(tmp_path):
+    """test_sonata_adaptor.py:125-157: mode 'a' adds /spikes/V2 beside an existing (here empty) /spikes/V1 and
+    raises ValueError when /spikes/V2 is already there."""
+    path = str(tmp_path / "a.h5")
+    h5lite.write(path, {"spikes": {"V1": {}}}, attrs=_magic())
+    new = {"V2": (np.zeros(100, np.int64), np.linspace(0, 1.0, 100))}
+    sonata.write_spikes(path, new, mode="a", sort_order="by_id")
+    with h5lite.File(path) as h5:
+        assert "/spikes/V1" in h5 and "/spikes/V2" in h5
+        assert h5["/spikes/V2/node_ids"].shape == (100,) and h5["/spikes/V2/timestamps"].shape == (100,)
+    path2 = str(tmp_path / "b.h5")
+    h5lite.write(path2, {"spikes": {"V2": {}}}, attrs=_magic())
+    with pytest.raises(ValueError):
+        sonata.write_spikes(path2, new, mode="a", sort_order="by_id")
+    # appending to a file that holds data keeps that data
+    sonata.write_spikes(path, {"V3": (np.array([4, 2]), np.array([1.5, 0.5]))}, mode="a", sort_order="by_time")
+    got = sonata.read_spikes(path)
+    assert set(got) == {"V2", "V3"} and got["V2"][0].size == 100
+    np.testing.assert_array_equal(got["V3"][0], [2, 4])
+
+
+def test_older_spike_file_layout_and_mixed_file(tmp_path):
+    """test_sonata_adaptor.py:242-262 and :268-300: /spikes/gids + /spikes/timestamps without a population group
+    is read under the placeholder population; empty population groups are skipped."""
+    ids = np.array([0, 0, 0, 0, 2, 1, 2], np.uint64)
+    ts = np.array([0.25, 0.5, 0.75, 1.0, 3.0, 0.001, 2.0])
+    old = str(tmp_path / "old.h5")
+    h5lite.write(old, {"spikes": {"gids": ids, "timestamps": ts}}, attrs=_magic())
+    got = sonata.read_spikes(old)
+    assert list(got) == ["<sonata:none>"]
+    g_ids, g_ts, _ = got["<sonata:none>"]
+    assert g_ids.size == 7 and set(g_ids.tolist()) == {0, 1, 2}
+    np.testing.assert_allclose(np.sort(g_ts[g_ids == 0]), [0.25, 0.5, 0.75, 1.0])
+    new = str(tmp_path / "new.h5")
+    h5lite.write(new, {"spikes": {"V1": {"node_ids": ids, "timestamps": ts},
+                                  "V2": {"node_ids": np.array([10, 10, 10], np.uint64),
+                                         "timestamps": np.array([4.0, 4.0, 4.0])},
+                                  "V3": {}}}, attrs=_magic())
+    got = sonata.read_spikes(new)
+    assert set(got) == {"V1", "V2"} and got["V2"][0].tolist() == [10, 10, 10]
+    assert sonata.read_spikes(new, populations=["V2"]).keys() == {"V2"}
+    with pytest.raises(ValueError):
+        bad = str(tmp_path / "bad.h5")
+        h5lite.write(bad, {"other": {}}, attrs=_magic())
+        sonata.read_spikes(bad)
+
+
+def test_csv_without_population_column(tmp_path):
+    """bmtk/tests/utils/reports/spike_trains/test_csv_adaptor.py:135-160."""
+    path = str(tmp_path / "s.csv")
+    with open(path, "w") as fh:
+        fh.write("timestamps node_ids\n0.25 0\n0.5 0\n3.0 2\n0.001 1\n")
+    got = sonata.read_spikes_csv(path)
+    assert list(got) == ["<sonata:none>"]
+    assert got["<sonata:none>"][0].tolist() == [0, 0, 2, 1]
