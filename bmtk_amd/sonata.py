@@ -19,6 +19,7 @@ HDF5 access goes through bmtk_amd.h5lite (h5py is not required).
 """
 import json
 import os
+import re
 
 import numpy as np
 import pandas as pd
@@ -62,12 +63,20 @@ def load_config(path):
     base = os.path.dirname(path)
     manifest = {"$configdir": base, "$workingdir": os.getcwd()}
     raw = dict(cfg.get("manifest", {}))
-    for _ in range(len(raw) + 1):
-        for k, v in raw.items():
-            v = _substitute(v, dict(sorted(manifest.items(), key=lambda kv: -len(kv[0]))))
-            if v == "." or v.startswith("./"):
-                v = os.path.normpath(os.path.join(base, v))
-            manifest[k] = v
+    # a variable is taken into the manifest once nothing in it is left to expand; one that names an unknown
+    # variable, or two that name each other, never get there (sonata_config.py:258-330 raises for both)
+    pending = dict(raw)
+    while pending:
+        known = dict(sorted(manifest.items(), key=lambda kv: -len(kv[0])))
+        done = {}
+        for k, v in pending.items():
+            v = _substitute(v, known)
+            if not re.search(r"\$\{?[A-Za-z_]\w*\}?", v):
+                done[k] = os.path.normpath(os.path.join(base, v)) if v == "." or v.startswith("./") else v
+        if not done:
+            raise ValueError("{}: manifest variables {} cannot be resolved".format(path, sorted(pending)))
+        manifest.update(done)
+        pending = {k: v for k, v in pending.items() if k not in done}
     cfg = _substitute(cfg, dict(sorted(manifest.items(), key=lambda kv: -len(kv[0]))))
     for key in ("network", "simulation"):
         if isinstance(cfg.get(key), str):

@@ -368,3 +368,25 @@ def test_csv_without_population_column(tmp_path):
     got = sonata.read_spikes_csv(path)
     assert list(got) == ["<sonata:none>"]
     assert got["<sonata:none>"][0].tolist() == [0, 0, 2, 1]
+
+
+def _config(tmp_path, d):
+    path = str(tmp_path / "cfg.json")
+    with open(path, "w") as fh:
+        json.dump(d, fh)
+    return sonata.load_config(path)
+
+
+def test_manifest_rules(tmp_path):
+    """bmtk/tests/utils/sonata/test_config.py:156-198: variables may build on each other in both spellings; an
+    unknown variable or a circular definition raises."""
+    cfg = _config(tmp_path, {"manifest": {"$BASE_DIR": "/base", "$TMP_DIR": "$BASE_DIR/tmp",
+                                          "$SHARE_DIR": "${TMP_DIR}_1/share"}, "x": "$SHARE_DIR/y"})
+    assert cfg["x"] == "/base/tmp_1/share/y"
+    cfg = _config(tmp_path, {"manifest": {"$DIR_DATA": "data", "$DIR_MAT": "mat",
+                                          "$APPS": "/${DIR_DATA}/$DIR_MAT/apps"}, "x": "$APPS"})
+    assert cfg["x"] == "/data/mat/apps"
+    with pytest.raises(ValueError):
+        _config(tmp_path, {"manifest": {"$BASE": "/base", "$TMP": "$VAR/Smat"}})
+    with pytest.raises(ValueError):
+        _config(tmp_path, {"manifest": {"$BASE": "$TMP/share", "$TMP": "$BASE/share"}})
