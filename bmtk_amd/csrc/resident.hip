@@ -50,11 +50,14 @@ constexpr int kMaxSlack = 31;
 
 #ifdef BMTK_RES_PROFILE
 __device__ unsigned long long g_prof[8];
+__device__ unsigned long long g_prof_blk[256][4];  // per workgroup: update, pull, wait, segment pull
+#define PROF_BLK(i, a, b) if (threadIdx.x == 0) atomicAdd(&g_prof_blk[blockIdx.x & 255][i], (unsigned long long)((b) - (a)))
 #define PROF_T(var) const long long var = wall_clock64()
 #define PROF_ADD(i, a, b) if (threadIdx.x == 0 && blockIdx.x == 0) atomicAdd(&g_prof[i], (unsigned long long)((b) - (a)))
 #else
 #define PROF_T(var)
 #define PROF_ADD(i, a, b)
+#define PROF_BLK(i, a, b)
 #endif
 
 struct Resident {
@@ -110,23 +113,24 @@ constexpr int kActCap = 8192;   // active-row list in LDS (entries)
 constexpr int kScanWords = 4;   // ballot words per thread and round
 constexpr unsigned kInputTag = 0x80000000u;
 
-// Spikes and input events of step `tp`, handed over as if emitted in step
-// `ts` (= tp + delay offset) -> this workgroup's ring slice.
+// Spikes and input events of one step, read from row `hist_row` of the ballot
+// history and handed over as if emitted in the step whose ring slot is `slot0`
+// (the step they were emitted in plus the delay offset) -> this workgroup's
+// ring slice.
 // Pass by pass: every thread reads kScanWords ballot words and one input
 // event (independent loads), a workgroup-wide prefix sum packs the rows that
 // fired into one LDS list, then one thread per listed row pulls this
 // workgroup's segment of it.  Must be called by all threads of the workgroup.
-__device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int64_t tp, int64_t ts,
+__device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int hist_row, int slot0,
                                           float *ring_l, unsigned *act, unsigned *scan_l, int e0, int64_t words,
                                           int64_t k0, int64_t k1)
 {
     const int tid = threadIdx.x;
     const int L = s.ring_slots;
-    const int slot0 = (int)(ts % L);
     const int wave = tid / kWave;
     const bool has_rec = s.rec_seg != nullptr;
     const unsigned long long *bits =
-        reinterpret_cast<const unsigned long long *>(s.work_bits) + (tp % r.hist) * (words + 1);
+        reinterpret_cast<const unsigned long long *>(s.work_bits) + (int64_t)hist_row * (words + 1);
     const int64_t n_words = has_rec ? words : 0;
     const int64_t word_rounds = (n_words + (int64_t)kScanWords * kResBlock - 1) / ((int64_t)kScanWords * kResBlock);
     const int64_t event_rounds = (k1 - k0 + kResBlock - 1) / kResBlock;
@@ -204,6 +208,7 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
         PROF_ADD(4, p0, p1);
         PROF_ADD(5, p1, p2);
         PROF_ADD(6, p2, p3);
+        PROF_BLK(3, p2, p3);
     }
 }
 
@@ -260,8 +265,17 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
 #ifdef BMTK_RES_PROFILE
     long long prof_prev = 0, prof_c1 = 0;
 #endif
+    // ring slot of step t-1 and history rows of steps t and t-1-B, counted along instead of taking three
+    // 64-bit remainders per step (every instruction of the loop costs all 16 wavefronts an issue slot)
+    auto wrap = [](int64_t a, int m) { return (int)(((a % m) + m) % m); };
+    int next_slot_prev = wrap(r.step0 - 1, L), next_row_t = wrap(r.step0, r.hist),
+        next_row_p = wrap(r.step0 - 1 - B, r.hist);
     for (int64_t k = 0; k < r.n_steps; ++k) {
         const int64_t t = r.step0 + k;
+        const int slot_prev = next_slot_prev, row_t = next_row_t, row_p = next_row_p;
+        next_slot_prev = slot_prev + 1 == L ? 0 : slot_prev + 1;
+        next_row_t = row_t + 1 == r.hist ? 0 : row_t + 1;
+        next_row_p = row_p + 1 == r.hist ? 0 : row_p + 1;
         PROF_T(c0);
 #ifdef BMTK_RES_PROFILE
         if (k > 0) PROF_ADD(1, prof_prev, c0);
@@ -272,7 +286,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         float frac = 0.0f;
         if (own) {
             if (k > 0) {
-                float *prev = ring_l + (int)((t - 1) % L) * GLIF3_NREC * span + tid;
+                float *prev = ring_l + slot_prev * GLIF3_NREC * span + tid;
 #pragma unroll
                 for (int q = 0; q < GLIF3_NREC; ++q) {
                     const float a = prev[q * span];
@@ -285,7 +299,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         const unsigned long long m = __ballot(spike);
         // only the wavefronts that cover this workgroup's span own a ballot word
         if (lane == 0 && tid < span && (e & ~(int64_t)(kWave - 1)) < ne) {
-            __hip_atomic_store(reinterpret_cast<unsigned long long *>(s.work_bits) + (t % r.hist) * (words + 1) + (e >> 6),
+            __hip_atomic_store(reinterpret_cast<unsigned long long *>(s.work_bits) + (int64_t)row_t * (words + 1) + (e >> 6),
                                m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (s.spike_bits) s.spike_bits[k * s.spike_bits_stride + (e >> 6)] = m;
         }
@@ -321,6 +335,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
                 __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
             PROF_ADD(0, c0, c1);
+            PROF_BLK(0, c0, c1);
 #ifdef BMTK_RES_PROFILE
             prof_c1 = c1;
 #endif
@@ -332,7 +347,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         // 3. pull the spikes and input events of step t-1-B while the barrier fills (the first step of a
         //    call pulls nothing: the call before it closed with that pull)
         if (k > 0 && t - 1 - B >= 0 && mine > 0)
-            pull_step(s, r, g, t - 1 - B, t - 1, ring_l, act, scan_l, e0, words, ka, kb);
+            pull_step(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb);
         ka = kb;
         kb = kn;
         if (late) {
@@ -376,6 +391,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         PROF_T(c4);
         PROF_ADD(2, c2, c3);
         PROF_ADD(3, c3, c4);
+        PROF_BLK(1, c2, c3);
+        PROF_BLK(2, c3, c4);
 #ifdef BMTK_RES_PROFILE
         prof_prev = c4;
 #endif
@@ -388,7 +405,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     if (!aborted && done > 0) {
         // closing: spikes and inputs of the last step (less the delay offset), then fold the last slot
         const int64_t tl = r.step0 + done - 1;
-        if (tl - B >= 0 && mine > 0) pull_step(s, r, g, tl - B, tl, ring_l, act, scan_l, e0, words, ka, kb);
+        if (tl - B >= 0 && mine > 0)
+            pull_step(s, r, g, wrap(tl - B, r.hist), wrap(tl, L), ring_l, act, scan_l, e0, words, ka, kb);
         __syncthreads();
         if (own) {
             float *prev = ring_l + (int)(tl % L) * GLIF3_NREC * span + tid;
@@ -501,6 +519,10 @@ using namespace bmtk;
 extern "C" void bmtk_debug_read_prof(unsigned long long *out)
 {
     (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_prof), sizeof(g_prof));
+}
+extern "C" void bmtk_debug_read_prof_blocks(unsigned long long *out)
+{
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_prof_blk), sizeof(g_prof_blk));
 }
 #endif
 
