@@ -53,7 +53,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 5  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 6  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -83,6 +83,9 @@ SIGNATURES = {
     "bmtk_glif3_simulate_bwd": (c_int32, [C.POINTER(Glif3Bwd), c_int64, c_int64, c_void_p]),
     "bmtk_spike_counts": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
 }
+
+
+RES_SYNC_WORDS = 65 * 1088  # BMTK_RES_SYNC_WORDS
 
 
 class LibraryMissing(RuntimeError):

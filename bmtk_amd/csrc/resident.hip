@@ -16,9 +16,16 @@
 // Nothing but spike ballots, segment offsets and the synapses actually used
 // crosses the memory system: no global atomics, no state traffic.
 //
-// Ballots are triple-buffered: buffer t%3 is written in step t, read in step
-// t+1 and next overwritten in step t+3, which a workgroup can only reach after
-// the barrier of step t+2, i.e. after every workgroup finished reading it.
+// Ballots live in a history of D rows, row t%D for step t.  With D = 3 a
+// workgroup waits for the barrier of step t at the end of step t: row t%3 is
+// read in step t+1 and next overwritten in step t+3, which a workgroup can only
+// reach after the barrier of step t+2, i.e. after every workgroup finished
+// reading it.  With a fourth row the wait moves to where the barrier is needed,
+// just before the pull in step t+1: the update of step t+1 needs no spike newer
+// than step t-1 (delays are at least one step, and arrivals enter y1 a step
+// late), so it runs while the barrier of step t fills, and the wait is
+// normally over before it begins.  A workgroup writing row t%4 is then at most
+// two steps ahead of one still reading row (t-3)%4.
 //
 // With a delay offset B (tables hold delays shortened by B steps) step t pulls
 // the spikes of step t-1-B from a history of D rows, and a workgroup only has
@@ -46,6 +53,12 @@ namespace bmtk {
 constexpr int kResBlock = 1024;
 constexpr unsigned kMaxSpin = 4000000u;  // polls of the barrier word before giving up (seconds)
 constexpr int kBarrierWords = 64;        // per-step arrival counters, used round-robin
+// Words between two counters.  The arrivals of one step are a burst of one atomic per workgroup on one address,
+// which the memory side works off one after the other (a few microseconds for 248 of them); a look at the
+// counter of the step before must not queue up behind that burst, so every counter lives in a memory channel
+// of its own rather than side by side in one cache line.
+constexpr int kBarrierStride = BMTK_RES_SYNC_STRIDE;
+static_assert(BMTK_RES_SYNC_WORDS >= (1 + kBarrierWords) * kBarrierStride, "res_sync too small");
 constexpr int kMaxSlack = 31;
 
 #ifdef BMTK_RES_PROFILE
@@ -237,7 +250,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     const int64_t e = e0 + tid;
     unsigned *act = reinterpret_cast<unsigned *>(ring_l + s.ring_slots * GLIF3_NREC * r.span);
     unsigned *abort_word = s.res_sync + 1;
-    unsigned *arrivals = s.res_sync + 2;  // [kBarrierWords]
+    unsigned *arrivals = s.res_sync + kBarrierStride;  // [kBarrierWords] counters, kBarrierStride words apart
 
     for (int c = tid; c < L * GLIF3_NREC * span; c += kResBlock) {
         const int dr = c / span, i = c - dr * span;
@@ -265,6 +278,40 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
 #ifdef BMTK_RES_PROFILE
     long long prof_prev = 0, prof_c1 = 0;
 #endif
+    // Wait until every workgroup has arrived at the barrier of step j of this call (all threads call it;
+    // false = the run was given up).  No acquire fence: it would invalidate this XCD's L2 every step, and
+    // the only data other workgroups write during the run are the ballots, which are read with agent-scope
+    // loads that bypass the non-coherent caches.
+    auto counter_of = [&](int64_t j) { return arrivals + ((j < 0 ? 0 : j) & (kBarrierWords - 1)) * kBarrierStride; };
+    auto wait_for = [&](int64_t j) -> bool {
+        if (tid == 0) {
+            const unsigned *word = counter_of(j);
+            const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
+            unsigned spins = 0;
+            int ok = 1;
+            while (load_agent(word) < target) {
+                if (load_agent(abort_word) != 0u) {
+                    ok = 0;
+                    break;
+                }
+                if (++spins > (s.res_spin_limit ? s.res_spin_limit : kMaxSpin)) {
+                    __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ok = 0;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            go_on = ok;
+        }
+        __syncthreads();
+        return go_on != 0;
+    };
+    // Without slack, the pull of step t-1-B (in step t) is all that needs the barrier of step t-1, and the
+    // update of step t needs neither: when the history has a row to spare (D >= B + 4) the wait for the barrier
+    // of step t-1 moves from the end of step t-1 to just before that pull.  By then every workgroup arrived an
+    // update and a pull ago, so the wait is over before it begins.  A workgroup writing row t%D may then be up
+    // to two steps ahead of one still reading row (t-3-B)%D, hence the spare row.
+    const bool defer = !kLate && r.hist >= B + 4;
     // ring slot of step t-1 and history rows of steps t and t-1-B, counted along instead of taking three
     // 64-bit remainders per step (every instruction of the loop costs all 16 wavefronts an issue slot)
     auto wrap = [](int64_t a, int m) { return (int)(((a % m) + m) % m); };
@@ -332,13 +379,17 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
             PROF_T(c1);
             // 2. arrive at the barrier of step t (ballots of this workgroup are out)
             if (tid == 0)
-                __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
+                __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)) * kBarrierStride, 1u, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
             PROF_ADD(0, c0, c1);
             PROF_BLK(0, c0, c1);
 #ifdef BMTK_RES_PROFILE
             prof_c1 = c1;
 #endif
+            if (defer && k > 0 && !wait_for(k - 1)) {
+                aborted = true;
+                break;
+            }
         }
         PROF_T(c2);
 #ifdef BMTK_RES_PROFILE
@@ -358,36 +409,16 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         //  writes below was last read before the barrier that precedes the arrival)
         PROF_T(c3);
         if (late && tid == 0)
-            __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)), 1u, __ATOMIC_RELAXED,
+            __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)) * kBarrierStride, 1u, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
         // 4. every `check` steps (each step without slack) wait until every workgroup has published
         //    step k - S + (check - 1): enough for the steps up to the next look
         if (late && k % check != check - 1 && k + 1 < r.n_steps) continue;
-        if (tid == 0) {
+        bool ok = true;
+        if (!defer) {
             int64_t j = late ? k - r.slack + (check - 1) : k;  // step of this call everybody must have published
-            j = j < k ? j : k;
-            const unsigned *word = arrivals + ((j < 0 ? 0 : j) & (kBarrierWords - 1));
-            const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
-            unsigned spins = 0;
-            int ok = 1;
-            while (load_agent(word) < target) {
-                if (load_agent(abort_word) != 0u) {
-                    ok = 0;
-                    break;
-                }
-                if (++spins > (s.res_spin_limit ? s.res_spin_limit : kMaxSpin)) {
-                    __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    ok = 0;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(2);
-            }
-            // No acquire fence here: it would invalidate this XCD's L2 every step.  The only
-            // data other workgroups write during the run are the ballots, which are read with
-            // agent-scope loads that bypass the non-coherent caches.
-            go_on = ok;
+            ok = wait_for(j < k ? j : k);
         }
-        __syncthreads();
         PROF_T(c4);
         PROF_ADD(2, c2, c3);
         PROF_ADD(3, c3, c4);
@@ -396,11 +427,13 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
 #ifdef BMTK_RES_PROFILE
         prof_prev = c4;
 #endif
-        if (!go_on) {
+        if (!ok) {
             aborted = true;
             break;
         }
     }
+    // with the deferred wait the closing pull is the first to need the barrier of the last step
+    if (defer && !aborted && done > 0 && !wait_for(done - 1)) aborted = true;
 
     if (!aborted && done > 0) {
         // closing: spikes and inputs of the last step (less the delay offset), then fold the last slot
@@ -429,6 +462,13 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
 __global__ void zero_words_kernel(unsigned *w, int n)
 {
     if ((int)threadIdx.x < n) w[threadIdx.x] = 0u;
+}
+
+// abort flag and arrival counters of a resident run
+__global__ void zero_sync_kernel(unsigned *sync)
+{
+    if (threadIdx.x < 2) sync[threadIdx.x] = 0u;
+    if ((int)threadIdx.x < kBarrierWords) sync[(1 + (int)threadIdx.x) * kBarrierStride] = 0u;
 }
 
 __global__ __launch_bounds__(kBlock) void segment_offsets_kernel(int64_t n_rows, const int32_t *__restrict__ indptr,
@@ -489,7 +529,7 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
                   n_cu, per_cu);
         return BMTK_E_LAUNCH;
     }
-    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(128), 0, stream, s.res_sync, 2 + kBarrierWords);
+    hipLaunchKernelGGL(zero_sync_kernel, dim3(1), dim3(128), 0, stream, s.res_sync);
     bmtk_glif3_sim s_copy = s;
     // BMTK_AMD_PLAIN_LAUNCH=1 uses an ordinary launch (co-residency then rests on the occupancy check
     // above and an otherwise idle device); for tools that cannot follow cooperative launches.

@@ -114,14 +114,15 @@ class Glif3Simulator:
         self.in_steps = 0
         self.step = 0
         self.words = n_words(self.ne)
-        # history of spike bits: 2B+3 rows let resident workgroups drift B steps apart, B+3 is the least
-        self.hist_slots = 2 * self.delay_offset + 3
+        # history of spike bits: 2B+3 rows let resident workgroups drift B steps apart, one more lets them look
+        # at the grid barrier only where the spikes behind it are needed; B+3 is the least
+        self.hist_slots = 2 * self.delay_offset + 4
         if self.hist_slots * (self.words + 1) * 8 > 2 ** 30:
             self.hist_slots = self.delay_offset + 3
         self.work_bits = torch.zeros(self.hist_slots * (self.words + 1), dtype=torch.int64, device=self.dev)
         if self.n >= 2 ** 24:
             raise ValueError("the packed synapse tables index at most 2^24 neurons")
-        self.res_sync = torch.zeros(80, dtype=torch.int32, device=self.dev)
+        self.res_sync = torch.zeros(_lib.RES_SYNC_WORDS, dtype=torch.int32, device=self.dev)
         self.res_span = self.res_groups = 0
         self.rec_seg = self.inp_seg = None
         self._pending_check = False

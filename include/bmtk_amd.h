@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 5
+#define BMTK_AMD_ABI_VERSION 6
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -155,6 +155,9 @@ int bmtk_csr_pack_wide(int64_t nnz, const int32_t *indices, const float *weights
 int bmtk_csr_segment_offsets(int64_t n_rows, const int32_t *indptr, const int32_t *indices, int32_t span,
                              int32_t n_groups, uint32_t *seg, int32_t *unsorted, void *stream);
 
+#define BMTK_RES_SYNC_STRIDE 1088                          /* words: 4 KiB + 256 B */
+#define BMTK_RES_SYNC_WORDS (65 * BMTK_RES_SYNC_STRIDE)    /* size of bmtk_glif3_sim.res_sync */
+
 /* Everything nest.Simulate needs for a forward run (bmtk/simulator/pointnet/pointsimulator.py:159-166). */
 typedef struct bmtk_glif3_sim {
     int64_t n_neurons;
@@ -192,7 +195,10 @@ typedef struct bmtk_glif3_sim {
      * delays.  In resident mode workgroups may then run up to min(B, hist_slots - 3 - B) steps apart before
      * one waits for another (at most 31) (what NEST's min_delay communication interval does between ranks). */
     int32_t delay_offset;        /* B >= 0 */
-    int32_t hist_slots;          /* rows of work_bits, at least delay_offset + 3; 0 stands for 3 */
+    int32_t hist_slots;          /* rows of work_bits, at least delay_offset + 3; 0 stands for 3.  One row more
+                                  * lets the resident mode, also with delay_offset 0, look at its grid barrier
+                                  * only when the spikes behind it are needed (after the next update) instead of
+                                  * stopping at it every step. */
     int32_t delay_bits;          /* width of the delay field of rec_packed / inp_packed: 0 or 6 = the standard
                                   * packing; 7..14 = bmtk_csr_pack_wide tables (launch-per-step mode without the
                                   * pull form only), ring_slots may then reach 2^delay_bits */
@@ -208,8 +214,9 @@ typedef struct bmtk_glif3_sim {
     int32_t res_groups;
     const uint32_t *rec_seg;     /* [neurons][res_groups+1] */
     const uint32_t *inp_seg;     /* [inputs][res_groups+1] */
-    uint32_t *res_sync;          /* 80 words of scratch: abort flag, per-step arrival counters; zeroed by the call.
-                                  * After the run, word 1 != 0 means the grid barrier timed out and the
+    uint32_t *res_sync;          /* BMTK_RES_SYNC_WORDS words of scratch: word 1 = abort flag, from word
+                                  * BMTK_RES_SYNC_STRIDE on 64 per-step arrival counters that many words apart; the call zeroes what it
+                                  * uses.  After the run, word 1 != 0 means the grid barrier timed out and the
                                   * results are invalid. */
     /* Pull form of the recurrent delivery for batched runs (optional; launch-per-step mode with delay_offset 0
      * and hist_slots == ring_slots): a TARGET-major packed copy of the recurrent table.  The recurrent arrivals

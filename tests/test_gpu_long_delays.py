@@ -57,7 +57,7 @@ def test_long_delays_equal_the_oracle_with_true_delays(extra, resident):
     sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
                          inp=cfg["inp_src"], resident=resident)
     assert sim.delay_offset == extra and sim.L == 5 and bool(sim.res_span) == resident
-    assert sim.hist_slots == 2 * extra + 3
+    assert sim.hist_slots == 2 * extra + 4
     sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
     a = sim.run(400)
     b = sim.run(600)

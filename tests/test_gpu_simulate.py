@@ -330,6 +330,7 @@ def test_resident_barrier_gives_up_cleanly():
     sim = _gpu_sim(cfg, resident=True)
     assert sim.res_groups > 8
     sim.spin_limit = 1
+    sim.hist_slots = 3  # no spare history row: the wait closes every step, when the barrier has only begun to fill
     sim.run(300)
     with pytest.raises(RuntimeError, match="barrier"):
         sim.check()
