@@ -283,26 +283,22 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     // the only data other workgroups write during the run are the ballots, which are read with agent-scope
     // loads that bypass the non-coherent caches.
     auto counter_of = [&](int64_t j) { return arrivals + ((j < 0 ? 0 : j) & (kBarrierWords - 1)) * kBarrierStride; };
-    auto wait_for = [&](int64_t j) -> bool {
-        if (tid == 0) {
-            const unsigned *word = counter_of(j);
-            const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
-            unsigned spins = 0;
-            int ok = 1;
-            while (load_agent(word) < target) {
-                if (load_agent(abort_word) != 0u) {
-                    ok = 0;
-                    break;
-                }
-                if (++spins > (s.res_spin_limit ? s.res_spin_limit : kMaxSpin)) {
-                    __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    ok = 0;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(2);
+    auto poll = [&](int64_t j) -> int {  // one thread: 1 = everybody arrived at step j, 0 = given up
+        const unsigned *word = counter_of(j);
+        const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
+        unsigned spins = 0;
+        while (load_agent(word) < target) {
+            if (load_agent(abort_word) != 0u) return 0;
+            if (++spins > (s.res_spin_limit ? s.res_spin_limit : kMaxSpin)) {
+                __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return 0;
             }
-            go_on = ok;
+            __builtin_amdgcn_s_sleep(2);
         }
+        return 1;
+    };
+    auto wait_for = [&](int64_t j) -> bool {
+        if (tid == 0) go_on = poll(j);
         __syncthreads();
         return go_on != 0;
     };
@@ -312,6 +308,10 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     // update and a pull ago, so the wait is over before it begins.  A workgroup writing row t%D may then be up
     // to two steps ahead of one still reading row (t-3-B)%D, hence the spare row.
     const bool defer = !kLate && r.hist >= B + 4;
+    // The look itself is taken by the last wavefront, while the others update: its 64 threads own no elements
+    // when the span is 960 or less, and the answer, a memory round trip away, is there when the workgroup meets
+    // after the update.
+    constexpr int kLooker = kResBlock - kWave;
     // ring slot of step t-1 and history rows of steps t and t-1-B, counted along instead of taking three
     // 64-bit remainders per step (every instruction of the loop costs all 16 wavefronts an issue slot)
     auto wrap = [](int64_t a, int m) { return (int)(((a % m) + m) % m); };
@@ -328,6 +328,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         if (k > 0) PROF_ADD(1, prof_prev, c0);
 #endif
         const int64_t kn = in_bound(t + 1 - B);
+        if (defer && k > 0 && tid == kLooker) go_on = poll(k - 1);
         // 1. fold the arrivals of slot t-1 and update
         bool spike = false;
         float frac = 0.0f;
@@ -386,7 +387,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
 #ifdef BMTK_RES_PROFILE
             prof_c1 = c1;
 #endif
-            if (defer && k > 0 && !wait_for(k - 1)) {
+            if (defer && k > 0 && !go_on) {  // written before the workgroup met above
                 aborted = true;
                 break;
             }
