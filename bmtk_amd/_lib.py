@@ -53,7 +53,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 6  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 7  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -85,7 +85,7 @@ SIGNATURES = {
 }
 
 
-RES_SYNC_WORDS = 65 * 1088  # BMTK_RES_SYNC_WORDS
+RES_SYNC_WORDS = (1 + 64 * 8) * 1088  # BMTK_RES_SYNC_WORDS
 
 
 class LibraryMissing(RuntimeError):

@@ -58,7 +58,12 @@ constexpr int kBarrierWords = 64;        // per-step arrival counters, used roun
 // counter of the step before must not queue up behind that burst, so every counter lives in a memory channel
 // of its own rather than side by side in one cache line.
 constexpr int kBarrierStride = BMTK_RES_SYNC_STRIDE;
-static_assert(BMTK_RES_SYNC_WORDS >= (1 + kBarrierWords) * kBarrierStride, "res_sync too small");
+// For the same reason a step's arrivals are spread over kWays counters (the workgroups of one XCD share one) and
+// a look adds them up: the burst on one address is then an eighth as long, and so is the time the barrier takes
+// to fill.  Counter (slot i, way x) is word (x * kBarrierWords + i) * kBarrierStride of the counter area.
+constexpr int kWays = BMTK_RES_SYNC_WAYS;
+constexpr int kWayStride = kBarrierWords * kBarrierStride;
+static_assert(BMTK_RES_SYNC_WORDS >= (1 + kWays * kBarrierWords) * kBarrierStride, "res_sync too small");
 constexpr int kMaxSlack = 31;
 
 #ifdef BMTK_RES_PROFILE
@@ -287,7 +292,16 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         const unsigned *word = counter_of(j);
         const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
         unsigned spins = 0;
-        while (load_agent(word) < target) {
+        auto arrived = [&]() {  // the loads of a look travel together
+            unsigned n[kWays];
+#pragma unroll
+            for (int x = 0; x < kWays; ++x) n[x] = load_agent(word + x * kWayStride);
+            unsigned sum = 0;
+#pragma unroll
+            for (int x = 0; x < kWays; ++x) sum += n[x];
+            return sum;
+        };
+        while (arrived() < target) {
             if (load_agent(abort_word) != 0u) return 0;
             if (++spins > (s.res_spin_limit ? s.res_spin_limit : kMaxSpin)) {
                 __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -380,7 +394,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
             PROF_T(c1);
             // 2. arrive at the barrier of step t (ballots of this workgroup are out)
             if (tid == 0)
-                __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)) * kBarrierStride, 1u, __ATOMIC_RELAXED,
+                __hip_atomic_fetch_add(counter_of(k) + (blockIdx.x & (kWays - 1)) * kWayStride, 1u, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
             PROF_ADD(0, c0, c1);
             PROF_BLK(0, c0, c1);
@@ -410,7 +424,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         //  writes below was last read before the barrier that precedes the arrival)
         PROF_T(c3);
         if (late && tid == 0)
-            __hip_atomic_fetch_add(arrivals + (k & (kBarrierWords - 1)) * kBarrierStride, 1u, __ATOMIC_RELAXED,
+            __hip_atomic_fetch_add(counter_of(k) + (blockIdx.x & (kWays - 1)) * kWayStride, 1u, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
         // 4. every `check` steps (each step without slack) wait until every workgroup has published
         //    step k - S + (check - 1): enough for the steps up to the next look
@@ -469,7 +483,7 @@ __global__ void zero_words_kernel(unsigned *w, int n)
 __global__ void zero_sync_kernel(unsigned *sync)
 {
     if (threadIdx.x < 2) sync[threadIdx.x] = 0u;
-    if ((int)threadIdx.x < kBarrierWords) sync[(1 + (int)threadIdx.x) * kBarrierStride] = 0u;
+    for (int c = threadIdx.x; c < kWays * kBarrierWords; c += blockDim.x) sync[(1 + c) * kBarrierStride] = 0u;
 }
 
 __global__ __launch_bounds__(kBlock) void segment_offsets_kernel(int64_t n_rows, const int32_t *__restrict__ indptr,
@@ -530,7 +544,7 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
                   n_cu, per_cu);
         return BMTK_E_LAUNCH;
     }
-    hipLaunchKernelGGL(zero_sync_kernel, dim3(1), dim3(128), 0, stream, s.res_sync);
+    hipLaunchKernelGGL(zero_sync_kernel, dim3(1), dim3(kBlock), 0, stream, s.res_sync);
     bmtk_glif3_sim s_copy = s;
     // BMTK_AMD_PLAIN_LAUNCH=1 uses an ordinary launch (co-residency then rests on the occupancy check
     // above and an otherwise idle device); for tools that cannot follow cooperative launches.

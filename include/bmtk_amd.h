@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 6
+#define BMTK_AMD_ABI_VERSION 7
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -156,7 +156,8 @@ int bmtk_csr_segment_offsets(int64_t n_rows, const int32_t *indptr, const int32_
                              int32_t n_groups, uint32_t *seg, int32_t *unsorted, void *stream);
 
 #define BMTK_RES_SYNC_STRIDE 1088                          /* words: 4 KiB + 256 B */
-#define BMTK_RES_SYNC_WORDS (65 * BMTK_RES_SYNC_STRIDE)    /* size of bmtk_glif3_sim.res_sync */
+#define BMTK_RES_SYNC_WAYS 8                               /* counters a step's arrivals are spread over */
+#define BMTK_RES_SYNC_WORDS ((1 + 64 * BMTK_RES_SYNC_WAYS) * BMTK_RES_SYNC_STRIDE) /* size of bmtk_glif3_sim.res_sync */
 
 /* Everything nest.Simulate needs for a forward run (bmtk/simulator/pointnet/pointsimulator.py:159-166). */
 typedef struct bmtk_glif3_sim {
@@ -215,9 +216,9 @@ typedef struct bmtk_glif3_sim {
     const uint32_t *rec_seg;     /* [neurons][res_groups+1] */
     const uint32_t *inp_seg;     /* [inputs][res_groups+1] */
     uint32_t *res_sync;          /* BMTK_RES_SYNC_WORDS words of scratch: word 1 = abort flag, from word
-                                  * BMTK_RES_SYNC_STRIDE on 64 per-step arrival counters that many words apart; the call zeroes what it
-                                  * uses.  After the run, word 1 != 0 means the grid barrier timed out and the
-                                  * results are invalid. */
+                                  * BMTK_RES_SYNC_STRIDE on 64 x BMTK_RES_SYNC_WAYS arrival counters that many
+                                  * words apart; the call zeroes what it uses.  After the run, word 1 != 0 means
+                                  * the grid barrier timed out and the results are invalid. */
     /* Pull form of the recurrent delivery for batched runs (optional; launch-per-step mode with delay_offset 0
      * and hist_slots == ring_slots): a TARGET-major packed copy of the recurrent table.  The recurrent arrivals
      * of step t-1 are then summed in one pass over that table from the spike-bit history
