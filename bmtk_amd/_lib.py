@@ -33,6 +33,8 @@ class Glif3Sim(C.Structure):
         ("pull_inp_work", c_void_p), ("in_hist", c_void_p), ("in_hist_stride", c_int64),
         ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
         ("save_v", c_void_p), ("save_flags", c_void_p),
+        ("probe_col", c_void_p), ("probe_v", c_void_p), ("probe_stride", c_int64), ("probe_every", c_int32),
+        ("_pad1", c_int32),
         ("spike_step", c_void_p), ("spike_elem", c_void_p), ("spike_frac", c_void_p),
         ("spike_cap", c_int64), ("spike_count", c_void_p),
     ]
@@ -53,7 +55,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 7  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 8  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {

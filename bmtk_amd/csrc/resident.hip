@@ -272,6 +272,10 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     }
     __syncthreads();
 
+    // membrane potential probes: this thread's column, and where in the sampling period the call begins
+    const int probe_col = (own && s.probe_col) ? s.probe_col[e] : -1;
+    int probe_phase = s.probe_col ? (int)((r.step0 + 1) % s.probe_every) : 1;  // 0: sample after this step
+    int64_t probe_row = 0;
     const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
     bool aborted = false;
     int64_t done = 0;  // steps whose update has run
@@ -357,6 +361,13 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
                 }
             }
             spike = glif3_update(st, p, s.h, zero, I, &frac);
+        }
+        if (s.probe_col) {
+            if (probe_phase == 0) {
+                if (probe_col >= 0) s.probe_v[probe_row * s.probe_stride + probe_col] = st.V;
+                ++probe_row;
+            }
+            probe_phase = probe_phase + 1 == s.probe_every ? 0 : probe_phase + 1;
         }
         const unsigned long long m = __ballot(spike);
         // only the wavefronts that cover this workgroup's span own a ballot word

@@ -43,6 +43,7 @@ struct SimLaunch {
     int pull;          // pull_syn holds the recurrent arrivals of step t-1, to be folded with slot t-1
     int pull_inp;      // pull_inp_syn holds the input arrivals of step t-1
     int idx_bits;      // width of the index field of the packed tables (24 in the standard packing)
+    int64_t probe_row; // row of probe_v this step's potentials go to, -1: not a sampled step
 };
 
 // walk one row of a packed table, four 64-synapse chunks in flight at a time
@@ -183,6 +184,10 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
             const int ref_before = st.ref;
             spike = glif3_update(st, p, s.h, zero, I, &frac);
             glif3_store(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
+            if (q.probe_row >= 0) {
+                const int col = s.probe_col[e];
+                if (col >= 0) s.probe_v[q.probe_row * s.probe_stride + col] = st.V;
+            }
             if (s.save_v) {
                 s.save_v[q.out_row * ne + e] = st.V;
                 s.save_flags[q.out_row * ne + e] = (uint8_t)((spike ? BMTK_F_SPIKE : 0) |
@@ -356,6 +361,8 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
         BMTK_REQUIRE(s.in_hist_stride >= (s.n_inputs * (int64_t)s.batch + 63) / 64 + 1,
                      "glif3_simulate_fwd: in_hist_stride must hold ceil(n_inputs*batch/64)+1 words");
     }
+    BMTK_REQUIRE(!s.probe_col || (s.probe_v && s.probe_every >= 1 && s.probe_stride >= 1),
+                 "glif3_simulate_fwd: probes need probe_v, probe_stride and probe_every >= 1");
     SimLaunch q{};
     q.n_update = (int)((ne + kSimBlock - 1) / kSimBlock);
     const int64_t max_deliver = (words + kSimWaves - 1) / kSimWaves;  // at least one word per wavefront
@@ -371,6 +378,10 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
         q.hist = hist;
         q.idx_bits = 30 - delay_bits;
         q.out_row = k;
+        // sampled steps: (t + 1) % every == 0; row = how many of them the call has seen before
+        q.probe_row = -1;
+        if (s.probe_col && !closing && (q.t + 1) % s.probe_every == 0)
+            q.probe_row = (q.t + 1) / s.probe_every - step0 / s.probe_every - 1;
         q.do_update = closing ? 0 : 1;
         q.fold_prev = k > 0;
         // the first launch of a call delivers nothing: the closing launch of the call before it did

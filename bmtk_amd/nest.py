@@ -394,9 +394,7 @@ def _build():
                           cat(ir, np.uint8), n_rows=max(1, gen_ids.size), major="source") if is_ else None
     try:
         # delays beyond the 63 steps of the ring are taken up by a delay offset (smallest delay - 1)
-        # a membrane record is kept by the launch-per-step driver only
-        sim = Glif3Simulator(n, par, dt, rec=rec, inp=inp, asc_init=asc_init, u_init=u_init,
-                             **(dict(resident=False, pull=False) if _S.mm_links else {}))
+        sim = Glif3Simulator(n, par, dt, rec=rec, inp=inp, asc_init=asc_init, u_init=u_init)
     except ValueError as err:
         if "delays span" in str(err):
             raise _Errors.BadDelay(str(err), "BadDelay")
@@ -450,10 +448,21 @@ def Simulate(t_ms):
             k = int(round((tt + dt) / dt))
             if step0 < k < step0 + n_steps:
                 bounds.add(k)
-    if _S.mm_links:  # the per-step membrane record is taken in pieces of bounded size
-        piece = max(1, (1 << 26) // max(1, sim.ne))
+    probed = None
+    if _S.mm_links:
+        # one set of probes serves every multimeter: the union of their neurons at the largest common interval;
+        # the record is taken in pieces of bounded size
+        import math
+        probed = np.unique(np.concatenate([s["n_of"][ids] for _, ids in _S.mm_links]))
+        every = 0
+        for m, _ in _S.mm_links:
+            every = math.gcd(every, int(round(float(_S.params[m - 1]["interval"]) / dt)))
+        sim.set_probes(probed, every=every)
+        piece = max(1, (1 << 26) * every // probed.size)
         for k in range(step0 + piece, step0 + n_steps, piece):
             bounds.add(k)
+    else:
+        sim.set_probes(None)
     bounds = sorted(bounds)
     want_record = bool(_S.rec_links)
     senders, times = [], []
@@ -462,18 +471,21 @@ def Simulate(t_ms):
         if _S.cur_links:
             sim.i_ext = torch.as_tensor(_current_at(a), device=sim.dev)
         cap = int(min(max(4096, (b - a) * sim.ne), 1 << 26)) if want_record else 0
-        out = sim.run(b - a, spike_bits=False, record_cap=cap, save_state=bool(_S.mm_links))
+        out = sim.run(b - a, spike_bits=False, record_cap=cap)
+        sampled = stamps = None
+        if _S.mm_links and out["probe"]["steps"].numel():
+            # NEST samples at the end of a step: the potential after step t is stamped (t + 1) * dt
+            stamps = out["probe"]["steps"].numpy() + 1
+            sampled = out["probe"]["v"].cpu().numpy().astype(np.float64)
         for m, ids in _S.mm_links:
-            # NEST samples at the end of a step: row k of the record is the potential at time (a + k + 1) * dt
+            if sampled is None:
+                break
             p = _S.params[m - 1]
             every = int(round(float(p["interval"]) / dt))
-            stamps = np.arange(a + 1, b + 1)
             keep = (stamps % every == 0) & (stamps * dt > float(p["start"]) + 1e-9) & \
                    (stamps * dt <= float(p["stop"]) + 1e-9)
             if keep.any():
-                cols = torch.as_tensor(s["n_of"][ids], device=sim.dev)
-                rows = torch.as_tensor(np.flatnonzero(keep), device=sim.dev)
-                v = out["saved"]["v"].view(b - a, sim.ne)[rows][:, cols].cpu().numpy().astype(np.float64)
+                v = sampled[keep][:, np.searchsorted(probed, s["n_of"][ids])]
                 v += s["e_l"][s["n_of"][ids]][None, :]
                 mm_rows[m][0].append(np.tile(ids, int(keep.sum())))
                 mm_rows[m][1].append(np.repeat(stamps[keep] * dt, ids.size))

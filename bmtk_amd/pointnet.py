@@ -19,6 +19,7 @@ entries of module ``multimeter_report`` / ``membrane_report`` for ``V_m``
 become SONATA cell-variable files
 (bmtk/simulator/pointnet/modules/multimeter_reporter.py:64-140).
 """
+import math
 import os
 
 import numpy as np
@@ -175,8 +176,15 @@ class PointSimulator:
         rec, inp = nw.device_tables(self._device)
         sim = Glif3Simulator(nw.n, nw.par, self.dt, class_id=nw.class_id, rec=rec, inp=inp,
                              asc_init=nw.asc_init[:, nw.class_id], u_init=nw.u_init[nw.class_id],
-                             i_ext=np.zeros(nw.n, np.float32), device=self._device,
-                             **(dict(resident=False, pull=False) if self.reports else dict(resident=self._resident)))
+                             i_ext=np.zeros(nw.n, np.float32), device=self._device, resident=self._resident)
+        probed = None
+        if self.reports:
+            # one set of probes serves every report: the union of their cells, at the largest common interval
+            probed = np.unique(np.concatenate([rep["node_ids"] for rep in self.reports.values()]))
+            every = 0
+            for rep in self.reports.values():
+                every = math.gcd(every, rep["every"])
+            sim.set_probes(probed, every=every)
         if inp is not None:
             sim.set_input_events(*bin_spike_times(self._trains, self.dt, self.n_steps))
         steps, elems, fracs = [], [], []
@@ -185,23 +193,24 @@ class PointSimulator:
         pieces = []
         for a, b, cur in self._segments():
             # a membrane record is taken in pieces of bounded size
-            piece = max(1, (1 << 26) // nw.n) if self.reports else b - a
+            piece = max(1, (1 << 26) * sim.probe_every // probed.size) if self.reports else b - a
             pieces += [(k, min(k + piece, b), cur) for k in range(a, b, piece)]
         for a, b, cur in pieces:
             sim.i_ext.copy_(torch.as_tensor(cur, device=sim.dev))
             cap = record_cap or max(1 << 16, (b - a) * nw.n // 8)
-            out = sim.run(b - a, spike_bits=False, record_cap=cap, save_state=bool(self.reports))
+            out = sim.run(b - a, spike_bits=False, record_cap=cap)
             sim.check()
-            for rep in self.reports.values():
+            if self.reports and out["probe"]["steps"].numel():
                 # the sample stamped t is the potential at the end of the step that ends at t
-                stamps = np.arange(a + 1, b + 1)
-                keep = (stamps % rep["every"] == 0) & (stamps * self.dt > rep["tstart"] + 1e-9) & \
-                       (stamps * self.dt <= rep["tstop"] + 1e-9)
-                if keep.any():
-                    rows = torch.as_tensor(np.flatnonzero(keep), device=sim.dev)
-                    cols = torch.as_tensor(rep["node_ids"], device=sim.dev)
-                    v = out["saved"]["v"].view(b - a, nw.n)[rows][:, cols].cpu().numpy().astype(np.float64)
-                    rep["rows"].append((stamps[keep] * self.dt, v + e_l[rep["node_ids"]][None, :]))
+                stamps = out["probe"]["steps"].numpy() + 1
+                sampled = out["probe"]["v"].cpu().numpy().astype(np.float64)
+                for rep in self.reports.values():
+                    keep = (stamps % rep["every"] == 0) & (stamps * self.dt > rep["tstart"] + 1e-9) & \
+                           (stamps * self.dt <= rep["tstop"] + 1e-9)
+                    if keep.any():
+                        cols = np.searchsorted(probed, rep["node_ids"])
+                        rep["rows"].append((stamps[keep] * self.dt,
+                                            sampled[keep][:, cols] + e_l[rep["node_ids"]][None, :]))
             r = out["record"]
             c = int(r["count"].item())
             if c > cap:

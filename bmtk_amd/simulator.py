@@ -126,6 +126,8 @@ class Glif3Simulator:
         self.res_span = self.res_groups = 0
         self.rec_seg = self.inp_seg = None
         self._pending_check = False
+        self.probe_ids = self.probe_col = None
+        self.probe_every = 1
         self.spin_limit = 0  # resident mode: polls of the grid barrier before giving up (0 = built-in limit)
         if resident:
             self._setup_resident(required=(resident is True))
@@ -249,11 +251,29 @@ class Glif3Simulator:
             s.spike_cap, s.spike_count = record["step"].numel(), _p(record["count"])
         return s
 
+    def set_probes(self, element_ids, every=1):
+        """Record the membrane potential of some elements (what a multimeter connected to them does): after every
+        step t with (t + 1) % every == 0, in both modes.  ``run`` then returns ``probe`` = dict(v=[samples,
+        len(element_ids)] fp32 of U = V_m - E_L, steps=int64 [samples], the sampled steps).  None switches it off."""
+        if element_ids is None:
+            self.probe_ids = self.probe_col = None
+            return
+        ids = np.asarray(element_ids, np.int64).reshape(-1)
+        if ids.size == 0 or ids.min() < 0 or ids.max() >= self.ne or np.unique(ids).size != ids.size:
+            raise ValueError("probes need distinct element ids in 0..{}".format(self.ne - 1))
+        if int(every) < 1:
+            raise ValueError("every must be at least 1")
+        col = np.full(self.ne, -1, np.int32)
+        col[ids] = np.arange(ids.size, dtype=np.int32)
+        self.probe_ids, self.probe_every = ids, int(every)
+        self.probe_col = torch.as_tensor(col, device=self.dev)
+
     def run(self, n_steps, spike_bits=True, record_cap=0, save_state=False):
         """Advance ``n_steps`` steps.  Returns a dict with ``bits`` (int64
         [n_steps, words], spike bits per step) and, when ``record_cap`` > 0,
         the atomic spike record with crossing fractions; ``save_state`` adds the
-        per-step record (potentials and flags) the backward pass reads.  Does not
+        per-step record (potentials and flags) the backward pass reads; ``probe``
+        holds the potentials asked for with ``set_probes``.  Does not
         synchronise."""
         if self.in_ptr is not None and self.step + n_steps > self.in_steps:
             raise ValueError("input event lists cover {} steps, run would reach {}".format(
@@ -273,10 +293,19 @@ class Glif3Simulator:
             saved = dict(v=torch.empty(n_steps, self.ne, device=self.dev),
                          flags=torch.empty(n_steps, self.ne, dtype=torch.uint8, device=self.dev), step0=self.step)
             s.save_v, s.save_flags = _p(saved["v"]), _p(saved["flags"])
+        probe = None
+        if self.probe_col is not None:
+            every = self.probe_every
+            first = -(-(self.step + 1) // every) * every - 1  # first step t >= self.step with (t + 1) % every == 0
+            steps = torch.arange(first, self.step + n_steps, every, dtype=torch.int64)
+            probe = dict(v=torch.empty(max(1, steps.numel()), self.probe_ids.size, device=self.dev)[:steps.numel()],
+                         steps=steps)
+            s.probe_col, s.probe_v = _p(self.probe_col), probe["v"].data_ptr()
+            s.probe_stride, s.probe_every = self.probe_ids.size, every
         _lib.check(self.lib.bmtk_glif3_simulate_fwd(C.byref(s), self.step, n_steps, _stream()))
         self.step += n_steps
         self._pending_check = bool(self.res_span)
-        return dict(bits=bits, record=record, saved=saved)
+        return dict(bits=bits, record=record, saved=saved, probe=probe)
 
     def spikes_from_bits(self, bits, step0=0):
         """Spike bits -> (step int64[], element int64[]) ascending, via the

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 7
+#define BMTK_AMD_ABI_VERSION 8
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -246,6 +246,15 @@ typedef struct bmtk_glif3_sim {
      * save_v[k][e] = membrane potential after step step0+k, save_flags[k][e] = BMTK_F_* bits */
     float *save_v;
     uint8_t *save_flags;
+    /* optional membrane potential probes (both modes; what a NEST multimeter connected to some neurons records):
+     * probe_col[e] = column of element e in probe_v, or -1.  After every step t with (t + 1) % probe_every == 0
+     * the potentials U = V_m - E_L of the probed elements go to the next row of probe_v, row 0 being the first
+     * such step of the call; probe_v must hold as many rows of probe_stride floats as the call has such steps. */
+    const int32_t *probe_col;    /* [ne] or NULL */
+    float *probe_v;
+    int64_t probe_stride;
+    int32_t probe_every;         /* >= 1 */
+    int32_t _pad1;
     /* optional spike record with sub-step crossing fractions, appended with
      * atomics (unordered within a step); all NULL to disable */
     int32_t *spike_step;

@@ -339,3 +339,32 @@ def test_resident_barrier_gives_up_cleanly():
     out = sim.run(300)
     sim.check()
     assert (sim.raster(out["bits"]).cpu().numpy() == want["raster"][:300]).mean() >= 0.999
+
+
+@pytest.mark.parametrize("every", [1, 3])
+def test_membrane_probes_equal_the_per_step_record(every):
+    """set_probes on both drivers against the full per-step record of the launch-per-step driver: same potentials,
+    bit for bit (exact weights), at the sampled steps, over two calls whose boundary is no multiple of `every`."""
+    cfg = synthetic.small_glif3_network(n=3000, n_in=500, steps=200, seed=8, in_w_scale=3.0, in_fanout=300,
+                                        p_conn=0.03, w_scale=1.5)
+    cfg["rec_src"] = _integer_weights(cfg["rec_src"])
+    cfg["inp_src"] = _integer_weights(cfg["inp_src"])
+    ref = _gpu_sim(cfg, resident=False)
+    full = ref.run(200, save_state=True)["saved"]["v"].view(200, cfg["n"]).cpu().numpy()
+    ids = np.array([2999, 0, 17, 1500, 64, 959, 960])
+    for resident in (False, True):
+        sim = _gpu_sim(cfg, resident=resident)
+        sim.set_probes(ids, every=every)
+        got_v, got_steps = [], []
+        for n in (70, 130):
+            out = sim.run(n)["probe"]
+            got_v.append(out["v"].cpu().numpy())
+            got_steps.append(out["steps"].numpy())
+        sim.check()
+        steps = np.concatenate(got_steps)
+        np.testing.assert_array_equal(steps, np.arange(every - 1, 200, every))
+        np.testing.assert_array_equal(np.concatenate(got_v), full[steps][:, ids])
+    with pytest.raises(ValueError):
+        sim.set_probes([1, 1])
+    with pytest.raises(ValueError):
+        sim.set_probes([cfg["n"]])
