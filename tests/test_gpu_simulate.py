@@ -246,6 +246,37 @@ def test_v1_scale_resident_equals_per_step_launches():
     assert torch.equal(bits[0], bits[1])
 
 
+def test_resident_with_every_thread_owning_an_element():
+    """250,000 neurons on 248 workgroups make the span 1024: the sixteenth wavefront, which otherwise only looks at
+    the grid barrier while the others update, has elements of its own here.  Same spikes and state as the
+    per-step launches."""
+    import torch
+    rng = np.random.default_rng(5)
+    n, n_in, steps = 250_000, 5000, 200
+    par = synthetic.random_cells(rng, 37)
+    cid = rng.integers(0, 37, n).astype(np.int32)
+    _, by_src, _ = synthetic.device_network(n, 40, "lognormal", seed=6)
+    by_src = (by_src[0], by_src[1], (torch.round(by_src[2] * 4) / 4 + torch.sign(by_src[2]) * 0.25) * 4.0, by_src[3],
+              by_src[4])
+    inp = synthetic.device_input_table(n_in, n, 2_000_000, seed=7, w_scale=9.0)
+    inp = (inp[0], inp[1], torch.round(inp[2] * 4) / 4 + 0.25, inp[3], inp[4])
+    in_ptr, in_ev = synthetic.device_poisson_events(n_in, 20.0, 1.0, steps, seed=8)
+    bits, states = [], []
+    for resident in (False, True):
+        sim = Glif3Simulator(n, par, 1.0, class_id=cid, rec=by_src, inp=inp, resident=resident)
+        assert bool(sim.res_span) == resident and (not resident or sim.res_span == 1024)
+        sim.set_input_events(in_ptr, in_ev)
+        out = sim.run(steps)
+        sim.check()
+        bits.append(out["bits"].cpu())
+        states.append(sim.state.to_numpy())
+        del sim
+    assert int(ops_popcount(bits[0])) > 20000
+    assert torch.equal(bits[0], bits[1])
+    for k in states[0]:
+        np.testing.assert_array_equal(states[0][k], states[1][k], err_msg=k)
+
+
 def ops_popcount(bits):
     import torch
     x = bits.reshape(-1)
