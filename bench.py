@@ -124,7 +124,7 @@ def bench_compaction(torch, steps=200, warmup=20):
         per = dev / steps
         count = int(comp.count.item())
         alg = scan_bytes + 4 * count
-        out.append({"kernel": "compact_count/scan/write (%s)" % name,
+        out.append({"kernel": "compact_count + compact_write_fused (%s)" % name,
                     "workload": "compaction of %d elements, %d spikes" % (n, count),
                     "elements_per_s": n / per, "us_per_call": per * 1e6,
                     "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -210,6 +210,68 @@ __global__ __launch_bounds__(kBlock) void compact_write_kernel(const uint64_t *_
     }
 }
 
+// Two launches instead of three or four, for up to kMaxFused blocks: the first counts (from flags it also packs
+// the bits, 64 flags per thread), the second has every workgroup add up the counts of the workgroups before
+// it by itself -- a few KB from L2 -- instead of waiting for a scan launch in between.
+constexpr int kMaxFused = 4096;
+
+// bits 0..3 = which of the four bytes of x are non-zero
+__device__ __forceinline__ unsigned nonzero_bytes(unsigned x)
+{
+    const unsigned high = (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;  // bit 7 of every non-zero byte
+    return (((high >> 7) * 0x00204081u) >> 21) & 0xFu;                             // bits 0, 8, 16, 24 -> 0..3
+}
+
+__global__ __launch_bounds__(kBlock) void compact_count_flags_kernel(const uint8_t *__restrict__ z, int64_t n,
+                                                                     int64_t n_words, uint64_t *__restrict__ bits,
+                                                                     uint32_t *__restrict__ block_count)
+{
+    const int64_t w = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x;
+    unsigned long long v = 0ull;
+    if (w < n_words) {
+        const int64_t e0 = w << 6;
+        if (e0 + 64 <= n) {
+            const uint4 *q = reinterpret_cast<const uint4 *>(z + e0);  // z is 16-byte aligned (checked by the caller)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint4 x = q[i];
+                const unsigned long long part = nonzero_bytes(x.x) | (nonzero_bytes(x.y) << 4) |
+                                                (nonzero_bytes(x.z) << 8) | (nonzero_bytes(x.w) << 12);
+                v |= part << (16 * i);
+            }
+        } else {
+            for (int64_t e = e0; e < n; ++e) v |= (unsigned long long)(z[e] != 0) << (e - e0);
+        }
+        bits[w] = v;
+    }
+    unsigned total;
+    block_exclusive_scan((unsigned)__popcll(v), &total);
+    if (threadIdx.x == 0) block_count[blockIdx.x] = total;
+}
+
+// block_count holds the plain per-block counts here
+__global__ __launch_bounds__(kBlock) void compact_write_fused_kernel(const uint64_t *__restrict__ bits, int64_t n_words,
+                                                                     int64_t n, const uint32_t *__restrict__ block_count,
+                                                                     int32_t *__restrict__ ids,
+                                                                     int32_t *__restrict__ count)
+{
+    unsigned before = 0;
+    for (int b = threadIdx.x; b < (int)blockIdx.x; b += kBlock) before += block_count[b];
+    unsigned offset;
+    block_exclusive_scan(before, &offset);  // the block sum is what is wanted
+    const int64_t w = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x;
+    unsigned long long v = load_word(bits, w, n_words, n);
+    unsigned total;
+    unsigned pos = offset + block_exclusive_scan((unsigned)__popcll(v), &total);
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) *count = (int32_t)(offset + total);
+    const int32_t base = (int32_t)(w << 6);
+    while (v) {
+        const int b = __ffsll((long long)v) - 1;
+        v &= v - 1ull;
+        ids[pos++] = base + b;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Event-driven scatter: one wavefront per active element walks the source's
 // out-going synapses 64 at a time (coalesced table reads), fp32 atomics into
@@ -365,6 +427,13 @@ static int compact_from_bits(const uint64_t *bits, int64_t n, int32_t *ids, int3
 {
     const int64_t n_words = n_words_of(n);
     const int n_blocks = (int)n_blocks_of(n);
+    if (n_blocks <= kMaxFused) {
+        hipLaunchKernelGGL(compact_count_kernel, dim3(n_blocks), dim3(kBlock), 0, stream, bits, n_words, n, block_count);
+        hipLaunchKernelGGL(compact_write_fused_kernel, dim3(n_blocks), dim3(kBlock), 0, stream, bits, n_words, n,
+                           (const uint32_t *)block_count, ids, count);
+        BMTK_CHECK_LAUNCH("spikes_compact");
+        return BMTK_OK;
+    }
     hipLaunchKernelGGL(compact_count_kernel, dim3(n_blocks), dim3(kBlock), 0, stream, bits, n_words, n, block_count);
     hipLaunchKernelGGL(compact_scan_kernel, dim3(1), dim3(kBlock), 0, stream, block_count, n_blocks, count);
     hipLaunchKernelGGL(compact_write_kernel, dim3(n_blocks), dim3(kBlock), 0, stream, bits, n_words, n,
@@ -379,6 +448,15 @@ int bmtk_spikes_compact(const uint8_t *z, int64_t n, int32_t *ids, int32_t *coun
     BMTK_REQUIRE(z && ids && count && workspace, "spikes_compact: pointers must be non-null");
     uint64_t *bits = (uint64_t *)workspace;
     uint32_t *block_count = (uint32_t *)(bits + n_words_of(n) + 1);
+    const int n_blocks = (int)n_blocks_of(n);
+    if (n_blocks <= kMaxFused && (reinterpret_cast<uintptr_t>(z) & 15u) == 0) {
+        hipLaunchKernelGGL(compact_count_flags_kernel, dim3(n_blocks), dim3(kBlock), 0, (hipStream_t)stream, z, n,
+                           n_words_of(n), bits, block_count);
+        hipLaunchKernelGGL(compact_write_fused_kernel, dim3(n_blocks), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const uint64_t *)bits, n_words_of(n), n, (const uint32_t *)block_count, ids, count);
+        BMTK_CHECK_LAUNCH("spikes_compact");
+        return BMTK_OK;
+    }
     const unsigned grid = (unsigned)((n + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(pack_bits_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, z, n, bits);
     return compact_from_bits(bits, n, ids, count, block_count, (hipStream_t)stream);

@@ -24,6 +24,26 @@ def test_compaction_is_flatnonzero(n, p):
         np.testing.assert_array_equal(ids[:c].cpu().numpy(), want)
 
 
+def test_compaction_other_paths():
+    """Flags that do not start on a 16-byte boundary (the packing then goes through the one-flag-per-thread kernel),
+    non-zero flags other than 1, and an input beyond the size the fused two-launch form takes."""
+    rng = np.random.default_rng(77)
+    z = (rng.random(100_001) < 0.01).astype(np.uint8) * rng.integers(1, 256, 100_001).astype(np.uint8)
+    dev = to_dev(z)
+    for off in (1, 5, 16):
+        comp = ops.SpikeCompactor(z.size - off)
+        ids, count = comp(dev[off:])
+        want = np.flatnonzero(z[off:]).astype(np.int32)
+        assert int(count.item()) == want.size
+        np.testing.assert_array_equal(ids[:want.size].cpu().numpy(), want)
+    n = (1 << 26) + 5
+    big = torch.zeros(n, dtype=torch.uint8, device=dev.device)
+    hot = torch.as_tensor(np.sort(rng.choice(n, 50_000, replace=False)), device=dev.device)
+    big[hot] = 1
+    ids, count = ops.SpikeCompactor(n)(big)
+    assert int(count.item()) == 50_000 and torch.equal(ids[:50_000].long(), hot)
+
+
 def test_compaction_ignores_bits_beyond_n():
     z = np.zeros(100, np.uint8)
     z[[3, 99]] = 1
