@@ -146,3 +146,24 @@ def test_known_answer_at_fine_resolution(golden_dir, h, atol):
         assert c == len(exp["times"])
         t = (rec["step"][:c].cpu().numpy() + rec["frac"][:c].cpu().numpy().astype(np.float64)) * h
         np.testing.assert_allclose(t, exp["times"], atol=atol, rtol=0)
+
+
+def test_probes_with_a_delay_offset():
+    """Membrane potential probes of the resident kernel running with slack (delays 101..104 steps) equal the
+    launch-per-step driver's, bit for bit."""
+    cfg = _network(100, steps=300)
+    ids = np.array([5, 1000, 2999])
+    got = []
+    for resident in (False, True):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], resident=resident)
+        assert sim.delay_offset == 100
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        sim.set_probes(ids, every=2)
+        a = sim.run(101)["probe"]
+        b = sim.run(199)["probe"]
+        sim.check()
+        assert np.array_equal(np.concatenate([a["steps"].numpy(), b["steps"].numpy()]), np.arange(1, 300, 2))
+        got.append(np.concatenate([a["v"].cpu().numpy(), b["v"].cpu().numpy()]))
+    assert np.abs(got[0]).max() > 1.0
+    np.testing.assert_array_equal(got[0], got[1])
