@@ -90,7 +90,7 @@ class PointSimulator:
             kind = entry.get("input_type")
             if kind == "spikes":
                 sim.add_spike_inputs(_read_input_spikes(entry), entry.get("node_set"))
-            elif kind == "current_clamp":
+            elif entry.get("module") == "IClamp" or kind == "current_clamp":
                 sim.add_current_clamp(entry)
             else:
                 raise NotImplementedError("input {!r}: input_type {!r} is not supported".format(name, kind))
@@ -109,14 +109,7 @@ class PointSimulator:
         var = var[0] if isinstance(var, (list, tuple)) and len(var) == 1 else var
         if var != "V_m":
             raise NotImplementedError("report {!r}: only V_m is recorded, not {!r}".format(name, var))
-        cells = entry.get("cells", "all")
-        if isinstance(cells, dict):
-            if cells.get("population", self.net.population) != self.net.population:
-                raise ValueError("report {!r}: population {!r} is not simulated".format(name, cells["population"]))
-            cells = cells.get("node_id", cells.get("node_ids", "all"))
-        ids = np.arange(self.net.n) if isinstance(cells, str) else np.asarray(cells, np.int64)
-        if ids.size and (ids.min() < 0 or ids.max() >= self.net.n):
-            raise ValueError("report {!r}: node id outside 0..{}".format(name, self.net.n - 1))
+        ids = self._node_ids_of(entry.get("cells", "all"))
         interval = float(entry.get("dt") or self.dt)
         every = interval / self.dt
         if every < 1 - 1e-9 or abs(every - round(every)) > 1e-6:
@@ -144,31 +137,79 @@ class PointSimulator:
                     self._trains[row] = ts[a:b]
 
     def add_current_clamp(self, entry):
-        """A step current on a list of node ids: ``amp`` pA from ``delay`` for ``duration`` ms
-        (bmtk/simulator/pointnet/modules/iclamp.py:8-54, NEST step_current_generator semantics: an amplitude set
-        for time t acts on the update that starts at t + dt)."""
-        ids = entry.get("node_set", {})
-        ids = ids.get("node_id", ids.get("node_ids")) if isinstance(ids, dict) else ids
-        if ids is None or isinstance(ids, str):
-            raise NotImplementedError("current_clamp needs an explicit node id list")
-        amps = np.atleast_1d(np.asarray(entry["amp"], np.float64))
-        delays = np.atleast_1d(np.asarray(entry["delay"], np.float64))
-        durs = np.atleast_1d(np.asarray(entry["duration"], np.float64))
-        for a, t0, dur in zip(amps, delays, durs):
-            self._clamps.append((np.asarray(ids, np.int64), float(a), float(t0), float(t0 + dur)))
+        """One current generator on a set of nodes, as bmtk's IClamp module sets up a NEST
+        ``step_current_generator`` (bmtk/simulator/pointnet/modules/iclamp.py:8-54, readers in
+        bmtk/simulator/core/modules/iclamp.py:9-58).  ``input_type`` "current_clamp": ``amp`` (pA), ``delay``,
+        ``duration`` (ms), scalars or lists of one length; an amplitude is switched off at delay + duration unless
+        the next one has begun by then.  "csv": ``file`` with the columns ``timestamps`` and ``amps`` (other names
+        through ``timestamps_column`` / ``amplitudes_column``, ``separator`` " "), taken as they are.  Onsets at or
+        before the resolution are skipped, as bmtk does.  An amplitude set for time t acts on the update that
+        starts at t + dt (NEST)."""
+        kind = entry.get("input_type", "current_clamp")
+        if kind == "current_clamp":
+            amps, delays, durs = (list(v) if isinstance(v, (list, tuple, np.ndarray)) else [v]
+                                  for v in (entry["amp"], entry["delay"], entry["duration"]))
+            if not len(amps) == len(delays) == len(durs):
+                raise ValueError("current clamp parameters amp, delay, duration must be same length when using list.")
+        elif kind == "csv":
+            import pandas as pd
+            table = pd.read_csv(entry["file"], sep=entry.get("separator", " "))
+            if len(table) < 2:
+                raise ValueError("csv file must be row oriented and contain two or more values.")
+            for col in (entry.get("timestamps_column", "timestamps"), entry.get("amplitudes_column", "amps")):
+                if col not in table.columns:
+                    raise ValueError('csv file missing column "{}".'.format(col))
+            delays = table[entry.get("timestamps_column", "timestamps")].to_numpy(np.float64).tolist()
+            amps = table[entry.get("amplitudes_column", "amps")].to_numpy(np.float64).tolist()
+            durs = None
+        else:
+            raise NotImplementedError("current clamp input_type {!r} is not supported".format(kind))
+        times, values = [], []
+        for i, (start, amp) in enumerate(zip(delays, amps)):
+            if start <= self.dt:
+                continue
+            times.append(float(start))
+            values.append(float(amp))
+            if durs is not None:
+                stop = start + durs[i]
+                if i + 1 == len(delays) or stop <= delays[i + 1]:
+                    times.append(float(stop))
+                    values.append(0.0)
+        if any(b <= a for a, b in zip(times[:-1], times[1:])):
+            raise ValueError("current clamp: amplitude times must be strictly increasing")  # NEST's BadProperty
+        self._clamps.append((self._node_ids_of(entry.get("node_set")), np.asarray(times), np.asarray(values)))
+
+    def _node_ids_of(self, node_set):
+        """Node ids of a ``node_set``: a list, a population name (or "all"), or {"population":…, "node_id"/"node_ids":
+        […]} with the ids optional."""
+        if isinstance(node_set, dict):
+            pop = node_set.get("population", self.net.population)
+            if pop != self.net.population:
+                raise ValueError("population {!r} is not simulated".format(pop))
+            node_set = node_set.get("node_id", node_set.get("node_ids"))
+        if node_set is None or (isinstance(node_set, str) and node_set in ("all", self.net.population)):
+            return np.arange(self.net.n)
+        if isinstance(node_set, str):
+            raise NotImplementedError("node set {!r}: only the simulated population or id lists".format(node_set))
+        ids = np.asarray(node_set, np.int64)
+        if ids.size and (ids.min() < 0 or ids.max() >= self.net.n):
+            raise ValueError("node id outside 0..{}".format(self.net.n - 1))
+        return ids
 
     def _segments(self):
         """Step ranges with a constant external current, and that current."""
+        def first_step(t):  # the update an amplitude set for time t first acts on
+            return min(self.n_steps, max(0, int(round(t / self.dt)) + 1))
         marks = {0, self.n_steps}
-        for _, _, t0, t1 in self._clamps:
-            for t in (t0, t1):
-                marks.add(min(self.n_steps, max(0, int(round(t / self.dt)) + 1)))
+        for _, times, _ in self._clamps:
+            marks.update(first_step(t) for t in times)
         marks = sorted(marks)
         for a, b in zip(marks[:-1], marks[1:]):
             cur = np.zeros(self.net.n, np.float32)
-            for ids, amp, t0, t1 in self._clamps:
-                if int(round(t0 / self.dt)) + 1 <= a < int(round(t1 / self.dt)) + 1:
-                    cur[ids] += amp
+            for ids, times, values in self._clamps:
+                on = [v for t, v in zip(times, values) if first_step(t) <= a]
+                if on:
+                    cur[ids] += np.float32(on[-1])
             yield a, b, cur
 
     def run(self, record_cap=None):

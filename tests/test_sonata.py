@@ -390,3 +390,55 @@ def test_manifest_rules(tmp_path):
         _config(tmp_path, {"manifest": {"$BASE": "/base", "$TMP": "$VAR/Smat"}})
     with pytest.raises(ValueError):
         _config(tmp_path, {"manifest": {"$BASE": "$TMP/share", "$TMP": "$BASE/share"}})
+
+
+def _bare_simulator(dt=0.1, tstop=3500.0, n=120):
+    from types import SimpleNamespace
+    from bmtk_amd import pointnet
+    net_ = SimpleNamespace(n=n, n_inputs=0, population="cortex", virtual={})
+    return pointnet.PointSimulator(net_, dt, tstop)
+
+
+def test_current_clamp_amplitude_lists():
+    """The amplitude times/values bmtk's IClamp module hands to a step_current_generator
+    (bmtk/simulator/pointnet/modules/iclamp.py:13-39) for the inputs of examples/point_iclamp."""
+    sim = _bare_simulator()
+    # config.simulation_iclamp.aslist.json: three steps, each switched off before the next begins
+    sim.add_current_clamp({"input_type": "current_clamp", "module": "IClamp", "node_set": {"population": "cortex"},
+                           "amp": [0.15, 0.175, 0.2], "delay": [500.0, 1500.0, 2500.0],
+                           "duration": [500.0, 500.0, 500.0]})
+    ids, times, values = sim._clamps[-1]
+    assert ids.tolist() == list(range(120))
+    assert times.tolist() == [500.0, 1000.0, 1500.0, 2000.0, 2500.0, 3000.0]
+    assert values.tolist() == [0.15, 0.0, 0.175, 0.0, 0.2, 0.0]
+    # an amplitude still on when the next begins is replaced, not switched off; an onset at or before dt is skipped
+    sim.add_current_clamp({"input_type": "current_clamp", "node_set": {"population": "cortex", "node_ids": [3, 4]},
+                           "amp": [9.0, 1.0, 2.0], "delay": [0.1, 10.0, 15.0], "duration": [5.0, 20.0, 5.0]})
+    ids, times, values = sim._clamps[-1]
+    assert ids.tolist() == [3, 4] and times.tolist() == [10.0, 15.0, 20.0] and values.tolist() == [1.0, 2.0, 0.0]
+    # config.simulation_iclamp.csv.json: the file's rows as they are
+    sim.add_current_clamp({"input_type": "csv", "module": "IClamp", "node_set": {"population": "cortex"},
+                           "file": os.path.join(G, "point_iclamp", "iclamp_inputs_1.csv")})
+    _, times, values = sim._clamps[-1]
+    assert times.tolist() == [800.0, 1300.0, 1800.0, 2300.0, 2800.0, 3300.0]
+    assert values.tolist() == [0.15, 0.0, 0.175, 0.0, 0.2, 0.0]
+    with pytest.raises(ValueError):
+        sim.add_current_clamp({"input_type": "current_clamp", "node_set": [0], "amp": [1.0, 2.0], "delay": [5.0],
+                               "duration": [1.0]})
+    with pytest.raises(ValueError):
+        sim.add_current_clamp({"input_type": "current_clamp", "node_set": {"population": "thalamus"}, "amp": 1.0,
+                               "delay": 5.0, "duration": 1.0})
+    with pytest.raises(NotImplementedError):
+        sim.add_current_clamp({"input_type": "nwb", "node_set": [0], "file": "x.nwb", "sweep_id": 5})
+
+
+def test_current_segments_add_up_the_generators():
+    """An amplitude set for time t acts from the step that starts at t + dt; the generators on a node add up."""
+    sim = _bare_simulator(dt=0.5, tstop=50.0, n=4)
+    sim.add_current_clamp({"input_type": "current_clamp", "node_set": [0, 1], "amp": 10.0, "delay": 5.0,
+                           "duration": 10.0})
+    sim.add_current_clamp({"input_type": "current_clamp", "node_set": [1, 2], "amp": -4.0, "delay": 10.0,
+                           "duration": 30.0})
+    segs = [(a, b, cur.tolist()) for a, b, cur in sim._segments()]
+    assert segs == [(0, 11, [0, 0, 0, 0]), (11, 21, [10, 10, 0, 0]), (21, 31, [10, 6, -4, 0]),
+                    (31, 81, [0, -4, -4, 0]), (81, 100, [0, 0, 0, 0])]
