@@ -23,6 +23,10 @@ class Glif3Simulator:
     rec, inp    source-major synapse tables (numpy tuples, see bmtk_amd.network):
                 recurrent (rows = neurons) and external (rows = input sources)
     ring_slots  slots of the delay ring buffer; default = largest (residual) delay + 1
+    resident    "auto": every ``run`` is one cooperative launch that keeps the state in registers and the ring in
+                LDS (the resident kernel) whenever the network fits it -- batch 1, at most 1024 elements per
+                compute unit, ring slice within LDS; True: insist on it (ValueError otherwise); False: one launch
+                per step, which takes any batch and size
     pull        launch-per-step mode only: sum the recurrent arrivals of a step in one pass over a target-major
                 copy of the table from the spike-bit history, instead of pushing them into the ring with global
                 atomics as spikes occur -- the faster form for batched runs.  "auto": batch >= 8 (and delay_offset
