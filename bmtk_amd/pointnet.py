@@ -69,6 +69,39 @@ def _read_input_spikes(entry):
     raise NotImplementedError("spikes input module {!r} is not supported".format(module))
 
 
+def _read_nwb_stimulus(entry):
+    """Times (ms) and amplitudes of one sweep of an Allen Cell Types NWB file, as bmtk's NWBReader takes them
+    (bmtk/simulator/core/modules/iclamp.py:61-113): ``/epochs/Sweep_<id>/stimulus/timeseries/data`` times 1e9,
+    one value per 1000 / rate ms (attribute ``rate`` of ``starting_time``); ``downsample`` (ms) keeps every n-th
+    value, ``sweep_window`` [start, stop] ms cuts, ``delay`` shifts."""
+    from . import h5lite
+    sweep = entry["sweep_id"]
+    try:
+        sweep = "Sweep_{}".format(int(sweep))
+    except ValueError:
+        pass
+    with h5lite.File(entry["file"]) as h5:
+        if "/epochs" not in h5 or sweep not in h5["/epochs"].keys():
+            raise ValueError("{} missing sweep group {}.".format(entry["file"], sweep))
+        grp = h5["/epochs/{}/stimulus/timeseries".format(sweep)]
+        idt = 1000.0 / float(np.asarray(grp["starting_time"].attrs["rate"]).reshape(-1)[0])
+        amps = np.asarray(grp["data"][()], np.float64) * 1.0e9
+    delays = np.arange(amps.size) * idt
+    down = entry.get("downsample")
+    if down is not None and down > idt:
+        stride = int(np.round(down / idt))
+        amps, delays = amps[::stride], delays[::stride]
+    window = entry.get("sweep_window")
+    if window is not None:
+        if len(window) != 2 or window[0] >= window[1] or window[0] < 0:
+            raise ValueError('"sweep_window" parameter must be set to [start_time, stop_time] where '
+                             "0 <= start_time < stop_time.")
+        first = int(np.argwhere(delays >= window[0]).flatten()[0])
+        last = int(np.argwhere(delays <= window[1]).flatten()[-1]) + 1
+        amps, delays = amps[first:last], delays[first:last]
+    return (delays + float(entry.get("delay", 0.0))).tolist(), amps.tolist()
+
+
 class PointSimulator:
     def __init__(self, network, dt, tstop, device=None, resident="auto"):
         self.net, self.dt, self.tstop = network, float(dt), float(tstop)
@@ -142,7 +175,8 @@ class PointSimulator:
         bmtk/simulator/core/modules/iclamp.py:9-58).  ``input_type`` "current_clamp": ``amp`` (pA), ``delay``,
         ``duration`` (ms), scalars or lists of one length; an amplitude is switched off at delay + duration unless
         the next one has begun by then.  "csv": ``file`` with the columns ``timestamps`` and ``amps`` (other names
-        through ``timestamps_column`` / ``amplitudes_column``, ``separator`` " "), taken as they are.  Onsets at or
+        through ``timestamps_column`` / ``amplitudes_column``, ``separator`` " "), taken as they are; "nwb": one sweep of an
+        Allen Cell Types file (``file``, ``sweep_id``, optional ``downsample``, ``sweep_window``, ``delay``).  Onsets at or
         before the resolution are skipped, as bmtk does.  An amplitude set for time t acts on the update that
         starts at t + dt (NEST)."""
         kind = entry.get("input_type", "current_clamp")
@@ -161,6 +195,9 @@ class PointSimulator:
                     raise ValueError('csv file missing column "{}".'.format(col))
             delays = table[entry.get("timestamps_column", "timestamps")].to_numpy(np.float64).tolist()
             amps = table[entry.get("amplitudes_column", "amps")].to_numpy(np.float64).tolist()
+            durs = None
+        elif kind == "nwb":
+            delays, amps = _read_nwb_stimulus(entry)
             durs = None
         else:
             raise NotImplementedError("current clamp input_type {!r} is not supported".format(kind))

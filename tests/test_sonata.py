@@ -429,7 +429,34 @@ def test_current_clamp_amplitude_lists():
         sim.add_current_clamp({"input_type": "current_clamp", "node_set": {"population": "thalamus"}, "amp": 1.0,
                                "delay": 5.0, "duration": 1.0})
     with pytest.raises(NotImplementedError):
-        sim.add_current_clamp({"input_type": "nwb", "node_set": [0], "file": "x.nwb", "sweep_id": 5})
+        sim.add_current_clamp({"input_type": "movie", "node_set": [0]})
+
+
+def test_current_clamp_from_nwb_sweep(tmp_path):
+    """The stimulus of one sweep of an Allen Cell Types NWB file (bmtk/simulator/core/modules/iclamp.py:61-113): a
+    file of that layout written here, 20 kHz, a 0.5 nA step from 10 to 20 ms."""
+    data = np.zeros(800)
+    data[200:400] = 0.5e-9
+    path = str(tmp_path / "ephys.nwb")
+    h5lite.write(path, {"epochs": {"Sweep_55": {"stimulus": {"timeseries": {
+        "data": data, "starting_time": (np.float64(0.0), {"rate": np.float64(20000.0)})}}}}})
+    sim = _bare_simulator(dt=0.01, tstop=100.0, n=3)
+    sim.add_current_clamp({"input_type": "nwb", "module": "IClamp", "node_set": {"population": "cortex"},
+                           "file": path, "sweep_id": 55, "downsample": 0.1})
+    ids, times, values = sim._clamps[-1]
+    assert ids.tolist() == [0, 1, 2]
+    # every second sample (0.1 ms) except the first, whose onset is not after the resolution
+    np.testing.assert_allclose(times, np.arange(1, 400) * 0.1)
+    on = (times >= 10.0 - 1e-9) & (times < 20.0 - 1e-9)
+    np.testing.assert_allclose(values[on], 0.5)
+    assert on.sum() == 100 and np.all(values[~on] == 0.0)
+    sim.add_current_clamp({"input_type": "nwb", "node_set": [1], "file": path, "sweep_id": "55",
+                           "sweep_window": [5.0, 12.0], "delay": 100.0})
+    _, times, values = sim._clamps[-1]
+    np.testing.assert_allclose(times[[0, -1]], [105.0, 112.0])
+    assert values[0] == 0.0 and values[-1] == 0.5
+    with pytest.raises(ValueError):
+        sim.add_current_clamp({"input_type": "nwb", "node_set": [1], "file": path, "sweep_id": 7})
 
 
 def test_current_segments_add_up_the_generators():
