@@ -48,7 +48,8 @@ class Config(dict):
 
     @property
     def tstop(self):
-        return float(self["run"]["tstop"])
+        run = self["run"]  # "duration" goes before "tstop" (bmtk/simulator/pointnet/pointsimulator.py:218-221)
+        return float(run["duration"] if "duration" in run else run["tstop"])
 
 
 class PointNetwork(sonata.PointNetwork):
@@ -249,7 +250,10 @@ class PointSimulator:
                     cur[ids] += np.float32(on[-1])
             yield a, b, cur
 
-    def run(self, record_cap=None):
+    def run(self, tstop=None, record_cap=None):
+        if tstop is not None:
+            self.tstop = float(tstop)
+            self.n_steps = int(round(self.tstop / self.dt))
         nw = self.net
         rec, inp = nw.device_tables(self._device)
         sim = Glif3Simulator(nw.n, nw.par, self.dt, class_id=nw.class_id, rec=rec, inp=inp,
