@@ -9,6 +9,8 @@ seeded run produces the trains bmtk would write to ``inputs/*.h5``.
 bmtk hands it those trains (bmtk/simulator/pointnet/pointnetwork.py:39-61) and
 turns them into the per-step event lists the kernels consume.
 """
+import os
+
 import numpy as np
 
 
@@ -27,24 +29,23 @@ def _refractory_rate_correction(abs_ref, tau_ref):
     return float(np.max(after)), inverse
 
 
-class PoissonSpikeGenerator(object):
-    """Homogeneous / inhomogeneous Poisson spike trains (times stored in ms)."""
+class SpikeTrains(object):
+    """Spike trains of one or more populations in memory, with the calls of bmtk's ``SpikeTrains``
+    (bmtk/utils/reports/spike_trains/spike_trains_api.py:37-309): adding and querying spikes, SONATA/csv files,
+    and the comparisons ``==``, ``<=``, ``<`` (equal, subset, strict subset; per node, sorted times within
+    ``err``).  Times are kept in ms."""
 
-    def __init__(self, population=None, seed=None, output_units="ms", **kwargs):
+    def __init__(self, population=None, **kwargs):
         self.default_population = kwargs.get("default_population", population)
-        if seed:  # a seed of 0 / 0.0 / None leaves the global stream where it is, as the reference does
-            np.random.seed(seed)
-        units = output_units.lower()
-        if units in ("ms", "millisecond", "milliseconds"):
-            self.units, self.output_conversion = "ms", 1000.0
-        elif units in ("s", "second", "seconds"):
-            self.units, self.output_conversion = "s", 1.0
-        else:
-            raise AttributeError("Unknown output_units value {}".format(output_units))
+        self.units = "ms"
         self._trains = {}  # population -> {node_id: [chunks of times]}
 
     # -- container ---------------------------------------------------------
-    def add_spikes(self, node_ids, timestamps, population=None):
+    def add_spike(self, node_id, timestamp, population=None, **kwargs):
+        self.add_spikes(int(node_id), [timestamp], population)
+
+    def add_spikes(self, node_ids, timestamps, population=None, **kwargs):
+        """One node id with its times, or one id per time."""
         pop = population if population is not None else self.default_population
         store = self._trains.setdefault(pop, {})
         timestamps = np.atleast_1d(np.asarray(timestamps, np.float64))
@@ -75,6 +76,9 @@ class PoissonSpikeGenerator(object):
         pops = [population] if population is not None else self.populations
         return int(sum(sum(c.size for c in chunks) for p in pops for chunks in self._trains.get(p, {}).values()))
 
+    def __len__(self):
+        return self.n_spikes()
+
     def time_range(self, population=None):
         pops = [population] if population is not None else self.populations
         ts = np.concatenate([self.get_times(n, p) for p in pops for n in self.node_ids(p)])
@@ -94,6 +98,13 @@ class PoissonSpikeGenerator(object):
                            "population": rows_p, "node_ids": np.concatenate(rows_n) if rows_n else []})
         return df if with_population_col else df.drop(columns="population")
 
+    def spikes(self, populations=None):
+        """Iterates (timestamp, population, node id)."""
+        for p in (self.populations if populations is None else np.atleast_1d(populations).tolist()):
+            for n in self.node_ids(p):
+                for t in self.get_times(n, p):
+                    yield float(t), p, int(n)
+
     def _as_spikes(self):
         out = {}
         for p in self.populations:
@@ -103,6 +114,7 @@ class PoissonSpikeGenerator(object):
                       else np.zeros(0, np.int64), np.concatenate(ts) if ts else np.zeros(0))
         return out
 
+    # -- files ---------------------------------------------------------------
     def to_sonata(self, path, mode="w", sort_order="none", **kwargs):
         """``/spikes/<population>/{node_ids,timestamps}`` as bmtk/utils/reports/spike_trains/spike_trains_api.py:147-158
         writes them; the file is stored uncompressed whatever ``compression`` asks."""
@@ -116,6 +128,85 @@ class PoissonSpikeGenerator(object):
         if mode != "w":
             raise NotImplementedError("to_csv only writes a new file")
         sonata.write_spikes_csv(path, self._as_spikes(), sort_order=getattr(sort_order, "value", sort_order))
+
+    @classmethod
+    def _from_spikes(cls, spikes, **kwargs):
+        st = cls(**kwargs)
+        for pop, entry in spikes.items():
+            ids, ts = np.asarray(entry[0]), np.asarray(entry[1], np.float64)
+            order = np.argsort(ids, kind="stable")
+            ids, ts = ids[order], ts[order]
+            uniq, first = np.unique(ids, return_index=True)
+            store = st._trains.setdefault(pop, {})
+            for u, a, b in zip(uniq, first, list(first[1:]) + [ids.size]):
+                store[int(u)] = [ts[a:b]]
+        return st
+
+    @classmethod
+    def from_sonata(cls, path, population=None, **kwargs):
+        from . import sonata
+        return cls._from_spikes(sonata.read_spikes(path, None if population is None else np.atleast_1d(population)),
+                                **kwargs)
+
+    @classmethod
+    def from_csv(cls, path, **kwargs):
+        from . import sonata
+        return cls._from_spikes(sonata.read_spikes_csv(path), **kwargs)
+
+    @classmethod
+    def load(cls, path, file_type=None, **kwargs):
+        """By extension (or ``file_type`` "h5"/"sonata"/"csv"), as spike_trains.py:46-73 does."""
+        kind = (file_type or os.path.splitext(path)[1].lstrip(".")).lower()
+        if kind in ("h5", "hdf5", "sonata"):
+            return cls.from_sonata(path, **kwargs)
+        if kind in ("csv", "txt"):
+            return cls.from_csv(path, **kwargs)
+        raise ValueError("cannot tell the type of spikes file {}".format(path))
+
+    # -- comparisons -----------------------------------------------------------
+    def is_equal(self, other, err=0.00001):
+        from . import sonata
+        return sonata.spikes_equal(self._as_spikes(), other._as_spikes(), err=err)
+
+    def is_subset(self, other, err=0.00001, strict=False):
+        from . import sonata
+        return sonata.spikes_is_subset(self._as_spikes(), other._as_spikes(), err=err, strict=strict)
+
+    def __eq__(self, other):
+        return self.is_equal(other)
+
+    def __ne__(self, other):
+        return not self == other
+
+    def __lt__(self, other):
+        return self.is_subset(other, strict=True)
+
+    def __le__(self, other):
+        return self.is_subset(other)
+
+    def __gt__(self, other):
+        return other < self
+
+    def __ge__(self, other):
+        return other <= self
+
+    __hash__ = None
+
+
+class PoissonSpikeGenerator(SpikeTrains):
+    """Homogeneous / inhomogeneous Poisson spike trains (times stored in ms)."""
+
+    def __init__(self, population=None, seed=None, output_units="ms", **kwargs):
+        super().__init__(population=population, **kwargs)
+        if seed:  # a seed of 0 / 0.0 / None leaves the global stream where it is, as the reference does
+            np.random.seed(seed)
+        units = output_units.lower()
+        if units in ("ms", "millisecond", "milliseconds"):
+            self.units, self.output_conversion = "ms", 1000.0
+        elif units in ("s", "second", "seconds"):
+            self.units, self.output_conversion = "s", 1.0
+        else:
+            raise AttributeError("Unknown output_units value {}".format(output_units))
 
     # -- generators --------------------------------------------------------
     def add(self, node_ids, firing_rate, population=None, times=(0.0, 1.0), abs_ref=0, tau_ref=0):

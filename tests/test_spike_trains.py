@@ -105,3 +105,32 @@ def test_binning_to_step_events():
     # off-grid times are carried to the end of their step; on-grid times stay put
     in_ptr, ev = bin_spike_times([[0.2, 1.0, 1.01]], dt=1.0, n_steps=4)
     assert in_ptr.tolist() == [0, 2, 3, 3, 3]
+
+
+def test_equals_and_subset_operators(tmp_path):
+    """bmtk/tests/utils/reports/spike_trains/test_spikes_core.py:47-78."""
+    from bmtk_amd.spike_trains import SpikeTrains
+    st1 = SpikeTrains()
+    st1.add_spikes(node_ids=0, population="V1", timestamps=[0.1, 0.2, 0.3, 0.4])
+    st1.add_spikes(node_ids=1, population="V1", timestamps=[1.0])
+    st2 = SpikeTrains()
+    st2.add_spikes(node_ids=1, population="V1", timestamps=[1.0])
+    st2.add_spikes(node_ids=0, population="V1", timestamps=[0.3, 0.2, 0.1, 0.4])
+    assert st1 == st2 and st1 <= st2 and st1 >= st2 and not st1 != st2
+    st2 = SpikeTrains()
+    st2.add_spikes(node_ids=1, population="V1", timestamps=[1.0])
+    st2.add_spikes(node_ids=0, population="V1", timestamps=[0.3, 0.2, 0.1, 0.4, 0.5])
+    st2.add_spike(node_id=2, population="V1", timestamp=0.5)
+    st2.add_spikes(node_ids=0, population="V2", timestamps=np.linspace(0.0, 1.0, 11))
+    assert st1 != st2 and st1 < st2 and st2 > st1 and st1 <= st2 and st2 >= st1
+    assert len(st2) == 18 and st2.n_spikes("V2") == 11 and sorted(st2.populations) == ["V1", "V2"]
+    # through the two file formats and back
+    for name in ("s.h5", "s.csv"):
+        path = str(tmp_path / name)
+        (st2.to_sonata if name.endswith("h5") else st2.to_csv)(path, sort_order="by_time")
+        back = SpikeTrains.load(path)
+        assert back == st2 and set(back.node_ids("V1")) == {0, 1, 2}
+        assert len(list(back.spikes())) == 18
+    assert SpikeTrains.from_sonata(str(tmp_path / "s.h5"), population="V2").populations == ["V2"]
+    with pytest.raises(ValueError):
+        SpikeTrains.load(str(tmp_path / "s.xyz"))
