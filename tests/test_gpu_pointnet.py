@@ -142,6 +142,31 @@ def test_current_clamp_segments(tmp_path):
     assert len(got & want) / max(1, len(got | want)) >= 0.999
 
 
+def test_current_clamp_from_csv_equals_the_list_form(tmp_path):
+    """The same stimulus given as a csv file of amplitude changes and as amp/delay/duration lists: same spikes;
+    the clamp goes to the whole population (no node ids in the node set)."""
+    dt, tstop = 0.1, 200.0
+    csv = str(tmp_path / "stim.csv")
+    with open(csv, "w") as fh:
+        fh.write("timestamps amps\n20.0 300.0\n60.0 0.0\n100.0 450.0\n150.0 0.0\n")
+    forms = ({"input_type": "csv", "module": "IClamp", "node_set": {"population": "v1"}, "file": csv},
+             {"input_type": "current_clamp", "module": "IClamp", "node_set": {"population": "v1"},
+              "amp": [300.0, 450.0], "delay": [20.0, 100.0], "duration": [40.0, 50.0]})
+    got = []
+    for k, form in enumerate(forms):
+        os.makedirs(str(tmp_path / str(k)))
+        conf = pointnet.Config.from_json(_write_configs(str(tmp_path / str(k)), dt, tstop, {"clamp": form}))
+        del conf["inputs"]["LGN_spikes"]
+        graph = pointnet.PointNetwork.from_config(conf, unsupported="silence")
+        sim = pointnet.PointSimulator.from_config(conf, graph)
+        assert [(a, b) for a, b, _ in sim._segments()] == [(0, 201), (201, 601), (601, 1001), (1001, 1501),
+                                                            (1501, 2000)]
+        got.append(sim.run()["v1"])
+    assert got[0][0].size > 300
+    assert np.array_equal(got[0][0], got[1][0]) and np.array_equal(got[0][1], got[1][1])
+    assert got[0][1].min() > 20.0
+
+
 def test_example_at_its_own_resolution(tmp_path):
     """The example's configured resolution, dt = 0.001 ms: its 2 ms delays are 2000 steps, far beyond the ring,
     so the run rests on the delay offset (1999 steps) and a ring of 2 slots.  200 ms = 200,000 steps, resident
