@@ -4,11 +4,18 @@
 Workload (N=1): the V1-scale forward simulation -- 230,924 GLIF3 neurons in 111
 parameter classes, lognormal in-degree with mean 300 (~70 M recurrent
 synapses), 17,400 Poisson inputs at 5 Hz through ~8 M input synapses, 4
-receptors, delays 1-5 steps, dt = 1 ms, batch 1.  One "step" is one simulation
-step (1 ms) of the whole network; --steps defaults to the configuration's 3000.
+receptors, delays 1-5 steps, dt = 1 ms, batch 1, 3000 simulation steps.
+
+One "step" of this benchmark (--steps K, --warmup W) is one PASS of the hot
+path over that workload: one call of the forward simulation over 3000
+simulation steps of 1 ms, i.e. what one ``nest.Simulate(3000.0)`` is for the
+reference (bmtk/simulator/pointnet/pointsimulator.py:159-166).  Before the
+warm-up passes the network runs untimed until it has left the transient from
+rest (at least 400 steps), so every timed pass sees the settled activity
+(~2.8 Hz, ~230 k synaptic events per simulation step) whatever K and W are.
 Recurrent weights are lognormal(0,1) pA signed by the source class as
 specified; input weights are scaled by 7 because at 1 pA the network stays
-silent and there would be no synaptic events to count (it settles at ~3 Hz).
+silent and there would be no synaptic events to count.
 
 Prints ONE JSON line: value = neuron-updates/s of the whole job; synaptic
 events/s, the roofline of the dominant kernel, the isolated state-update and
@@ -17,6 +24,7 @@ propagation kernels, and the CPU baseline ride along in the same object.
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -30,12 +38,22 @@ B_PER_EVENT = 18               # 4 index + 4 weight + 1 delay + 1 receptor + 8 r
 
 N_V1, N_IN, MEAN_IN, N_IN_SYN, N_CLASSES = 230924, 17400, 300, 8_000_000, 111
 IN_RATE_HZ, IN_W_SCALE = 5.0, 7.0
-# HBM bytes per simulated step of the headline workload from rocprofv3 FETCH_SIZE / WRITE_SIZE counter
-# runs (summaries under profiles/; one FETCH_SIZE count = 2 KiB, one WRITE_SIZE count = 1 KiB by the
-# 1 GiB copy calibration).  Measured at the default operating point; not re-measured by this script.
-TRAFFIC_BYTES_PER_STEP = {"resident": 4.07e6 + 0.20e6, "per_step": 18.8e6 + 22.0e6}
-TRAFFIC_STATE_UPDATE_1M = 176.2e6 + 51.4e6   # glif3_step_kernel, per launch
-TRAFFIC_PULL_52K_B64 = 455e6 + 53.2e6        # pull_kernel, per launch, pooled over the three rates
+SIM_STEPS = 3000               # simulation steps of one pass (the configuration's run length)
+SETTLE_STEPS, SETTLE_MAX_STEPS = 400, 2000
+CPU_MIN_STEPS = 200
+
+
+def profile_traffic(file_name, key):
+    """HBM bytes from a committed rocprofv3 counter summary: the value of the line ``TRAFFIC <key> = <number>``
+    in profiles/<file_name> (written there from the FETCH_SIZE / WRITE_SIZE runs the file describes), or None
+    when the file or the line is missing.  These are constants of those profile runs; this script does not
+    re-measure them."""
+    try:
+        txt = open(os.path.join(ROOT, "profiles", file_name)).read()
+    except OSError:
+        return None
+    m = re.search(r"^TRAFFIC\s+%s\s*=\s*([0-9.eE+-]+)" % re.escape(key), txt, flags=re.M)
+    return float(m.group(1)) if m else None
 
 
 def build_v1(torch, steps_total, resident="auto"):
@@ -76,29 +94,44 @@ def time_region(torch, fn):
 
 
 def bench_state_update(torch, steps=1000, warmup=50):
-    """Isolated fused state update: N = 1,048,576, per-neuron parameters,
-    Gaussian(0, 50 pA) currents from a pool of 8 pre-generated vectors."""
+    """Isolated fused state update: N = 1,048,576, Gaussian(0, 50 pA) currents from a pool of 8 pre-generated
+    vectors, in two forms: parameters from a table of 111 classes (the form the V1-scale simulation uses:
+    101 B of state, current and flag plus the 2 B class id per update) and per-neuron parameters (29
+    propagator words more per update)."""
     import numpy as np
     from bmtk_amd import ops, synthetic
     n = 1 << 20
-    rng = np.random.default_rng(1)
-    par = synthetic.random_cells(rng, n)
-    prop = ops.glif3_precompute(par, 1.0)
-    st = ops.Glif3State.from_numpy(synthetic.random_state(rng, par, n, 1))
-    pool = [torch.randn(n, device="cuda") * 50.0 for _ in range(8)]
-    z = torch.zeros(n, dtype=torch.uint8, device="cuda")
-    for k in range(warmup):
-        ops.glif3_step_fwd(st, prop, 1.0, i_ext=pool[k % 8], z=z)
-    wall, dev = time_region(torch, lambda: [ops.glif3_step_fwd(st, prop, 1.0, i_ext=pool[k % 8], z=z)
-                                            for k in range(steps)])
-    per = dev / steps
-    # per-neuron parameters: 29 propagator words are read per update on top of the 101 B
-    alg = n * (B_PER_UPDATE_PLAIN + 29 * 4)
-    return {"kernel": "glif3_step_kernel", "workload": "state update N=1048576, per-neuron parameters, 1000 steps",
-            "neuron_updates_per_s": n / per, "us_per_launch": per * 1e6,
-            "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": TRAFFIC_STATE_UPDATE_1M},
-            "bytes_per_update": B_PER_UPDATE_PLAIN + 29 * 4}
+    out = []
+    for form in ("class table", "per-neuron parameters"):
+        rng = np.random.default_rng(1)
+        if form == "class table":
+            par = synthetic.random_cells(rng, N_CLASSES)
+            cid_h = rng.integers(0, N_CLASSES, n).astype(np.int32)
+            cid = torch.as_tensor(cid_h, device="cuda")
+            per_update = B_PER_UPDATE_CLASS
+            key = "hbm_bytes_per_launch_class_table"
+        else:
+            par = synthetic.random_cells(rng, n)
+            cid_h = cid = None
+            per_update = B_PER_UPDATE_PLAIN + 29 * 4
+            key = "hbm_bytes_per_launch"
+        prop = ops.glif3_precompute(par, 1.0)
+        st = ops.Glif3State.from_numpy(synthetic.random_state(rng, par, n, 1, class_id=cid_h))
+        pool = [torch.randn(n, device="cuda") * 50.0 for _ in range(8)]
+        z = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        for k in range(warmup):
+            ops.glif3_step_fwd(st, prop, 1.0, class_id=cid, i_ext=pool[k % 8], z=z)
+        wall, dev = time_region(torch, lambda: [ops.glif3_step_fwd(st, prop, 1.0, class_id=cid, i_ext=pool[k % 8], z=z)
+                                                for k in range(steps)])
+        per = dev / steps
+        alg = n * per_update
+        out.append({"kernel": "glif3_step_kernel", "workload": "state update N=1048576, %s, %d steps" % (form, steps),
+                    "neuron_updates_per_s": n / per, "us_per_launch": per * 1e6,
+                    "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": alg / per / 1e9 / HBM_PEAK_GBS,
+                                 "traffic": profile_traffic("glif3_step_kernel_state_update_1M.txt", key)},
+                    "bytes_per_update": per_update})
+    return out
 
 
 def bench_compaction(torch, steps=200, warmup=20):
@@ -182,7 +215,8 @@ def bench_propagation(torch, steps=200, warmup=20):
                         "us_per_launch": per * 1e6,
                         "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS,
                                      "unit": "GB/s", "frac": alg / per / 1e9 / HBM_PEAK_GBS,
-                                     "traffic": TRAFFIC_PULL_52K_B64 if mode == "pull" else None}})
+                                     "traffic": profile_traffic("propagation_kernels_52k_batch64.txt",
+                                                                "hbm_bytes_per_launch_" + mode)}})
     return out
 
 
@@ -234,10 +268,10 @@ def bench_bptt(torch, steps=600):
             "grad_norm_rec": float(bptt.d_rec_w.norm().item()), "grad_norm_inp": float(bptt.d_inp_w.norm().item())}
 
 
-def cpu_baseline(torch, sim, par, class_id, sample_steps):
-    """The NEST-algorithm CPU restatement (fp64, event-driven source-major
-    delivery into per-neuron ring buffers, OpenMP) on the first `sample_steps`
-    steps of the same network, from rest."""
+def cpu_baseline(torch, sim, par, class_id, settled, sample_steps):
+    """The NEST-algorithm CPU restatement (fp64, event-driven source-major delivery into per-neuron ring
+    buffers, OpenMP) on `sample_steps` steps of the same network, started from the settled state the GPU's
+    timed region started from (copied to the host), so that it sees the same activity."""
     import numpy as np
     from oracle import glif3_oracle as orc
     rec = tuple(t.cpu().numpy() for t in (sim.rec.indptr, sim.rec.indices, sim.rec.weights, sim.rec.delays,
@@ -247,35 +281,73 @@ def cpu_baseline(torch, sim, par, class_id, sample_steps):
     in_ptr = sim.in_ptr.cpu().numpy()
     in_ev = sim.in_events.cpu().numpy()
     prop = orc.precompute(par, 1.0)
+    step0 = settled["step"]
     res = {}
-    for label, threads, steps in (("all", orc.max_threads(), sample_steps), ("one", 1, max(20, sample_steps // 3))):
+    for label, threads, steps in (("all", orc.max_threads(), sample_steps), ("one", 1, max(CPU_MIN_STEPS, sample_steps // 10))):
         orc.set_threads(threads)
-        st = orc.new_state(N_V1, 1, np.float64)
-        ring = np.zeros((sim.L, 4, N_V1))
+        st = {k: np.ascontiguousarray(v, np.int32 if k == "ref" else np.float64) for k, v in settled["state"].items()}
+        ring = np.ascontiguousarray(settled["ring"], np.float64)
         t0 = time.perf_counter()
         out = orc.simulate(st, prop, 1.0, steps, class_id=class_id, ring=ring, rec=rec, inp=inp, in_ptr=in_ptr,
-                           in_events=in_ev, spike_cap=steps * N_V1 // 16)
+                           in_events=in_ev, spike_cap=max(1024, steps * N_V1 // 16), step0=step0)
         dt = time.perf_counter() - t0
         deg = np.diff(rec[0])
-        ev = int(deg[out["elem"]].sum()) + int(np.diff(inp[0])[in_ev[:in_ptr[steps]]].sum())
+        ev = int(deg[out["elem"]].sum()) + int(np.diff(inp[0])[in_ev[in_ptr[step0]:in_ptr[step0 + steps]]].sum())
         res[label] = dict(threads=threads, steps=steps, seconds=dt, updates_per_s=N_V1 * steps / dt,
-                          events_per_s=ev / dt)
+                          events_per_s=ev / dt, rate_hz=out["count"] / (N_V1 * steps * 1e-3))
     orc.set_threads(res["all"]["threads"])
     a, o = res["all"], res["one"]
     return {"value": a["updates_per_s"], "unit": "neuron-updates/s", "cores": a["threads"], "kind": "port",
-            "sample": "first %d steps of the same 230,924-neuron network from rest (%.1f s); NEST-algorithm "
-                      "restatement in C, fp64, OpenMP, not NEST" % (a["steps"], a["seconds"]),
+            "sample": "%d steps of the same 230,924-neuron network from the settled state the GPU run was timed "
+                      "from (%.1f s, %.2f Hz mean rate); NEST-algorithm restatement in C, fp64, OpenMP, not NEST"
+                      % (a["steps"], a["seconds"], a["rate_hz"]),
             "synaptic_events_per_s": a["events_per_s"],
             "one_thread": {"value": o["updates_per_s"], "synaptic_events_per_s": o["events_per_s"],
                            "steps": o["steps"], "seconds": o["seconds"]},
             "host_cpu_count": os.cpu_count()}
 
 
+def settle(torch, sim, min_steps=SETTLE_STEPS, max_steps=SETTLE_MAX_STEPS, block=100):
+    """Run the network, untimed, until it has left the transient from rest: at least `min_steps` steps and
+    then until the spike count of a block of 100 steps lies within 10 % of the mean of the three blocks before it
+    (or `max_steps`).  Returns the number of steps taken."""
+    from bmtk_amd import training
+    counts, done = [], 0
+    while done < max_steps:
+        out = sim.run(block)
+        counts.append(int(training.spike_counts(out["bits"], sim.ne).sum().item()))
+        done += block
+        if done >= min_steps and len(counts) >= 4:
+            prev = sum(counts[-4:-1]) / 3.0
+            if prev > 0 and abs(counts[-1] - prev) <= 0.1 * prev:
+                break
+    sim.check()
+    return done, counts
+
+
+def launch_overhead(torch, sim, n1=100, n2=1100, reps=3):
+    """Fixed cost of one `bmtk_glif3_simulate_fwd` call as the intercept of two run lengths (HIP events, best
+    of `reps`): (seconds per step at the margin, fixed seconds per call)."""
+    best = {}
+    for n in (n1, n2):
+        ts = []
+        for _ in range(reps):
+            _, dev = time_region(torch, lambda: sim.run(n, spike_bits=False))
+            ts.append(dev)
+        best[n] = min(ts)
+    slope = (best[n2] - best[n1]) / (n2 - n1)
+    return slope, best[n1] - slope * n1
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=3000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=5,
+                    help="timed passes; one pass = one call of the forward simulation over --sim-steps steps of "
+                         "1 ms (what one nest.Simulate(tstop) does for the reference)")
+    ap.add_argument("--warmup", type=int, default=1, help="untimed passes before the timed ones")
+    ap.add_argument("--sim-steps", type=int, default=SIM_STEPS,
+                    help="simulation steps per pass (the configuration's 3000)")
     ap.add_argument("--cpu-steps", type=int, default=3000, help="steps of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the isolated-kernel measurements")
     ap.add_argument("--kernels", default="state,compaction,propagation,bptt",
@@ -292,7 +364,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
-    from bmtk_amd import _lib
+    from bmtk_amd import _lib, training
     _lib.load()
     if args.calibrate_copy:
         src = torch.ones(1 << 28, device="cuda")       # 1 GiB of fp32
@@ -303,53 +375,84 @@ def main():
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "copies": 10}))
         return
 
-    K, W = args.steps, args.warmup
-    sim, par, class_id = build_v1(torch, W + K, resident=False if args.per_step else "auto")
-    sim.run(W, spike_bits=False)
-    res = {}
-    wall, dev = time_region(torch, lambda: res.update(sim.run(K)))
-    bits = res["bits"]
-    rec_ev, in_ev = count_events(torch, sim, bits, W)
-    events = rec_ev + in_ev
-    n_spikes = int(sim.raster(bits[::10]).sum().item()) * 10 if K >= 10 else 0
+    K, W, S = args.steps, args.warmup, args.sim_steps
+    if K < 1 or W < 0 or S < 1:
+        sys.exit("bench.py: --steps and --sim-steps must be positive, --warmup non-negative")
+    if K * S * ((N_V1 + 63) // 64) * 8 > 100e9:
+        sys.exit("bench.py: --steps x --sim-steps spike bits would exceed 100 GB; use fewer passes")
+    overhead_steps = 3 * (100 + 1100)
+    sim, par, class_id = build_v1(torch, SETTLE_MAX_STEPS + (W + K) * S + overhead_steps,
+                                  resident=False if args.per_step else "auto")
+    # untimed: leave the transient from rest behind, whatever --warmup says
+    settled_steps, settle_counts = settle(torch, sim)
+    torch.cuda.synchronize()
+    settled = {"step": sim.step, "state": sim.state.to_numpy(), "ring": sim.ring.cpu().numpy()}
+    for _ in range(W):
+        sim.run(S, spike_bits=False)
+    step_timed = sim.step
+    passes = []
+    wall, dev = time_region(torch, lambda: [passes.append(sim.run(S)) for _ in range(K)])
     sim.check()
+    rec_ev = in_ev = n_spikes = 0
+    for k, out in enumerate(passes):
+        r, i = count_events(torch, sim, out["bits"], step_timed + k * S)
+        rec_ev, in_ev = rec_ev + r, in_ev + i
+        n_spikes += int(training.spike_counts(out["bits"], sim.ne).sum().item())
+        out["bits"] = None
+    events = rec_ev + in_ev
+    total_steps = K * S
     resident = bool(sim.res_span)
-    # resident mode: the timed region is ONE launch of sim_resident_kernel covering all K steps;
-    # otherwise K+1 launches of sim_step_kernel
-    launches = 1 if resident else K + 1
+    # resident mode: every pass is ONE launch of sim_resident_kernel covering its S steps;
+    # otherwise S+1 launches of sim_step_kernel per pass
+    launches = K if resident else K * (S + 1)
     per_launch = dev / launches
-    alg_step = N_V1 * B_PER_UPDATE_CLASS + events / K * B_PER_EVENT
-    alg = alg_step * K / launches
+    alg_step = N_V1 * B_PER_UPDATE_CLASS + events / total_steps * B_PER_EVENT
+    alg = alg_step * total_steps / launches
+    slope, fixed = launch_overhead(torch, sim)
+    sim.check()
+    traffic_step = profile_traffic("sim_resident_kernel_v1_forward_230k.txt" if resident else
+                                   "sim_step_kernel_v1_forward_230k_per_step_launches.txt", "hbm_bytes_per_step")
     line = {
         "metric": "neuron-updates/s (with synaptic events/s) at 230k neurons; % of HBM roofline",
-        "value": N_V1 * K / wall, "unit": "neuron-updates/s",
+        "value": N_V1 * total_steps / wall, "unit": "neuron-updates/s",
         "synaptic_events_per_s": events / wall,
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall / K * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "V1-scale forward simulation: 230,924 GLIF3 neurons, 111 classes, %d recurrent + %d "
-                               "input synapses, 17,400 Poisson inputs at 5 Hz, dt 1 ms, batch 1" %
-                               (sim.rec.nnz, sim.inp.nnz),
-                   "mode": "resident (one cooperative launch)" if resident else "one launch per step",
-                   "mean_rate_hz": n_spikes / (N_V1 * K * 1e-3) if K else 0.0,
-                   "recurrent_events": rec_ev, "input_events": in_ev, "input_weight_scale": IN_W_SCALE},
+                               "input synapses, 17,400 Poisson inputs at 5 Hz, dt 1 ms, batch 1, %d simulation steps "
+                               "per pass" % (sim.rec.nnz, sim.inp.nnz, S),
+                   "step_definition": "one pass = one forward-simulation call over %d steps of 1 ms (one "
+                                      "nest.Simulate(tstop) of the reference); --steps counts passes" % S,
+                   "sim_steps_per_pass": S, "sim_steps_timed": total_steps,
+                   "settle_steps_untimed": settled_steps, "settle_spikes_per_100_steps": settle_counts[-4:],
+                   "mode": "resident (one cooperative launch per pass)" if resident else "one launch per step",
+                   "mean_rate_hz": n_spikes / (N_V1 * total_steps * 1e-3),
+                   "spikes": n_spikes, "recurrent_events": rec_ev, "input_events": in_ev,
+                   "events_per_sim_step": events / total_steps, "us_per_sim_step": wall / total_steps * 1e6,
+                   "input_weight_scale": IN_W_SCALE},
         "roofline": {"bound": "hbm", "kernel": "sim_resident_kernel" if resident else "sim_step_kernel",
                      "achieved": alg / per_launch / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": alg / per_launch / 1e9 / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC_BYTES_PER_STEP["resident" if resident else "per_step"] * K / launches,
+                     "traffic": None if traffic_step is None else traffic_step * total_steps / launches,
+                     "traffic_source": "profiles/ (rocprofv3 FETCH_SIZE + WRITE_SIZE summary; a constant of that "
+                                       "profile run, not re-measured here)",
                      "launches": launches, "algorithmic_bytes_per_launch": alg, "us_per_launch": per_launch * 1e6,
-                     "algorithmic_bytes_per_step": alg_step, "us_per_step": dev / K * 1e6},
+                     "algorithmic_bytes_per_step": alg_step, "us_per_step": dev / total_steps * 1e6,
+                     "launch_overhead_us": fixed * 1e6, "marginal_us_per_step": slope * 1e6,
+                     "frac_at_the_margin": alg_step / slope / 1e9 / HBM_PEAK_GBS},
     }
     if not args.no_kernels:
         want = set(args.kernels.split(","))
         unknown = want - {"state", "compaction", "propagation", "bptt"}
         if unknown:
             sys.exit("bench.py: unknown --kernels entries: %s" % ", ".join(sorted(unknown)))
-        line["kernels"] = (([bench_state_update(torch)] if "state" in want else []) +
+        del passes
+        line["kernels"] = ((bench_state_update(torch) if "state" in want else []) +
                            (bench_compaction(torch) if "compaction" in want else []) +
                            (bench_propagation(torch) if "propagation" in want else []) +
                            ([bench_bptt(torch)] if "bptt" in want else []))
     if args.cpu_steps > 0:
-        line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, min(args.cpu_steps, W + K))
+        line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, settled, max(CPU_MIN_STEPS, args.cpu_steps))
     print(json.dumps(line))
 
 
