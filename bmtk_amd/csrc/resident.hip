@@ -127,7 +127,6 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
     for (uint32_t p = lo + (uint32_t)kTogether; p < hi; ++p) add(rows[p]);
 }
 
-constexpr int kActCap = 8192;   // active-row list in LDS (entries)
 constexpr int kScanWords = 4;   // ballot words per thread and round
 constexpr unsigned kInputTag = 0x80000000u;
 
@@ -256,6 +255,12 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     unsigned *act = reinterpret_cast<unsigned *>(ring_l + s.ring_slots * GLIF3_NREC * r.span);
     unsigned *abort_word = s.res_sync + 1;
     unsigned *arrivals = s.res_sync + kBarrierStride;  // [kBarrierWords] counters, kBarrierStride words apart
+    // a run before this one gave up and nobody has looked yet: do nothing, so that the failure is still there to see
+    // (one thread looks for the whole workgroup, so that all of its threads take the same way)
+    if (tid == 0) go_on = load_agent(abort_word) == 0u;
+    __syncthreads();
+    if (!go_on) return;
+    __syncthreads();  // go_on is written again in the loop
 
     for (int c = tid; c < L * GLIF3_NREC * span; c += kResBlock) {
         const int dr = c / span, i = c - dr * span;
@@ -493,7 +498,8 @@ __global__ void zero_words_kernel(unsigned *w, int n)
 // abort flag and arrival counters of a resident run
 __global__ void zero_sync_kernel(unsigned *sync)
 {
-    if (threadIdx.x < 2) sync[threadIdx.x] = 0u;
+    // word 1, the abort flag, is left alone: it stays set until the host has read and cleared it
+    if (threadIdx.x == 0) sync[0] = 0u;
     for (int c = threadIdx.x; c < kWays * kBarrierWords; c += blockDim.x) sync[(1 + c) * kBarrierStride] = 0u;
 }
 

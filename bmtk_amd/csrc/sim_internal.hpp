@@ -5,6 +5,10 @@
 
 namespace bmtk {
 
+constexpr int kActCap = 8192;                                   // active-row list of the resident kernel (entries)
+constexpr size_t kResLdsBytes = 160u * 1024u;                   // LDS of one gfx950 compute unit
+constexpr size_t kResLdsExtra = kActCap * sizeof(int) + 256u;   // the list plus the kernel's static LDS (rounded up)
+
 // Whole run as one cooperative launch with state in registers and the ring in
 // LDS (resident.hip).  Arguments have been validated by the caller.
 int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream);

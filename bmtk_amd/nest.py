@@ -504,6 +504,7 @@ def Simulate(t_ms):
             # interpolated threshold crossing (step + fraction) * resolution
             times.append(((st + fr) * dt)[order])
             senders.append(s["neuron_ids"][el[order]])
+    sim.check()  # also without a recorder: Simulate returns only after the run is known to be valid
     s["steps_done"] = step0 + n_steps
     _S.status["biological_time"] = s["steps_done"] * dt
     for m, (a_s, a_t, a_v) in mm_rows.items():

@@ -100,3 +100,27 @@ def check_csr(csr, n_rows, n_cols, ring_slots):
             raise ValueError("delays must lie in 1..{} steps for a ring of {} slots".format(ring_slots - 1, ring_slots))
         if r.max() >= NREC:
             raise ValueError("receptor outside 0..{}".format(NREC - 1))
+
+
+def check_input_events(in_ptr, in_events, n_ids):
+    """Host-side validation of per-step input event lists (``in_events[in_ptr[t]:in_ptr[t+1]]`` are the
+    element ids source*batch+trial emitted in step t): ``in_ptr`` non-decreasing from 0 to the number of
+    events, ids within 0..n_ids-1 and ascending within every step (the input-weight gradient kernel gives a
+    source's run of events one writer and relies on the order).  Returns True when some id occurs more than
+    once within a step -- two spikes of one generator inside one resolution step, which NEST delivers both;
+    such lists must stay on the event-list form of the delivery."""
+    in_ptr = np.asarray(in_ptr)
+    in_events = np.asarray(in_events)
+    if in_ptr.size < 1 or in_ptr[0] != 0 or np.any(np.diff(in_ptr) < 0) or in_ptr[-1] != in_events.size:
+        raise ValueError("in_ptr must be non-decreasing from 0 to len(in_events)")
+    if in_events.size and (in_events.min() < 0 or in_events.max() >= n_ids):
+        raise ValueError("input event id outside 0..n_inputs*batch-1")
+    if in_events.size < 2:
+        return False
+    step_start = np.zeros(in_events.size + 1, bool)
+    step_start[in_ptr] = True                 # an event that opens a step may be smaller than the one before it
+    d = np.diff(in_events.astype(np.int64))
+    inside = ~step_start[1:-1]
+    if np.any((d < 0) & inside):
+        raise ValueError("input events must be ascending within every step")
+    return bool(np.any((d == 0) & inside))

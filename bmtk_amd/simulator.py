@@ -15,6 +15,25 @@ from .layout import NPARAM, NPROP, NREC
 from .ops import Glif3State, SpikeCompactor, SynapseTable, _dev, _p, _stream, glif3_precompute, n_words, unpack_bits
 
 
+RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
+RES_ACT_ENTRIES = 8192          # active-row list of the resident kernel (kActCap of csrc/resident.hip), 4 B each
+RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static LDS (rounded up)
+
+
+def resident_span(ne, batch, ring_slots, n_cu):
+    """Elements per workgroup of the resident kernel for a network of ``ne`` elements on ``n_cu`` compute
+    units, or 0 when the network does not fit: batch 1, one workgroup per compute unit (rounded down to a
+    multiple of 8), at most 1024 elements each, and ring slice + active-row list + static LDS within the
+    compute unit's LDS.  ``bmtk_glif3_simulate_fwd`` applies the same bound."""
+    cus = n_cu - n_cu % 8
+    if batch != 1 or cus <= 0 or ne <= 0:
+        return 0
+    span = -(-(-(-ne // cus)) // 64) * 64
+    if span > 1024 or ring_slots * NREC * span * 4 + RES_LDS_EXTRA > RES_LDS_BYTES:
+        return 0
+    return span
+
+
 class Glif3Simulator:
     """A population of GLIF3 neurons with recurrent and external synapses.
 
@@ -116,6 +135,8 @@ class Glif3Simulator:
             raise ValueError("i_ext needs one entry per element")
         self.in_ptr = self.in_events = None
         self.in_steps = 0
+        self.in_duplicates = False
+        self._inp_form = None  # "pull" or "list" once a run has delivered inputs with the pull tables present
         self.step = 0
         self.words = n_words(self.ne)
         # history of spike bits: 2B+3 rows let resident workgroups drift B steps apart, one more lets them look
@@ -161,14 +182,14 @@ class Glif3Simulator:
     def _setup_resident(self, required):
         """Resident mode keeps state in registers and the ring in LDS for a whole
         run; it needs batch 1, at most 1024 elements per compute unit and a ring
-        slice that fits in LDS."""
+        slice that fits in LDS beside the kernel's active-row list."""
         n_cu = torch.cuda.get_device_properties(self.dev).multi_processor_count
-        span = -(-(-(-self.ne // (n_cu - n_cu % 8))) // 64) * 64
-        fits = self.batch == 1 and span <= 1024 and self.L * NREC * span * 4 <= 150 * 1024
-        if not fits:
+        span = resident_span(self.ne, self.batch, self.L, n_cu)
+        if not span:
             if required:
                 raise ValueError("network does not fit resident mode (batch 1, <= 1024 elements per compute unit, "
-                                 "ring slice <= 150 KB)")
+                                 "ring slice + {} bytes of lists within the {} bytes of LDS)".format(
+                                     RES_LDS_EXTRA, RES_LDS_BYTES))
             return
         groups = -(-self.ne // span)
         if self.rec is not None:
@@ -180,11 +201,15 @@ class Glif3Simulator:
         self.res_span, self.res_groups = span, groups
 
     def check(self):
-        """Raise if the last resident run gave up on its grid barrier (synchronises)."""
+        """Raise if a resident run since the last check gave up on its grid barrier (synchronises).  The abort
+        word is sticky on the device: a run that finds it set gives up at once, so a failure cannot be lost
+        between two checks; it is cleared here."""
         if self._pending_check:
             self._pending_check = False
             if int(self.res_sync[1].item()) != 0:
-                raise RuntimeError("resident simulation aborted: grid barrier timed out; results are invalid")
+                self.res_sync[1] = 0
+                raise RuntimeError("resident simulation aborted: grid barrier timed out; results since the last "
+                                   "check are invalid")
 
     def _table(self, csr, n_rows):
         if torch.is_tensor(csr[0]):
@@ -196,7 +221,13 @@ class Glif3Simulator:
 
     def set_input_events(self, in_ptr, in_events):
         """Per-step event lists: events in_events[in_ptr[t]:in_ptr[t+1]] are
-        emitted in step t (their spike stamp is t+1)."""
+        emitted in step t (their spike stamp is t+1).  Within a step the ids
+        (source*batch+trial) must be ascending -- the input-weight gradient kernel
+        gives every source's run of events one writer and relies on it.  The same id
+        may occur more than once in a step (two spikes of one generator inside one
+        resolution step, which NEST delivers both): every occurrence is delivered;
+        such lists keep the inputs on the event-list form of the delivery, because
+        the bit rows of the pull form can hold an id only once per step."""
         if self.inp is None:
             raise ValueError("no input synapse table")
         if torch.is_tensor(in_ptr):
@@ -205,19 +236,27 @@ class Glif3Simulator:
                 ok = ok and bool((in_events.min() >= 0) & (in_events.max() < self.n_inputs * self.batch))
             if not ok or in_ptr.dtype != torch.int64 or in_events.dtype != torch.int32:
                 raise ValueError("device input event lists are inconsistent")
+            dup = False
+            if in_events.numel() > 1:
+                step_start = torch.zeros(in_events.numel() + 1, dtype=torch.bool, device=in_events.device)
+                step_start[in_ptr] = True                      # an event that opens a step may be smaller than the last
+                d = in_events[1:] - in_events[:-1]
+                inside = ~step_start[1:-1]
+                if bool(((d < 0) & inside).any()):
+                    raise ValueError("input events must be ascending within every step")
+                dup = bool(((d == 0) & inside).any())
             self.in_ptr = in_ptr.contiguous()
             self.in_events = in_events.contiguous() if in_events.numel() else in_events.new_zeros(1)
             self.in_steps = in_ptr.numel() - 1
+            self.in_duplicates = dup
             return
         in_ptr = np.ascontiguousarray(in_ptr, np.int64)
         in_events = np.ascontiguousarray(in_events, np.int32)
-        if in_ptr[0] != 0 or np.any(np.diff(in_ptr) < 0) or in_ptr[-1] != in_events.size:
-            raise ValueError("in_ptr must be non-decreasing from 0 to len(in_events)")
-        if in_events.size and (in_events.min() < 0 or in_events.max() >= self.n_inputs * self.batch):
-            raise ValueError("input event id outside 0..n_inputs*batch-1")
+        dup = net.check_input_events(in_ptr, in_events, self.n_inputs * self.batch)
         self.in_ptr = torch.as_tensor(in_ptr, device=self.dev)
         self.in_events = torch.as_tensor(in_events if in_events.size else np.zeros(1, np.int32), device=self.dev)
         self.in_steps = in_ptr.size - 1
+        self.in_duplicates = dup
 
     def _struct(self, bits=None, record=None):
         s = _lib.Glif3Sim()
@@ -240,7 +279,14 @@ class Glif3Simulator:
         if self.pull_table is not None:
             s.pull_indptr, s.pull_packed = _p(self.pull_table.indptr), _p(self.pull_table.packed())
             s.pull_syn, s.pull_work = _p(self.pull_syn), _p(self.pull_work)
-            if self.pull_inp_table is not None and self.in_ptr is not None:
+            # the form the inputs take is fixed by the first run: arrivals still ahead live in the ring (event
+            # lists) or in the input-bit history (pull form), and a later run must find them where they are
+            if self.pull_inp_table is not None and self.in_ptr is not None and self._inp_form is None:
+                self._inp_form = "list" if self.in_duplicates else "pull"
+            if self._inp_form == "pull" and self.in_duplicates:
+                raise ValueError("input events repeat an id within a step, which the pull form of the inputs this "
+                                 "simulator has been running with cannot hold; build the simulator anew")
+            if self._inp_form == "pull":
                 s.pull_inp_indptr, s.pull_inp_packed = _p(self.pull_inp_table.indptr), _p(self.pull_inp_table.packed())
                 s.pull_inp_syn, s.pull_inp_work = _p(self.pull_inp_syn), _p(self.pull_inp_work)
                 s.in_hist, s.in_hist_stride = _p(self.in_hist), self.in_hist_stride

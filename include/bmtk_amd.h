@@ -180,7 +180,11 @@ typedef struct bmtk_glif3_sim {
     /* external spike sources: per-step event lists + source-major table */
     int64_t n_inputs;
     const int64_t *in_ptr;       /* [total steps + 1], indexed by absolute step */
-    const int32_t *in_events;    /* element ids source*batch+trial, emitted in that step */
+    const int32_t *in_events;    /* element ids source*batch+trial, emitted in that step; ascending within a step
+                                  * (the input-weight gradient relies on it).  An id may repeat within a step (two
+                                  * spikes of one source inside one resolution step): every occurrence is
+                                  * delivered, except by the pull form of the inputs (pull_inp_* below), whose
+                                  * bit rows hold an id once per step -- do not combine the two. */
     const int32_t *inp_indptr, *inp_indices;
     const float *inp_weights;
     const uint8_t *inp_delays, *inp_receptors;
@@ -215,10 +219,13 @@ typedef struct bmtk_glif3_sim {
     int32_t res_groups;
     const uint32_t *rec_seg;     /* [neurons][res_groups+1] */
     const uint32_t *inp_seg;     /* [inputs][res_groups+1] */
-    uint32_t *res_sync;          /* BMTK_RES_SYNC_WORDS words of scratch: word 1 = abort flag, from word
-                                  * BMTK_RES_SYNC_STRIDE on 64 x BMTK_RES_SYNC_WAYS arrival counters that many
-                                  * words apart; the call zeroes what it uses.  After the run, word 1 != 0 means
-                                  * the grid barrier timed out and the results are invalid. */
+    uint32_t *res_sync;          /* BMTK_RES_SYNC_WORDS words of scratch, zeroed by the caller once: word 1 =
+                                  * abort flag, from word BMTK_RES_SYNC_STRIDE on 64 x BMTK_RES_SYNC_WAYS arrival
+                                  * counters that many words apart, which every call zeroes again.  Word 1 != 0
+                                  * after a run means a grid barrier timed out and the results are invalid.  The
+                                  * flag is sticky: no call clears it, and a call that finds it set does nothing,
+                                  * so a failure cannot be overwritten before the host has seen it; the host
+                                  * clears it after reading. */
     /* Pull form of the recurrent delivery for batched runs (optional; launch-per-step mode with delay_offset 0
      * and hist_slots == ring_slots): a TARGET-major packed copy of the recurrent table.  The recurrent arrivals
      * of step t-1 are then summed in one pass over that table from the spike-bit history

@@ -365,9 +365,12 @@ def test_resident_barrier_gives_up_cleanly():
     assert sim.res_groups > 8
     sim.spin_limit = 1
     sim.hist_slots = 3  # no spare history row: the wait closes every step, when the barrier has only begun to fill
-    sim.run(300)
+    sim.run(200)
+    sim.spin_limit = 0
+    sim.run(100)            # finds the abort word set and does nothing: the failure cannot be overwritten unseen
     with pytest.raises(RuntimeError, match="barrier"):
         sim.check()
+    assert int(sim.res_sync[1].item()) == 0   # cleared by the check that reported it
     want, _, _ = _oracle_run(cfg, np.float64)
     sim = _gpu_sim(cfg, resident=True)
     out = sim.run(300)
@@ -402,3 +405,60 @@ def test_membrane_probes_equal_the_per_step_record(every):
         sim.set_probes([1, 1])
     with pytest.raises(ValueError):
         sim.set_probes([cfg["n"]])
+
+
+def _with_duplicate_events(cfg, rng, batch):
+    """The event lists of `cfg` with every fifth event of a step doubled or tripled (two or three spikes of one
+    source inside one step, which NEST delivers one by one), still ascending within each step."""
+    ptr, ev = cfg["in_ptr"], cfg["in_events"]
+    new_ptr, chunks = [0], []
+    for t in range(ptr.size - 1):
+        e = ev[ptr[t]:ptr[t + 1]]
+        extra = np.repeat(e[::5], rng.integers(1, 3, e[::5].size))
+        e = np.sort(np.concatenate([e, extra]))
+        chunks.append(e)
+        new_ptr.append(new_ptr[-1] + e.size)
+    return np.asarray(new_ptr, np.int64), np.concatenate(chunks).astype(np.int32)
+
+
+@pytest.mark.parametrize("batch,resident", [(1, False), (1, True), (8, False)])
+def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
+    """Two spikes of one generator inside one resolution step are two deliveries.  Every driver must count them:
+    the launch-per-step driver, the resident one, and the batched driver whose pull form of the inputs (bit rows:
+    one bit per id and step) steps aside for such lists.  Exact weights: bit-identical to the fp32 oracle."""
+    cfg = synthetic.small_glif3_network(n=700, n_in=300, steps=300, seed=14, in_w_scale=2.0, in_fanout=100,
+                                        p_conn=0.05, w_scale=1.5, batch=batch)
+    cfg["rec_src"] = _integer_weights(cfg["rec_src"])
+    cfg["inp_src"] = _integer_weights(cfg["inp_src"])
+    in_ptr, in_events = _with_duplicate_events(cfg, np.random.default_rng(3), batch)
+    assert in_events.size > 1.2 * cfg["in_events"].size
+    want, st, _ = _oracle_run(cfg, np.float32, batch=batch, in_ptr=in_ptr, in_events=in_events)
+    plain, _, _ = _oracle_run(cfg, np.float32, batch=batch)
+    assert want["count"] > 1.05 * plain["count"] > 500 * batch      # the repeats matter
+    sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
+                         inp=cfg["inp_src"], ring_slots=cfg["L"], resident=resident)
+    sim.set_input_events(in_ptr, in_events)
+    assert sim.in_duplicates
+    a, b = sim.run(120), sim.run(180)
+    sim.check()
+    if batch >= 8:
+        assert sim.pull_table is not None and sim.pull_inp_table is not None and sim._inp_form == "list"
+    ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
+    np.testing.assert_array_equal(ras, want["raster"])
+    got = sim.state.to_numpy()
+    for k in ("V", "asc", "y1", "y2", "ref"):
+        np.testing.assert_array_equal(got[k], st[k], err_msg=k)
+    # device tensors take the same checks
+    dev = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
+                         inp=cfg["inp_src"], ring_slots=cfg["L"], resident=resident)
+    dev.set_input_events(torch.as_tensor(in_ptr, device="cuda"), torch.as_tensor(in_events, device="cuda"))
+    assert dev.in_duplicates
+    dev.set_input_events(torch.as_tensor(cfg["in_ptr"], device="cuda"), torch.as_tensor(cfg["in_events"], device="cuda"))
+    assert not dev.in_duplicates
+    bad = in_events.copy()
+    k = int(in_ptr[np.flatnonzero(np.diff(in_ptr) >= 2)[0]])
+    bad[k] = bad[k + 1] + 1 if bad[k + 1] + 1 < 300 * batch else bad[k]      # descending pair inside a step
+    bad[k + 1] = bad[k + 1] if bad[k] > bad[k + 1] else bad[k] - 1
+    for form in (lambda x: x, lambda x: torch.as_tensor(x, device="cuda")):
+        with pytest.raises(ValueError, match="ascending"):
+            dev.set_input_events(form(in_ptr), form(bad))

@@ -67,3 +67,40 @@ def test_multimeter_at_any_resolution(dt, tmp_path):
     with pytest.raises(nest.kernel.NESTError):
         nest.SetStatus(mm, "interval", dt * 0.5)  # not a multiple of the resolution
     nest.ResetKernel()
+
+
+def test_input_event_lists_are_validated():
+    """Ascending ids within a step are required (the input-weight gradient relies on it); a repeated id within a
+    step is legal (NEST delivers both spikes) and is reported so that the bit-row form of the delivery is not used."""
+    ptr = np.array([0, 2, 2, 5], np.int64)
+    assert net.check_input_events(ptr, np.array([3, 7, 0, 4, 9], np.int32), 10) is False
+    assert net.check_input_events(ptr, np.array([3, 7, 0, 4, 4], np.int32), 10) is True
+    assert net.check_input_events(np.array([0, 0], np.int64), np.zeros(0, np.int32), 10) is False
+    # the first event of a step may be smaller than the last of the step before
+    assert net.check_input_events(np.array([0, 1, 2], np.int64), np.array([9, 0], np.int32), 10) is False
+    with pytest.raises(ValueError, match="ascending"):
+        net.check_input_events(ptr, np.array([7, 3, 0, 4, 9], np.int32), 10)
+    with pytest.raises(ValueError, match="outside"):
+        net.check_input_events(ptr, np.array([3, 7, 0, 4, 10], np.int32), 10)
+    with pytest.raises(ValueError, match="in_ptr"):
+        net.check_input_events(np.array([0, 3, 2, 5], np.int64), np.array([3, 7, 0, 4, 9], np.int32), 10)
+
+
+def test_resident_fit_bound_counts_the_active_row_list():
+    """The resident kernel keeps its ring slice AND an 8192-entry active-row list (plus a few static words) in
+    the 160 KB of LDS: ring slices between 128 KB and 150 KB used to pass the host check and then fail at launch."""
+    from bmtk_amd.simulator import RES_LDS_BYTES, RES_LDS_EXTRA, resident_span
+    assert resident_span(230924, 1, 6, 256) == 960                 # the 230k-neuron network: 92 KB ring slice
+    assert resident_span(230924, 2, 6, 256) == 0                   # batch 1 only
+    assert resident_span(256 * 1024 + 1, 1, 2, 256) == 0           # more than 1024 elements per compute unit
+    assert resident_span(256 * 960, 1, 8, 256) == 960              # 122,880 B + 33,024 B = 155,904 B fits
+    assert resident_span(256 * 960, 1, 9, 256) == 0                # 138,240 B ring slice: over with the list
+    assert resident_span(256 * 1024, 1, 8, 256) == 0               # 131,072 B ring slice: over with the list
+    assert resident_span(256 * 1024, 1, 7, 256) == 1024
+    for L in range(2, 40):
+        for ne in (1000, 100_000, 245_760, 262_144):
+            span = resident_span(ne, 1, L, 256)
+            if span:
+                assert span % 64 == 0 and span <= 1024 and span * 256 >= ne
+                assert L * 4 * span * 4 + RES_LDS_EXTRA <= RES_LDS_BYTES
+    assert resident_span(1000, 1, 6, 250) == 64                    # 248 usable compute units
