@@ -55,7 +55,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 8  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 9  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -70,6 +70,7 @@ SIGNATURES = {
     "bmtk_spikes_compact_workspace_bytes": (c_int64, [c_int64]),
     "bmtk_spikes_compact": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "bmtk_spikes_compact_bits": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "bmtk_spikes_compact_noalloc": (c_int32, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "bmtk_csr_propagate_scatter": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
                                              c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "bmtk_csr_propagate_gather": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -88,6 +89,7 @@ SIGNATURES = {
 
 
 RES_SYNC_WORDS = (1 + 64 * 8) * 1088  # BMTK_RES_SYNC_WORDS
+COMPACT_NOALLOC_MAX_N = 1 << 24       # BMTK_COMPACT_NOALLOC_MAX_N
 
 
 class LibraryMissing(RuntimeError):

@@ -4,6 +4,8 @@
 #include <math.h>
 #include <stdarg.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "glif3_update.hpp"
 #include "propagate.hpp"
@@ -460,6 +462,61 @@ int bmtk_spikes_compact(const uint8_t *z, int64_t n, int32_t *ids, int32_t *coun
     const unsigned grid = (unsigned)((n + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(pack_bits_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, z, n, bits);
     return compact_from_bits(bits, n, ids, count, block_count, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------
+// The same compaction with the workspace inside the library: a file-scope
+// device array, so that the call allocates nothing.  In host code the array's
+// name is only a handle; its device address is asked for once per device, with
+// that device current, and kept.
+// ---------------------------------------------------------------------------
+
+constexpr int64_t kNoAllocBytes = 8 * (BMTK_COMPACT_NOALLOC_MAX_N / 64 + 1) +
+                                  4 * (BMTK_COMPACT_NOALLOC_MAX_N / 64 / kWordsPerBlock + 2);
+static __device__ __align__(256) unsigned char scratch[(kNoAllocBytes + 255) / 256 * 256];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on every device seen so far
+static std::mutex g_scratch_mutex;
+
+// device address of this device's copy of `scratch`, or nullptr with the error message set
+static void *scratch_of_current_device()
+{
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("spikes_compact_noalloc: cannot tell the current device (%s)", hipGetErrorString(err));
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !ptr) {
+            set_error("spikes_compact_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(err));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
+int bmtk_spikes_compact_noalloc(const uint8_t *z, int64_t n, int32_t *ids, int32_t *count, void *stream)
+{
+    BMTK_REQUIRE(n > 0, "spikes_compact_noalloc: n must be positive");
+    BMTK_REQUIRE(n <= BMTK_COMPACT_NOALLOC_MAX_N,
+                 "spikes_compact_noalloc: n = %lld exceeds the %lld elements the built-in workspace holds; use "
+                 "bmtk_spikes_compact with a workspace of the caller's", (long long)n,
+                 (long long)BMTK_COMPACT_NOALLOC_MAX_N);
+    BMTK_REQUIRE(z && ids && count, "spikes_compact_noalloc: pointers must be non-null");
+    static_assert(kNoAllocBytes >= 8 * ((BMTK_COMPACT_NOALLOC_MAX_N + 63) / 64 + 1) +
+                                       4 * (((BMTK_COMPACT_NOALLOC_MAX_N + 63) / 64 + kWordsPerBlock - 1) / kWordsPerBlock + 1),
+                  "scratch smaller than bmtk_spikes_compact_workspace_bytes(BMTK_COMPACT_NOALLOC_MAX_N)");
+    void *ws = scratch_of_current_device();
+    if (!ws) return BMTK_E_DEVICE;
+    // every word of the workspace a kernel reads is written earlier in the same call, so what the call before
+    // left behind does not matter and nothing has to be cleared
+    return bmtk_spikes_compact(z, n, ids, count, ws, stream);
 }
 
 int bmtk_spikes_compact_bits(const uint64_t *zbits, int64_t n, int32_t *ids, int32_t *count, void *workspace,

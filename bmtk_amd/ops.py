@@ -138,6 +138,16 @@ class SpikeCompactor:
         return self.ids, self.count
 
 
+def spikes_compact_noalloc(z, ids, count):
+    """``bmtk_spikes_compact_noalloc``: byte flags ``z`` -> ascending ids in the caller's ``ids`` (int32, at least
+    ``z.numel()`` entries) and their number in ``count`` (int32 [1]); the workspace is inside the library, nothing
+    is allocated, ``z.numel()`` is limited to ``_lib.COMPACT_NOALLOC_MAX_N``.  Calls that overlap on one GPU race."""
+    lib = _lib.load()
+    n = z.numel()
+    _lib.check(lib.bmtk_spikes_compact_noalloc(_p(z, torch.uint8, n, "z"), n, _p(ids, torch.int32, n, "ids"),
+                                               _p(count, torch.int32, 1, "count"), _stream()))
+
+
 def spikes_compact(z):
     """Convenience form: returns the id list as a tensor of the exact length (synchronises)."""
     c = SpikeCompactor(z.numel())

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 8
+#define BMTK_AMD_ABI_VERSION 9
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -88,6 +88,18 @@ int bmtk_spikes_compact(const uint8_t *z, int64_t n, int32_t *ids, int32_t *coun
 /* Same from spike bits (n elements, ceil(n/64) words are read). */
 int bmtk_spikes_compact_bits(const uint64_t *zbits, int64_t n, int32_t *ids, int32_t *count, void *workspace,
                              void *stream);
+
+/* bmtk_spikes_compact without a workspace argument and without any allocation.  No counterpart in the
+ * reference: it exists for callers that cannot allocate device memory -- code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The workspace is an array inside the library (about 2.1 MB
+ * of device memory on every GPU the library runs on, held until the process ends), which bounds the input:
+ * n <= BMTK_COMPACT_NOALLOC_MAX_N, larger n returns BMTK_E_ARG.  z, ids (n entries) and count (one int32) are
+ * the caller's, as above; the result is the same as bmtk_spikes_compact's.  All calls on one GPU share that
+ * GPU's array: calls that overlap on one GPU (different streams or threads) race and must be serialised by the
+ * caller; calls on different GPUs are independent.  The first call on a device looks up the array's address
+ * (hipGetSymbolAddress, no allocation). */
+#define BMTK_COMPACT_NOALLOC_MAX_N (1ll << 24)
+int bmtk_spikes_compact_noalloc(const uint8_t *z, int64_t n, int32_t *ids, int32_t *count, void *stream);
 
 /* Event-driven delivery (NEST static_synapse::send -> RingBuffer::add_value,
  * wired by nest.Connect in bmtk/simulator/pointnet/pointnetwork.py:161-173,187-232):

@@ -67,6 +67,13 @@ def test_argument_validation_needs_no_gpu():
     assert lib.bmtk_glif3_simulate_fwd(None, 0, 1, None) == -1
     with pytest.raises(_lib.BmtkAmdError):
         _lib.check(lib.bmtk_csr_pack(-1, None, None, None, None, None, None))
+    # the entry point without allocation rejects sizes beyond its built-in workspace before touching a device
+    assert lib.bmtk_spikes_compact_noalloc(None, _lib.COMPACT_NOALLOC_MAX_N + 1, None, None, None) == -1
+    assert b"exceeds" in lib.bmtk_amd_last_error()
+    assert lib.bmtk_spikes_compact_noalloc(None, 16, None, None, None) == -1      # null pointers
+    limit = int(re.search(r"#define BMTK_COMPACT_NOALLOC_MAX_N \(1ll << (\d+)\)",
+                          open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()).group(1))
+    assert _lib.COMPACT_NOALLOC_MAX_N == 1 << limit
 
 
 def test_ops_refuse_to_run_without_a_gpu():
