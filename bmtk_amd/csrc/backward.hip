@@ -37,8 +37,8 @@ __global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, Bw
     const int tile0 = blockIdx.y * kWave;
     const bool lane_on = tile0 + b < batch;
     const int64_t e = j * batch + tile0 + b;
-    bool active = false;
-    if (lane_on) {
+    bool active = lane_on && a.save_flags == nullptr;  // without a forward record every element counts
+    if (lane_on && a.save_flags) {
         const uint8_t f = a.save_flags[q.row * ne + e];
         if (f & BMTK_F_INTEGRATING) {
             const int64_t col = a.class_id ? (int64_t)a.class_id[j] : j;
@@ -98,8 +98,8 @@ __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, B
     const int sub = lane / lp, b4 = (lane - sub * lp) * 4;
     const bool lane_on = b4 < batch;
     const int64_t e = j * batch + b4;
-    unsigned act = 0u;  // bit c: trial b4+c has a non-zero surrogate derivative in this step
-    if (lane_on) {
+    unsigned act = (lane_on && a.save_flags == nullptr) ? 0xFu : 0u;  // bit c: trial b4+c has a non-zero surrogate derivative in this step
+    if (lane_on && a.save_flags) {
         const uint32_t f4 = *reinterpret_cast<const uint32_t *>(a.save_flags + q.row * ne + e);
         const float4 v4 = *reinterpret_cast<const float4 *>(a.save_v + q.row * ne + e);
         const int64_t col = a.class_id ? (int64_t)a.class_id[j] : j;
@@ -369,6 +369,38 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
         if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(256), dim3(kBlock), 0, st, a, q);
     }
     BMTK_CHECK_LAUNCH("glif3_simulate_bwd");
+    return BMTK_OK;
+}
+
+extern "C" int bmtk_csr_propagate_bwd(const int32_t *indptr, const bmtk_synapse *packed, int64_t n_neurons,
+                                      int32_t batch, const float *lam_ring, int32_t L, int64_t step, float *gz,
+                                      int32_t trials_per_lane, void *stream)
+{
+    BMTK_REQUIRE(indptr && packed && lam_ring && gz, "csr_propagate_bwd: pointers must be non-null");
+    BMTK_REQUIRE(n_neurons > 0 && batch > 0 && step >= 0, "csr_propagate_bwd: bad sizes or step");
+    BMTK_REQUIRE(n_neurons * (int64_t)batch < (1ll << 31) && n_neurons < (1ll << 24), "csr_propagate_bwd: network too large");
+    BMTK_REQUIRE(L > 1 && L <= 64, "csr_propagate_bwd: L must lie in 2..64");
+    const bool can4 = batch % 4 == 0 && batch <= kWave;
+    BMTK_REQUIRE(trials_per_lane == 0 || trials_per_lane == 1 || (trials_per_lane == 4 && can4),
+                 "csr_propagate_bwd: trials_per_lane must be 0 (choose), 1, or 4 for batches that are a multiple of 4 up to 64");
+    bmtk_glif3_bwd a{};
+    a.n_neurons = n_neurons;
+    a.batch = batch;
+    a.ring_slots = L;
+    a.rec_indptr = indptr;
+    a.rec_packed = packed;
+    a.lam_ring = const_cast<float *>(lam_ring);
+    a.gz = gz;
+    BwdStep q{step, 0};
+    const unsigned rows_grid = (unsigned)((n_neurons + kBlock / kWave - 1) / (kBlock / kWave));
+    int bp = 1;
+    while (bp < batch && bp < kWave) bp <<= 1;
+    if (trials_per_lane == 4 || (trials_per_lane == 0 && can4))
+        hipLaunchKernelGGL(bwd_gather4_kernel, dim3(rows_grid), dim3(kBlock), 0, (hipStream_t)stream, a, q, bp / 4);
+    else
+        hipLaunchKernelGGL(bwd_gather_kernel, dim3(rows_grid, (unsigned)((batch + kWave - 1) / kWave)), dim3(kBlock), 0,
+                           (hipStream_t)stream, a, q, bp);
+    BMTK_CHECK_LAUNCH("csr_propagate_bwd");
     return BMTK_OK;
 }
 

@@ -303,18 +303,6 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const int32_t *__restri
 // in stored synapse order: deterministic and equal to a scalar loop.
 // ---------------------------------------------------------------------------
 
-__device__ __forceinline__ unsigned long long source_mask(const uint64_t *__restrict__ zbits, int src, int batch,
-                                                          int tile0, int width)
-{
-    const int64_t bit = (int64_t)src * batch + tile0;
-    const int64_t w = bit >> 6;
-    const int sh = (int)(bit & 63);
-    unsigned long long m = zbits[w] >> sh;
-    if (sh + width > 64) m |= zbits[w + 1] << (64 - sh);
-    if (width < 64) m &= (1ull << width) - 1ull;
-    return m;
-}
-
 __global__ __launch_bounds__(kBlock) void gather_kernel(const uint64_t *__restrict__ zbits, int batch, Table t,
                                                         float *__restrict__ ring, int L, int64_t n_tgt, int64_t ne,
                                                         int slot0)
@@ -569,183 +557,3 @@ int bmtk_csr_propagate_gather(const uint64_t *zbits, int64_t n_src, int32_t batc
 }
 
 }  // extern "C"
-
-// ---------------------------------------------------------------------------
-// Pull-mode propagation (batched runs): one pass over a packed target-major
-// table computes everything that arrives in one step from the spike bits of
-// the last L steps.  Lane = synapse; a lane walks the set bits of its source's
-// trial mask and adds its weight into the wavefront's LDS accumulators
-// [receptor][trial] -- work per 64-synapse chunk is the largest popcount among
-// its lanes, not the number of events.
-// ---------------------------------------------------------------------------
-
-namespace bmtk {
-
-// any_map[slot][j/32] bit (j%32): source neuron j fired in at least one trial in the step held by history row `slot`
-__global__ __launch_bounds__(kBlock) void pull_anymap_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride,
-                                                             int L, int batch, int64_t n_src, int n_w32,
-                                                             uint32_t *__restrict__ any_map)
-{
-    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const int slot = (int)(idx / ((int64_t)n_w32 * 32));
-    const int64_t j = idx - (int64_t)slot * n_w32 * 32;
-    bool any = false;
-    if (slot < L && j < n_src) {
-        const uint64_t *row = hist + (int64_t)slot * hist_stride;
-        for (int t0 = 0; t0 < batch && !any; t0 += kWave)
-            any = source_mask(row, (int)j, batch, t0, min(kWave, batch - t0)) != 0ull;
-    }
-    const unsigned long long m = __ballot(any);
-    if (slot < L && (lane_id() & 31) == 0 && j < (int64_t)n_w32 * 32)
-        any_map[(int64_t)slot * n_w32 + (j >> 5)] = (uint32_t)(m >> (lane_id() & 32));
-}
-
-constexpr int kPullBlock = 1024;  // 16 wavefronts share one staged activity map
-
-__global__ __launch_bounds__(kPullBlock) void pull_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride, int L,
-                                                      int batch, const int32_t *__restrict__ indptr,
-                                                      const bmtk_synapse *__restrict__ packed,
-                                                      float *__restrict__ syn, int64_t n_tgt, int64_t ne,
-                                                      int slot_now, const uint32_t *__restrict__ any_map, int n_w32)
-{
-    extern __shared__ uint32_t any_l[];  // [L][n_w32], then the accumulators
-    float(*acc_all)[GLIF3_NREC][kWave] =
-        reinterpret_cast<float(*)[GLIF3_NREC][kWave]>(any_l + (size_t)L * n_w32);
-    const int lane = lane_id();
-    const int wave = threadIdx.x / kWave;
-    float(*acc)[kWave] = acc_all[wave];
-    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
-    __syncthreads();
-    const int tile0 = blockIdx.y * kWave;
-    const int width = min(kWave, batch - tile0);
-    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(packed);
-    constexpr int kUnroll = 4;  // 64-synapse chunks per wavefront and iteration (8 costs occupancy)
-    const int64_t stride = (int64_t)gridDim.x * (kPullBlock / kWave);
-    auto fetch = [&](uint2 *dst, int base, int p1) {
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            // streamed once per step: keep it from displacing the spike history in L2
-            // streamed once per step: keep it from displacing the spike history in L2
-            const unsigned long long raw = __builtin_nontemporal_load(
-                reinterpret_cast<const unsigned long long *>(rows + min(base + u * kWave, p1 - 1)));
-            dst[u] = make_uint2((unsigned)raw, (unsigned)(raw >> 32));
-        }
-    };
-    // Software pipeline over (row, 256-synapse block) pairs: the synapses of the next block --
-    // possibly of the next row, whose bounds were fetched a row ahead -- are in flight while
-    // the current block is processed.
-    int64_t row = (int64_t)blockIdx.x * (kPullBlock / kWave) + wave;
-    if (row >= n_tgt) return;
-    int p0 = indptr[row], p1 = indptr[row + 1];
-    int np0 = 0, np1 = 0;
-    if (row + stride < n_tgt) {
-        np0 = indptr[row + stride];
-        np1 = indptr[row + stride + 1];
-    }
-    int base = p0 + lane;
-    uint2 cur[kUnroll], nxt[kUnroll];
-    if (p1 > p0) fetch(cur, base, p1);
-#pragma unroll
-    for (int r = 0; r < GLIF3_NREC; ++r) acc[r][lane] = 0.0f;
-    while (true) {
-        // where the next block lies (uniform across the wavefront)
-        int64_t nrow = row;
-        int nbase = base + kUnroll * kWave, nq0 = p0, nq1 = p1;
-        const bool row_done = (base - lane) + kUnroll * kWave >= p1;
-        if (row_done) {
-            nrow = row + stride;
-            nq0 = np0;
-            nq1 = np1;
-            nbase = nq0 + lane;
-            if (nrow + stride < n_tgt) {
-                np0 = indptr[nrow + stride];
-                np1 = indptr[nrow + stride + 1];
-            }
-        }
-        const bool more = nrow < n_tgt;
-        if (more && nq1 > nq0) fetch(nxt, nbase, nq1);
-        if (p1 > p0) {
-            unsigned long long m[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                int slot = slot_now - (int)(cur[u].x >> 26);
-                slot = slot < 0 ? slot + L : slot;
-                const int src = (int)(cur[u].x & 0xFFFFFFu);
-                const bool hit = base + u * kWave < p1 && ((any_l[slot * n_w32 + (src >> 5)] >> (src & 31)) & 1u);
-                m[u] = hit ? source_mask(hist + (int64_t)slot * hist_stride, src, batch, tile0, width) : 0ull;
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                float *a = acc[(cur[u].x >> 24) & 3];
-                const float w = __uint_as_float(cur[u].y);
-                unsigned lo = (unsigned)m[u], hi = (unsigned)(m[u] >> 32);
-                while (lo) {
-                    const int b = __ffs((int)lo) - 1;
-                    lo &= lo - 1u;
-                    atomicAdd(a + b, w);
-                }
-                while (hi) {
-                    const int b = __ffs((int)hi) - 1;
-                    hi &= hi - 1u;
-                    atomicAdd(a + 32 + b, w);
-                }
-            }
-        }
-        if (row_done) {
-            if (lane < width) {
-#pragma unroll
-                for (int r = 0; r < GLIF3_NREC; ++r) {
-                    syn[(int64_t)r * ne + row * batch + tile0 + lane] = acc[r][lane];
-                    acc[r][lane] = 0.0f;
-                }
-            }
-        }
-        if (!more) break;
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) cur[u] = nxt[u];
-        row = nrow;
-        base = nbase;
-        p0 = nq0;
-        p1 = nq1;
-    }
-}
-
-}  // namespace bmtk
-
-extern "C" int64_t bmtk_csr_propagate_pull_workspace_bytes(int32_t L, int64_t n_src)
-{
-    if (L <= 0 || n_src <= 0) return 0;
-    return (int64_t)L * ((n_src + 31) / 32) * 4;
-}
-
-extern "C" int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src,
-                                       int32_t batch, const int32_t *indptr, const bmtk_synapse *packed, float *syn,
-                                       int64_t n_tgt, int64_t t_arrive, void *workspace, void *stream)
-{
-    using namespace bmtk;
-    BMTK_REQUIRE(spike_hist && indptr && packed && syn && workspace, "csr_propagate_pull: pointers must be non-null");
-    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && n_src > 0 && t_arrive >= 0, "csr_propagate_pull: bad batch, sizes or step");
-    BMTK_REQUIRE(L > 1 && L <= 64, "csr_propagate_pull: L must lie in 2..64");
-    BMTK_REQUIRE(hist_stride >= (n_src * (int64_t)batch + 63) / 64 + 1,
-                 "csr_propagate_pull: hist_stride must hold ceil(n_src*batch/64)+1 words");
-    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31) && n_src < (1ll << 24), "csr_propagate_pull: network too large");
-    const int n_w32 = (int)((n_src + 31) / 32);
-    const size_t lds = (size_t)L * n_w32 * 4 + (size_t)(kPullBlock / kWave) * GLIF3_NREC * kWave * sizeof(float);
-    BMTK_REQUIRE(lds <= 64u * 1024u, "csr_propagate_pull: L * n_src too large for the activity map in LDS");
-    uint32_t *any_map = (uint32_t *)workspace;
-    const int64_t map_threads = (int64_t)L * n_w32 * 32;
-    hipLaunchKernelGGL(pull_anymap_kernel, dim3((unsigned)((map_threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       (hipStream_t)stream, spike_hist, hist_stride, L, batch, n_src, n_w32, any_map);
-    const unsigned rows_per_block = kPullBlock / kWave;
-    int dev = 0, n_cu = 256;
-    (void)hipGetDevice(&dev);
-    (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
-    const unsigned want = (unsigned)((n_tgt + rows_per_block - 1) / rows_per_block);
-    const unsigned cap = (unsigned)n_cu * 2u;  // persistent workgroups: the activity map is staged once per workgroup
-    const dim3 grid(want < cap ? want : cap, (unsigned)((batch + kWave - 1) / kWave));
-    BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_pull: batch too large");
-    hipLaunchKernelGGL(pull_kernel, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L, batch,
-                       indptr, packed, syn, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
-    BMTK_CHECK_LAUNCH("csr_propagate_pull");
-    return BMTK_OK;
-}

@@ -27,4 +27,18 @@ __device__ __forceinline__ void deliver_row(const Table &t, int j, int b, int ba
     }
 }
 
+// spike bits of source `src` in trials tile0 .. tile0+width-1 (width <= 64) as a lane mask: bit b = trial tile0+b.
+// Reads one or two words of a spike-bit row; rows carry a padding word so that the second read stays inside.
+__device__ __forceinline__ unsigned long long source_mask(const uint64_t *__restrict__ zbits, int src, int batch,
+                                                          int tile0, int width)
+{
+    const int64_t bit = (int64_t)src * batch + tile0;
+    const int64_t w = bit >> 6;
+    const int sh = (int)(bit & 63);
+    unsigned long long m = zbits[w] >> sh;
+    if (sh + width > 64) m |= zbits[w + 1] << (64 - sh);
+    if (width < 64) m &= (1ull << width) - 1ull;
+    return m;
+}
+
 }  // namespace bmtk

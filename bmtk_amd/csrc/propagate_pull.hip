@@ -1,0 +1,308 @@
+// Pull-mode propagation (batched runs): one pass over a packed target-major
+// table computes everything that arrives in one step from the spike bits of
+// the last L steps.
+//
+// A wavefront owns a target row at a time.  The row's synapses are streamed 64
+// per load instruction (lane = synapse); a per-source "fired in any trial" bit
+// map of the L steps, staged in LDS, filters the synapses whose source was
+// silent, and the others fetch their source's trial mask.  Every lane then
+// walks the set bits of its mask and adds its weight to the wavefront's LDS
+// accumulators [receptor][trial].
+//
+// The accumulators are 64-bit fixed point (Q31.32) and the additions are
+// 64-bit integer LDS atomics.  Two reasons, both measured on gfx950: an LDS
+// float atomic costs about three clocks per LANE (its lanes are worked off one
+// after the other), an integer one about nine clocks per 64-lane INSTRUCTION;
+// and integer additions commute exactly, so the sums do not depend on the
+// order in which lanes and wavefronts arrive: the result is deterministic and
+// equals the exact sum of the weights, rounded to fp32 once at the end of the
+// row.  An fp32 weight converts to Q31.32 without error down to 2^-32 pA
+// (smaller bits are dropped); weights must be finite and below 2^31 in size.
+
+#include "common.hpp"
+#include "propagate.hpp"
+
+namespace bmtk {
+
+// any_map[slot][j/32] bit (j%32): source neuron j fired in at least one trial in the step held by history row `slot`
+__global__ __launch_bounds__(kBlock) void pull_anymap_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride,
+                                                             int L, int batch, int64_t n_src, int n_w32,
+                                                             uint32_t *__restrict__ any_map)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int slot = (int)(idx / ((int64_t)n_w32 * 32));
+    const int64_t j = idx - (int64_t)slot * n_w32 * 32;
+    bool any = false;
+    if (slot < L && j < n_src) {
+        const uint64_t *row = hist + (int64_t)slot * hist_stride;
+        for (int t0 = 0; t0 < batch && !any; t0 += kWave)
+            any = source_mask(row, (int)j, batch, t0, min(kWave, batch - t0)) != 0ull;
+    }
+    const unsigned long long m = __ballot(any);
+    if (slot < L && (lane_id() & 31) == 0 && j < (int64_t)n_w32 * 32)
+        any_map[(int64_t)slot * n_w32 + (j >> 5)] = (uint32_t)(m >> (lane_id() & 32));
+}
+
+constexpr int kPullBlock = 1024;  // 16 wavefronts share one staged activity map
+// per wavefront: 4 x 64 accumulators of 8 bytes and a stage of 64 entries of 8 bytes
+constexpr size_t kPullAccBytes = (size_t)(kPullBlock / kWave) * (GLIF3_NREC + 1) * kWave * sizeof(unsigned long long);
+constexpr size_t kPullLdsMax = 80u * 1024u;  // two workgroups per compute unit: each may take half of the 160 KB of LDS
+
+// fp32 -> Q31.32 two's complement.  The size |w| is split with floor(): the integer part, and what is left, which
+// lies in [0, 1) and is exact (for a negative w, w - floor(w) = w + 1 would round); times 2^32 it is an integer
+// below 2^32 up to the bits under 2^-32, which the conversion drops.  The sign is applied to the integer.
+__device__ __forceinline__ unsigned long long to_fixed(float w)
+{
+    const float size = fabsf(w);
+    const float whole = floorf(size);
+    const unsigned lo = (unsigned)((size - whole) * 4294967296.0f);
+    const unsigned long long v = ((unsigned long long)(unsigned)whole << 32) | lo;
+    return w < 0.0f ? 0ull - v : v;
+}
+
+__device__ __forceinline__ float from_fixed(unsigned long long v)
+{
+    return (float)((double)(long long)v * (1.0 / 4294967296.0));
+}
+
+// One block of a row's synapse stream: positions [base, min(base + kPullChunks*64, p1)) of the packed table.
+constexpr int kPullChunks = 4;  // 64-synapse chunks per block
+struct PullBlock {
+    int64_t row;  // >= n_tgt: past the end
+    int base, p1;
+    bool last;    // last block of its row: the sums are stored after it
+};
+
+// The rows a wavefront owns (first, first + stride, ...) as a stream of blocks.  The bounds of the row after the
+// current one are fetched a row ahead.  Everything here is the same in all lanes (scalar registers and loads).
+struct PullCursor {
+    const int32_t *__restrict__ indptr;
+    int64_t n_tgt, stride, row;
+    int q, p1, np0, np1;
+
+    __device__ __forceinline__ void start(const int32_t *ip, int64_t n, int64_t first, int64_t step)
+    {
+        indptr = ip;
+        n_tgt = n;
+        stride = step;
+        row = first;
+        q = p1 = np0 = np1 = 0;
+        if (row < n_tgt) {
+            q = indptr[row];
+            p1 = indptr[row + 1];
+        }
+        if (row + stride < n_tgt) {
+            np0 = indptr[row + stride];
+            np1 = indptr[row + stride + 1];
+        }
+    }
+    __device__ __forceinline__ PullBlock next()
+    {
+        PullBlock b{row, q, p1, false};
+        if (row < n_tgt) {
+            q += kPullChunks * kWave;
+            if (q >= p1) {
+                b.last = true;
+                row += stride;
+                q = np0;
+                p1 = np1;
+                if (row + stride < n_tgt) {
+                    np0 = indptr[row + stride];
+                    np1 = indptr[row + stride + 1];
+                }
+            }
+        }
+        return b;
+    }
+};
+
+// kWords64: batch == 64, so that the trial mask of source j is word j of a history row; otherwise the general
+// bit-field read (any batch, tiles of 64 trials over blockIdx.y).
+//
+// Below ~5 Hz this kernel is bound by instruction issue, not by bandwidth: most synapses have a silent source, and
+// what is spent per 64-synapse chunk on the few that do not -- mask address, gather, weight conversion, bit walk --
+// costs the same whether 4 or 64 lanes take part.  So the synapses with an event are first packed into a
+// 64-entry stage in LDS (one ballot and one store per chunk), and the expensive part runs once per full stage:
+// one gather of 64 masks, one conversion, one bit walk with every lane busy.  At 1 Hz that is once per row
+// instead of sixteen times.  The per-synapse part uses 32-bit offsets against scalar base pointers and unsigned
+// wrap-around for the history row of a delay.
+template <bool kWords64>
+__global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride, int L,
+                                                         int batch, const int32_t *__restrict__ indptr,
+                                                         const bmtk_synapse *__restrict__ packed,
+                                                         float *__restrict__ syn, int64_t n_tgt, int64_t ne,
+                                                         int slot_now, const uint32_t *__restrict__ any_map, int n_w32)
+{
+    extern __shared__ unsigned long long pull_lds[];  // accumulators, stages, then the activity map [L][n_w32]
+    // (the wavefront's number through a scalar register, so that rows, bounds and base pointers stay scalar)
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    unsigned long long(*acc)[kWave] = reinterpret_cast<unsigned long long(*)[kWave]>(pull_lds) + wave * GLIF3_NREC;
+    uint2 *stage = reinterpret_cast<uint2 *>(pull_lds + (kPullBlock / kWave) * GLIF3_NREC * kWave) + wave * kWave;
+    uint32_t *any_l = reinterpret_cast<uint32_t *>(pull_lds + (kPullBlock / kWave) * (GLIF3_NREC + 1) * kWave);
+    const unsigned lane = (unsigned)lane_id();
+    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
+    __syncthreads();
+    const int tile0 = kWords64 ? 0 : (int)blockIdx.y * kWave;
+    const int width = kWords64 ? kWave : min(kWave, batch - tile0);
+    const unsigned hstride = (unsigned)hist_stride;  // L * hist_stride * 8 < 2^32 bytes (checked by the caller)
+    const unsigned uL = (unsigned)L, unow = (unsigned)slot_now, uw32 = (unsigned)n_w32;
+    const char *__restrict__ hist_bytes = reinterpret_cast<const char *>(hist);
+    // Block of the table: 64-bit words at a scalar base, 8 * (lane + u*64) bytes on.  Lanes past the end of the
+    // row read its last synapse again (and are ignored later): no branch, the four loads go out back to back.
+    auto fetch = [&](unsigned long long *dst, const PullBlock &blk) {
+        if (blk.row >= n_tgt || blk.base >= blk.p1) return;
+        const char *__restrict__ src = reinterpret_cast<const char *>(packed) + (size_t)blk.base * 8u;
+        const unsigned last = (unsigned)(blk.p1 - blk.base) - 1u;
+#pragma unroll
+        for (int u = 0; u < kPullChunks; ++u)
+            // streamed once per step: keep it from displacing the spike history in L2
+            dst[u] = __builtin_nontemporal_load(
+                reinterpret_cast<const unsigned long long *>(src + min(lane + u * kWave, last) * 8u));
+    };
+    PullCursor cursor;
+    cursor.start(indptr, n_tgt, (int64_t)blockIdx.x * (kPullBlock / kWave) + wave,
+                 (int64_t)gridDim.x * (kPullBlock / kWave));
+    // Three table blocks per wavefront: the one at hand and the two after it, whose loads stay in flight during
+    // the whole turn (a buffer is refilled, with the block three ahead, as soon as its turn is over).
+    PullBlock b0 = cursor.next();
+    if (b0.row >= n_tgt) return;
+    unsigned long long d0[kPullChunks] = {0ull, 0ull, 0ull, 0ull}, d1[kPullChunks] = {0ull, 0ull, 0ull, 0ull},
+                       d2[kPullChunks] = {0ull, 0ull, 0ull, 0ull};
+    fetch(d0, b0);
+    PullBlock b1 = cursor.next();
+    fetch(d1, b1);
+    PullBlock b2 = cursor.next();
+    fetch(d2, b2);
+#pragma unroll
+    for (int r = 0; r < GLIF3_NREC; ++r) acc[r][lane] = 0ull;
+    int staged = 0;  // entries in the stage (same in all lanes)
+    // the staged synapses: gather their trial masks, convert their weights, add
+    auto flush = [&]() {
+        if ((int)lane < staged) {
+            const uint2 e = stage[lane];  // {source | receptor << 24 | history row << 26, weight}
+            const unsigned src = e.x & 0xFFFFFFu, row = e.x >> 26;
+            unsigned long long mm;
+            if (kWords64)
+                mm = *reinterpret_cast<const unsigned long long *>(hist_bytes + (__umul24(row, hstride) + src) * 8u);
+            else
+                mm = source_mask(hist + (size_t)row * hstride, (int)src, batch, tile0, width);
+            unsigned long long *a = acc[(e.x >> 24) & 3u];
+            const unsigned long long w = to_fixed(__uint_as_float(e.y));
+            while (mm) {
+                const int b = __ffsll((long long)mm) - 1;
+                mm &= mm - 1ull;
+                atomicAdd(a + b, w);
+            }
+        }
+        staged = 0;
+    };
+    // one turn: the block `cb` with its table words `cd`; afterwards the buffer takes the block three ahead
+    auto turn = [&](PullBlock &cb, unsigned long long *cd) {
+        const unsigned left = cb.base < cb.p1 ? (unsigned)(cb.p1 - cb.base) : 0u;
+        // activity bits of the four chunks (LDS reads, no branch between them)
+        unsigned slot[kPullChunks], word[kPullChunks];
+#pragma unroll
+        for (int u = 0; u < kPullChunks; ++u) {
+            const unsigned tdr = (unsigned)cd[u];
+            // history row of the emitting step: (now - delay) mod L by unsigned wrap-around
+            const unsigned back = unow - (tdr >> 26);
+            slot[u] = min(back, back + uL);
+            word[u] = any_l[__umul24(slot[u], uw32) + ((tdr & 0xFFFFFFu) >> 5)];
+        }
+#pragma unroll
+        for (int u = 0; u < kPullChunks; ++u) {
+            const unsigned tdr = (unsigned)cd[u];
+            const bool hit = lane + u * kWave < left && ((word[u] >> (tdr & 31u)) & 1u);
+            const unsigned long long who = __ballot(hit);
+            const int n = __popcll(who);
+            if (n == 0) continue;
+            if (staged + n > kWave) flush();
+            if (hit) stage[staged + lane_prefix(who)] = make_uint2((tdr & 0x3FFFFFFu) | (slot[u] << 26), (unsigned)(cd[u] >> 32));
+            staged += n;
+        }
+        if (cb.last) {
+            flush();
+#pragma unroll
+            for (int r = 0; r < GLIF3_NREC; ++r) {
+                if ((int)lane < width) syn[(int64_t)r * ne + cb.row * batch + tile0 + lane] = from_fixed(acc[r][lane]);
+                acc[r][lane] = 0ull;
+            }
+        }
+        cb = cursor.next();
+        fetch(cd, cb);
+    };
+    // the buffers take turns in place, so that no register copy ties the arrival of a later block to the work on
+    // this one
+    while (true) {
+        turn(b0, d0);
+        if (b1.row >= n_tgt) break;
+        turn(b1, d1);
+        if (b2.row >= n_tgt) break;
+        turn(b2, d2);
+        if (b0.row >= n_tgt) break;
+    }
+}
+
+}  // namespace bmtk
+
+extern "C" int64_t bmtk_csr_propagate_pull_workspace_bytes(int32_t L, int64_t n_src)
+{
+    if (L <= 0 || n_src <= 0) return 0;
+    return (int64_t)L * ((n_src + 31) / 32) * 4;
+}
+
+extern "C" int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src,
+                                       int32_t batch, const int32_t *indptr, const bmtk_synapse *packed, float *syn,
+                                       int64_t n_tgt, int64_t t_arrive, void *workspace, void *stream)
+{
+    using namespace bmtk;
+    BMTK_REQUIRE(spike_hist && indptr && packed && syn && workspace, "csr_propagate_pull: pointers must be non-null");
+    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && n_src > 0 && t_arrive >= 0, "csr_propagate_pull: bad batch, sizes or step");
+    BMTK_REQUIRE(L > 1 && L <= 64, "csr_propagate_pull: L must lie in 2..64");
+    BMTK_REQUIRE(hist_stride >= (n_src * (int64_t)batch + 63) / 64 + 1,
+                 "csr_propagate_pull: hist_stride must hold ceil(n_src*batch/64)+1 words");
+    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31) && n_src < (1ll << 24), "csr_propagate_pull: network too large");
+    BMTK_REQUIRE((int64_t)L * hist_stride < (1ll << 29) && hist_stride < (1ll << 24),
+                 "csr_propagate_pull: spike history beyond 4 GiB");
+    const int n_w32 = (int)((n_src + 31) / 32);
+    const size_t lds = (size_t)L * n_w32 * 4 + kPullAccBytes;
+    BMTK_REQUIRE(lds <= kPullLdsMax, "csr_propagate_pull: L * n_src too large for the activity map in LDS");
+    uint32_t *any_map = (uint32_t *)workspace;
+    const int64_t map_threads = (int64_t)L * n_w32 * 32;
+    hipLaunchKernelGGL(pull_anymap_kernel, dim3((unsigned)((map_threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, spike_hist, hist_stride, L, batch, n_src, n_w32, any_map);
+    const unsigned rows_per_block = kPullBlock / kWave;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    static int cu_count[64];  // compute units of every device seen so far
+    int n_cu = (dev >= 0 && dev < 64) ? cu_count[dev] : 0;
+    if (n_cu <= 0) {
+        n_cu = 256;
+        (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (dev >= 0 && dev < 64) cu_count[dev] = n_cu;
+    }
+    const unsigned want = (unsigned)((n_tgt + rows_per_block - 1) / rows_per_block);
+    const unsigned cap = (unsigned)n_cu * 2u;  // persistent workgroups: the activity map is staged once per workgroup
+    const dim3 grid(want < cap ? want : cap, (unsigned)((batch + kWave - 1) / kWave));
+    BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_pull: batch too large");
+    // more than 64 KB of dynamic LDS has to be asked for, once per kernel and device
+    static bool asked[2][64];
+    if (dev >= 0 && dev < 64 && !asked[batch == kWave][dev]) {
+        const hipError_t err = hipFuncSetAttribute(
+            batch == kWave ? reinterpret_cast<const void *>(pull_kernel<true>) : reinterpret_cast<const void *>(pull_kernel<false>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPullLdsMax);
+        if (err != hipSuccess) {
+            set_error("csr_propagate_pull: cannot reserve %zu bytes of LDS: %s", kPullLdsMax, hipGetErrorString(err));
+            return BMTK_E_LAUNCH;
+        }
+        asked[batch == kWave][dev] = true;
+    }
+    if (batch == kWave)
+        hipLaunchKernelGGL(pull_kernel<true>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
+                           batch, indptr, packed, syn, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
+    else
+        hipLaunchKernelGGL(pull_kernel<false>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
+                           batch, indptr, packed, syn, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
+    BMTK_CHECK_LAUNCH("csr_propagate_pull");
+    return BMTK_OK;
+}

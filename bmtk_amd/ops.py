@@ -333,6 +333,24 @@ def csr_propagate_pull(spike_hist, n_src, table, syn, n_tgt, batch, t_arrive):
                                            int(t_arrive), _p(ws), _stream()))
 
 
+def csr_propagate_bwd(table, lam_ring, n, batch, step, gz=None, trials_per_lane=0):
+    """Transposed propagation (adjoint of the delivery) through a source-major table of ``n`` rows:
+    ``gz[j*batch+b] = sum_(j->i,w,d,r) w * lam_ring[(step+d) % L, r, i*batch+b]``.  ``trials_per_lane`` 0 lets the
+    library choose its kernel, 1 / 4 pick one (4 needs a batch that is a multiple of 4, at most 64)."""
+    lib = _lib.load()
+    L = lam_ring.shape[0]
+    if table.n_rows != n or lam_ring.numel() != L * NREC * n * batch:
+        raise ValueError("source-major table must have one row per neuron and lam_ring must be [L, 4, n*batch]")
+    if table.max_delay() >= L:
+        raise ValueError("adjoint ring of {} slots is shorter than the largest delay".format(L))
+    if gz is None:
+        gz = torch.empty(n * batch, device=lam_ring.device)
+    _lib.check(lib.bmtk_csr_propagate_bwd(_p(table.indptr, torch.int32), _p(table.packed()), n, batch,
+                                          _p(lam_ring, torch.float32), L, int(step),
+                                          _p(gz, torch.float32, n * batch, "gz"), int(trials_per_lane), _stream()))
+    return gz
+
+
 def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_active=None, zbits=None, n_src=None):
     """``mode`` "scatter" (source-major table + active list) or "gather"
     (target-major table + spike bits)."""

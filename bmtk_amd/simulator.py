@@ -15,6 +15,7 @@ from .layout import NPARAM, NPROP, NREC
 from .ops import Glif3State, SpikeCompactor, SynapseTable, _dev, _p, _stream, glif3_precompute, n_words, unpack_bits
 
 
+PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what is left of 80 KB beside its accumulators
 RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
 RES_ACT_ENTRIES = 8192          # active-row list of the resident kernel (kActCap of csrc/resident.hip), 4 B each
 RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static LDS (rounded up)
@@ -159,10 +160,10 @@ class Glif3Simulator:
         self.pull_table = self.pull_syn = self.pull_work = None
         self.pull_inp_table = self.pull_inp_syn = self.pull_inp_work = self.in_hist = None
         can_pull = (self.rec is not None and not self.res_span and self.delay_offset == 0
-                    and self.L * ((self.n + 31) // 32) * 4 + 16 * 1024 <= 64 * 1024)
+                    and self.L * ((self.n + 31) // 32) * 4 <= PULL_MAP_BYTES)
         if pull is True and not can_pull:
             raise ValueError("the pull form needs a recurrent table, launch-per-step mode, delay_offset 0 and "
-                             "ring_slots * n_neurons / 8 bytes of LDS (at most 48 KB)")
+                             "ring_slots * n_neurons / 8 bytes of LDS (at most 40 KB)")
         if can_pull and (pull is True or (pull == "auto" and self.batch >= 8)):
             self.pull_table = self.rec.transposed(self.n)
             self.pull_syn = torch.zeros(NREC, self.ne, device=self.dev)
@@ -171,7 +172,7 @@ class Glif3Simulator:
             # the history must hold one row per ring slot, row t % L = spikes of step t
             self.hist_slots = self.L
             self.work_bits = torch.zeros(self.hist_slots * (self.words + 1), dtype=torch.int64, device=self.dev)
-            if self.inp is not None and self.L * ((self.n_inputs + 31) // 32) * 4 + 16 * 1024 <= 64 * 1024:
+            if self.inp is not None and self.L * ((self.n_inputs + 31) // 32) * 4 <= PULL_MAP_BYTES:
                 self.pull_inp_table = self.inp.transposed(self.n)
                 self.pull_inp_syn = torch.zeros(NREC, self.ne, device=self.dev)
                 need = self.lib.bmtk_csr_propagate_pull_workspace_bytes(self.L, self.n_inputs)

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 9
+#define BMTK_AMD_ABI_VERSION 10
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -133,14 +133,16 @@ typedef struct bmtk_synapse {
  * packed TARGET-MAJOR table:
  *   syn[r][i*batch+b] = sum over synapses (j -> i, w, d, r) of w * bit(spike_hist[(t_arrive-d) mod L], j*batch+b)
  * syn ([4][n_tgt*batch]) is overwritten and is exactly the `syn` argument of
- * bmtk_glif3_step_fwd for step t_arrive.  One wavefront per target row, lane =
- * synapse, each lane adds its weight once per trial bit into LDS accumulators
- * (LDS atomics: the order of additions is not fixed).  A per-source "fired in
- * any trial" bit map of the L steps (built into `workspace`,
- * bmtk_csr_propagate_pull_workspace_bytes bytes, and staged in LDS) filters the
- * synapses whose source was silent, so the cost is one read of the table per
- * step plus one mask fetch per synapse with an active source.  L must exceed
- * the largest delay. */
+ * bmtk_glif3_step_fwd for step t_arrive.  A wavefront owns a target row at a time, lane = synapse; a per-source
+ * "fired in any trial" bit map of the L steps (built into `workspace`,
+ * bmtk_csr_propagate_pull_workspace_bytes bytes, and staged in LDS) filters the synapses whose source was
+ * silent, the others are gathered 64 at a time, fetch their source's trial mask and add their weight once per
+ * trial bit into LDS accumulators.  The accumulators are 64-bit fixed point (Q31.32) and the additions integer
+ * atomics, so the result does not depend on the order of the additions: it is the exact sum of the weights,
+ * rounded to fp32 once, the same in every run.  Weights must be finite and smaller than 2^31 in size; weight
+ * bits below 2^-32 are dropped.  The cost is one read of the table per step plus one mask fetch per synapse with
+ * an active source.  L must exceed the largest delay; L * hist_stride must stay below 2^29 words; the bit map,
+ * L * ceil(n_src/32) * 4 bytes, must fit in 40 KB of LDS (n_src <= 54,000 at L = 6). */
 int64_t bmtk_csr_propagate_pull_workspace_bytes(int32_t L, int64_t n_src);
 int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src, int32_t batch,
                             const int32_t *indptr, const bmtk_synapse *packed, float *syn, int64_t n_tgt,
@@ -363,6 +365,18 @@ typedef struct bmtk_glif3_bwd {
 /* Differentiate steps step0+n_steps-1 down to step0 (three launches per step:
  * transposed propagation, state adjoint, weight gradients). */
 int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_steps, void *stream);
+
+/* The transposed propagation of the backward pass on its own (the adjoint of the delivery; no counterpart in the
+ * reference): through a packed SOURCE-major table of n_neurons rows,
+ *   gz[j*batch+b] = sum over synapses (j -> i, w, d, r) of w * lam_ring[(step+d) % L][r][i*batch+b],
+ * lam_ring being [L][4][n_neurons*batch].  It is the exact transpose of the event-driven delivery: for spikes z
+ * emitted in `step`, <ring delivered from z, lam_ring> = <z, gz>.  One wavefront per source row; trials_per_lane
+ * picks the kernel: 1 = lane = (synapse, trial), any batch; 4 = four trials per lane and 16-byte reads of the
+ * adjoint rows, for batches that are a multiple of 4 up to 64; 0 = the one bmtk_glif3_simulate_bwd would take.
+ * Every element counts (bmtk_glif3_simulate_bwd skips rows whose surrogate derivative is zero in all trials). */
+int bmtk_csr_propagate_bwd(const int32_t *indptr, const bmtk_synapse *packed, int64_t n_neurons, int32_t batch,
+                           const float *lam_ring, int32_t L, int64_t step, float *gz, int32_t trials_per_lane,
+                           void *stream);
 
 /* Number of spikes of every element over n_steps rows of spike bits: counts[e] (int32). */
 int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_steps, int64_t ne, int32_t *counts,

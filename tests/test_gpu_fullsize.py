@@ -1,0 +1,220 @@
+"""Parity at the sizes the benchmarks time: the code paths small inputs never reach.
+
+The propagation kernels loop persistently over rows once there are more rows than resident wavefronts (8,192 on
+256 compute units), the scatter kernel strides once there are more active elements than wavefronts, and the
+backward kernels walk rows of 1,000 synapses with 16-byte adjoint reads at batch 32.  Weights here are multiples
+of a quarter pA, so every partial sum is exact in fp32 and results must agree BIT FOR BIT whatever the order of
+the additions; the checker is the fp32 oracle's row-by-row gather (``oracle.glif3_oracle.gather_rows``).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import glif3_oracle as orc
+from oracle import glif3_adjoint_ref as adj
+from bmtk_amd import network as net, ops, synthetic, training
+from bmtk_amd.simulator import Glif3Simulator
+from gpu_util import bits_of, to_dev
+
+pytestmark = pytest.mark.gpu
+
+N52K = 51978     # neurons of the isolated-propagation and training configurations
+
+
+def _quarter(w):
+    return (torch.round(w * 4.0) / 4.0 + torch.sign(w) * 0.25).to(torch.float32)
+
+
+def _network(n, mean_in, seed, L=6):
+    """Random network on the device with quarter-pA weights: (target-major, source-major) tables + host copies."""
+    by_tgt, by_src, _ = synthetic.device_network(n, mean_in, "poisson", seed=seed, max_delay=L - 1)
+    by_tgt = (by_tgt[0], by_tgt[1], _quarter(by_tgt[2]), by_tgt[3], by_tgt[4])
+    by_src = (by_src[0], by_src[1], _quarter(by_src[2]), by_src[3], by_src[4])
+    t_tgt = ops.SynapseTable.from_device(by_tgt, n, n, L)
+    t_src = ops.SynapseTable.from_device(by_src, n, n, L)
+    host_tgt = tuple(t.cpu().numpy() for t in by_tgt)
+    return t_tgt, t_src, host_tgt
+
+
+@pytest.mark.parametrize("rate_hz", [1.0, 5.0, 20.0])
+def test_propagation_at_52k_neurons_batch_64(rate_hz):
+    """51,978 rows x batch 64, in-degree ~120 (6.2 M synapses), spikes of L consecutive steps at 1 / 5 / 20 Hz:
+      - gather (deterministic) == fp32 oracle, the whole ring, bit for bit;
+      - pull (persistent row loop: 51,978 rows > 8,192 wavefronts) == the ring slot the gathers filled for the
+        arrival step, bit for bit;
+      - scatter (16.6 k and more active elements > 8,192 wavefronts at 5 and 20 Hz) == the same ring, bit for bit."""
+    n, batch, L = N52K, 64, 6
+    t_tgt, t_src, host_tgt = _network(n, 120, seed=21)
+    assert t_tgt.nnz > 6_000_000
+    ne = n * batch
+    rng = np.random.default_rng(int(rate_hz))
+    zs = [(rng.random(ne) < rate_hz * 1e-3).astype(np.uint8) for _ in range(L)]
+    bits = [to_dev(bits_of(z)) for z in zs]
+    hist = torch.stack(bits)
+    ring_o = np.zeros((L, 4, ne), np.float32)
+    ring_g = torch.zeros(L, 4, ne, device="cuda")
+    ring_s = torch.zeros(L, 4, ne, device="cuda")
+    comp = ops.SpikeCompactor(ne)
+    most_active = 0
+    for k in range(L):
+        orc.gather_rows(zs[k], batch, host_tgt, ring_o, n, k)
+        ops.csr_propagate_gather(bits[k], n, t_tgt, ring_g, n, batch, k)
+        ids, count = comp(to_dev(zs[k]))
+        most_active = max(most_active, int(count.item()))
+        ops.csr_propagate_scatter(ids, count, t_src, ring_s, n, batch, k)
+    assert np.abs(ring_o).max() > 0
+    if rate_hz >= 5.0:
+        assert most_active > 8192          # the scatter kernel's stride loop ran
+    np.testing.assert_array_equal(ring_g.cpu().numpy(), ring_o)
+    np.testing.assert_array_equal(ring_s.cpu().numpy(), ring_o)
+    # what arrives in step L: emitted in steps L-d, d = 1..L-1, i.e. slot 0 of a ring filled from steps 0..L-1
+    syn = torch.full((4, ne), 7.0, device="cuda")
+    ops.csr_propagate_pull(hist, n, t_tgt, syn, n, batch, L)
+    np.testing.assert_array_equal(syn.cpu().numpy(), ring_o[0])
+    # and the same call again: the pull form is deterministic
+    syn2 = torch.full((4, ne), -3.0, device="cuda")
+    ops.csr_propagate_pull(hist, n, t_tgt, syn2, n, batch, L)
+    assert torch.equal(syn, syn2)
+
+
+def test_pull_is_the_exact_sum_rounded_once_for_any_weights():
+    """Lognormal weights (not exactly summable in fp32): the pull kernel accumulates in 64-bit fixed point, so its
+    result is the exact sum rounded to fp32 -- equal to the fp64 oracle's sum rounded to fp32 wherever that sum is
+    itself exact, and the same in every run.  At 12,000 rows the persistent row loop runs."""
+    n, batch, L = 12000, 64, 6
+    by_tgt, by_src, _ = synthetic.device_network(n, 100, "poisson", seed=5, max_delay=L - 1)
+    t_tgt = ops.SynapseTable.from_device(by_tgt, n, n, L)
+    host = tuple(t.cpu().numpy() for t in by_tgt)
+    ne = n * batch
+    rng = np.random.default_rng(8)
+    zs = [(rng.random(ne) < 0.01).astype(np.uint8) for _ in range(L)]
+    hist = torch.stack([to_dev(bits_of(z)) for z in zs])
+    ring = np.zeros((L, 4, ne), np.float64)
+    for k in range(L):
+        orc.gather_rows(zs[k], batch, host, ring, n, k)
+    syn = torch.zeros(4, ne, device="cuda")
+    ops.csr_propagate_pull(hist, n, t_tgt, syn, n, batch, L)
+    got = syn.cpu().numpy()
+    want = ring[0].astype(np.float32)
+    assert np.abs(want).max() > 1.0
+    # fp64 sums of a few fp32 terms are exact except for rare cancellations: allow one fp32 unit on at most 1e-4 of
+    # the cells, none beyond
+    off = got != want
+    assert off.mean() < 1e-4
+    assert np.all(np.abs(got[off].astype(np.float64) - ring[0][off]) <= np.spacing(np.abs(want[off])))
+    again = torch.zeros(4, ne, device="cuda")
+    ops.csr_propagate_pull(hist, n, t_tgt, again, n, batch, L)
+    assert torch.equal(syn, again)
+
+
+def _adjoint_ring(rng, L, ne):
+    """Adjoint ring with values that are multiples of 1/8 in -4..4: products with quarter weights and their sums
+    stay exact in fp32."""
+    return (rng.integers(-32, 33, (L, 4, ne)) / 8.0).astype(np.float32)
+
+
+@pytest.mark.parametrize("batch", [32, 64, 8])
+def test_transposed_propagation_at_12k_neurons(batch):
+    """12,000 source rows of ~400 synapses at batch 32 (the training configuration's batch), 64 and 8:
+      - four trials per lane == one trial per lane, bit for bit (exact operands);
+      - both equal W^T lambda computed on the host from the transposed table;
+      - the adjoint identity <deliver(z), lambda> = <z, W^T lambda> against the forward gather kernel."""
+    n, L, step = 12000, 6, 3
+    t_tgt, t_src, host_tgt = _network(n, 400, seed=31)
+    ne = n * batch
+    rng = np.random.default_rng(batch)
+    lam = _adjoint_ring(rng, L, ne)
+    lam_d = to_dev(lam)
+    g1 = ops.csr_propagate_bwd(t_src, lam_d, n, batch, step, trials_per_lane=1)
+    g4 = ops.csr_propagate_bwd(t_src, lam_d, n, batch, step, trials_per_lane=4)
+    g0 = ops.csr_propagate_bwd(t_src, lam_d, n, batch, step)
+    assert torch.equal(g1, g4) and torch.equal(g0, g4)
+    # host: gz[j, b] = sum over synapses (j -> i) of w * lam[(step + d) % L, r, i, b], from the target-major copy
+    indptr, src, w, d, r = host_tgt
+    tgt = np.repeat(np.arange(n), np.diff(indptr))
+    want = np.zeros((n, batch), np.float64)
+    cells = lam.reshape(L, 4, n, batch)[(step + d.astype(np.int64)) % L, r, tgt]        # [nnz, batch]
+    np.add.at(want, src, w[:, None].astype(np.float64) * cells)
+    np.testing.assert_array_equal(g4.cpu().numpy().reshape(n, batch), want.astype(np.float32))
+    # adjoint identity with the forward kernel: spikes z emitted in `step`
+    z = (rng.random(ne) < 0.02).astype(np.uint8)
+    ring = torch.zeros(L, 4, ne, device="cuda")
+    ops.csr_propagate_gather(to_dev(bits_of(z)), n, t_tgt, ring, n, batch, step)
+    lhs = float((ring.double() * lam_d.double()).sum().item())
+    rhs = float((to_dev(z).double() * g4.double()).sum().item())
+    assert abs(lhs) > 100.0
+    assert abs(lhs - rhs) <= 1e-5 * abs(lhs)      # exact operands: in fact equal up to the fp64 summation
+
+
+def _net_cfg(n, n_in, batch, steps, seed, in_rate, in_w, w_scale, p_conn, in_fanout):
+    cfg = synthetic.small_glif3_network(n=n, n_in=n_in, steps=steps, seed=seed, in_rate=in_rate, in_w_scale=in_w,
+                                        w_scale=w_scale, in_fanout=in_fanout, p_conn=p_conn, batch=batch)
+    for k in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = cfg[k]
+        cfg[k] = (indptr, indices, (np.round(w * 4.0) / 4.0 + np.sign(w) * 0.25).astype(np.float32), d, r)
+    return cfg
+
+
+def test_weight_gradients_match_autograd_over_many_rows_and_long_event_lists():
+    """600 neurons, 3,000 input sources at 100 Hz, batch 4: 150 row blocks per backward launch, and about 1,200
+    input events per step -- more than the 1,024 wavefronts of the input-gradient kernel, so its stride loop runs.
+    Against torch.autograd over the fp64 restatement; tolerance 1e-4 of the table's largest gradient."""
+    batch, T = 4, 24
+    cfg = _net_cfg(n=600, n_in=3000, batch=batch, steps=T, seed=13, in_rate=100.0, in_w=1.5, w_scale=3.0,
+                   p_conn=0.08, in_fanout=40)
+    n, h = cfg["n"], cfg["h"]
+    ne = n * batch
+    assert np.diff(cfg["in_ptr"]).max() > 1024
+    prop = orc.precompute(cfg["par"], h)
+    sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                         resident=False)
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    fwd = sim.run(T, save_state=True)
+    ras = sim.raster(fwd["bits"]).cpu().numpy()
+    a = np.random.default_rng(3).normal(size=(T, ne))
+    bptt = training.Glif3Bptt(sim, dampening=0.3)
+    bptt.backward(fwd, dl_dz=torch.as_tensor(a.astype(np.float32), device="cuda"))
+    want = adj.simulate_with_grad(prop, h, T, n, batch, cfg["L"], cfg["rec_src"], cfg["inp_src"], cfg["in_ptr"],
+                                  cfg["in_events"], lambda z: (z * torch.as_tensor(a)).sum(), dampening=0.3)
+    np.testing.assert_array_equal(ras, want["raster"])
+    assert ras.sum() > 200 * batch
+    for got, ref in ((bptt.d_rec_w, want["d_rec_w"]), (bptt.d_inp_w, want["d_inp_w"])):
+        ref_max = np.abs(ref).max()
+        assert ref_max > 0
+        assert np.abs(got.cpu().numpy() - ref).max() < 1e-4 * ref_max
+
+
+def test_backward_at_10k_neurons_batch_32_chunked_equals_one_call():
+    """10,000 neurons x batch 32, ~100 synapses per row, 40 steps: the backward pass in one call and as three chunks
+    in reverse time order give the same gradients (to 1e-6 of the largest; the additions happen in the same order),
+    and the forward run they differentiate is the fp32 oracle's, spike for spike."""
+    n, batch, T = 10000, 32, 40
+    cfg = _net_cfg(n=n, n_in=2000, batch=batch, steps=T, seed=17, in_rate=60.0, in_w=4.0, w_scale=2.0,
+                   p_conn=0.01, in_fanout=200)
+    h = cfg["h"]
+    ne = n * batch
+    prop = orc.precompute(cfg["par"], h)
+    st = orc.new_state(n, batch, np.float32)
+    ring = np.zeros((cfg["L"], 4, ne), np.float32)
+    want = orc.simulate(st, prop, h, T, batch=batch, ring=ring, rec=cfg["rec_src"], inp=cfg["inp_src"],
+                        in_ptr=cfg["in_ptr"], in_events=cfg["in_events"], raster=True)
+    assert want["count"] > 20 * batch
+    a = torch.as_tensor(np.random.default_rng(1).normal(size=(T, ne)).astype(np.float32), device="cuda")
+    grads = []
+    for chunks in ([T], [15, 14, 11]):
+        sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"],
+                             ring_slots=cfg["L"], resident=False)
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        runs, k0 = [], 0
+        for c in chunks:
+            runs.append((sim.run(c, save_state=True), k0, c))
+            k0 += c
+        ras = np.concatenate([sim.raster(f["bits"]).cpu().numpy() for f, _, _ in runs])
+        np.testing.assert_array_equal(ras, want["raster"])
+        bptt = training.Glif3Bptt(sim)
+        for f, k0, c in reversed(runs):
+            bptt.backward(f, dl_dz=a[k0:k0 + c].contiguous())
+        grads.append((bptt.d_rec_w.cpu().numpy(), bptt.d_inp_w.cpu().numpy()))
+    for one, three in zip(grads[0], grads[1]):
+        assert np.abs(one).max() > 0
+        np.testing.assert_allclose(one, three, rtol=0, atol=1e-6 * np.abs(one).max())

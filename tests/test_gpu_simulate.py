@@ -426,8 +426,8 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     """Two spikes of one generator inside one resolution step are two deliveries.  Every driver must count them:
     the launch-per-step driver, the resident one, and the batched driver whose pull form of the inputs (bit rows:
     one bit per id and step) steps aside for such lists.  Exact weights: bit-identical to the fp32 oracle."""
-    cfg = synthetic.small_glif3_network(n=700, n_in=300, steps=300, seed=14, in_w_scale=2.0, in_fanout=100,
-                                        p_conn=0.05, w_scale=1.5, batch=batch)
+    cfg = synthetic.small_glif3_network(n=700, n_in=300, steps=300, seed=14, in_w_scale=3.0, in_fanout=100,
+                                        in_rate=30.0, p_conn=0.05, w_scale=1.5, batch=batch)
     cfg["rec_src"] = _integer_weights(cfg["rec_src"])
     cfg["inp_src"] = _integer_weights(cfg["inp_src"])
     in_ptr, in_events = _with_duplicate_events(cfg, np.random.default_rng(3), batch)
