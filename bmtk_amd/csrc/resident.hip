@@ -107,12 +107,29 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
     const SegBounds sb = *reinterpret_cast<const SegBounds *>(seg_row + g);
     const uint32_t lo = sb.lo, hi = sb.hi;
     const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(tab);
-    auto add = [&](const uint2 sy) {
+    // An LDS float atomic costs about three clocks per LANE on gfx950 (its lanes are worked off one after the
+    // other), an integer compare-and-swap a few clocks per INSTRUCTION.  Where most lanes of a wavefront take
+    // part -- the first two synapses of the segments -- the addition is therefore a compare-and-swap loop (a
+    // lane repeats only if another thread changed its cell in between, which is rare among 23,000 cells); the
+    // thinly populated later ones keep the float atomic.  The sum is the same either way.
+    auto add = [&](const uint2 sy, bool crowded) {
         int slot = slot0 + (int)(sy.x >> 26);
         slot = slot >= L ? slot - L : slot;
         const int r = (sy.x >> 24) & 3;
         const int i = (int)(sy.x & 0xFFFFFFu) - e0;
-        atomicAdd(ring_l + (slot * GLIF3_NREC + r) * span + i, __uint_as_float(sy.y));
+        float *cell = ring_l + (slot * GLIF3_NREC + r) * span + i;
+        const float w = __uint_as_float(sy.y);
+        if (!crowded) {
+            atomicAdd(cell, w);
+            return;
+        }
+        unsigned *bits = reinterpret_cast<unsigned *>(cell);
+        unsigned old = *reinterpret_cast<volatile unsigned *>(bits);
+        while (true) {
+            const unsigned seen = atomicCAS(bits, old, __float_as_uint(__uint_as_float(old) + w));
+            if (seen == old) break;
+            old = seen;
+        }
     };
     // all of a segment's loads go out together: a loop of dependent loads for the few long segments would
     // hold up the whole wavefront (1 in 25 segments has more than 3 synapses, 1 in 5000 more than 6)
@@ -123,8 +140,8 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
         if (lo + (uint32_t)u < hi) first[u] = rows[lo + (uint32_t)u];
 #pragma unroll
     for (int u = 0; u < kTogether; ++u)
-        if (lo + (uint32_t)u < hi) add(first[u]);
-    for (uint32_t p = lo + (uint32_t)kTogether; p < hi; ++p) add(rows[p]);
+        if (lo + (uint32_t)u < hi) add(first[u], u < 2);
+    for (uint32_t p = lo + (uint32_t)kTogether; p < hi; ++p) add(rows[p], false);
 }
 
 constexpr int kScanWords = 4;   // ballot words per thread and round
