@@ -116,3 +116,39 @@ def test_backward_argument_errors():
     z = torch.zeros(5, cfg["n"], device="cuda")
     with pytest.raises(BmtkAmdError):
         bptt.backward(fwd, dl_dz=z, dl_dz_const=z[0].contiguous())
+
+
+def test_state_adjoint_kernel_transposes_the_state_update():
+    """<J v, u> = <v, J^T u> on the device for the linear part of the update (leak, after-spike currents, both PSC
+    states) over three steps: J v as the difference of two forward runs of the step kernels from states x and x + v
+    that stay below threshold, J^T u from the backward pass started with the adjoint state u and no loss.  fp32
+    throughout: the identity is held to 1e-4 of its size."""
+    n, batch, T = 3000, 4, 3
+    ne = n * batch
+    rng = np.random.default_rng(21)
+    par = synthetic.random_cells(rng, n)
+    prop = orc.precompute(par, 1.0)
+    th = np.repeat(prop[orc.L["GLIF3_TH"]], batch)
+    x0 = dict(V=(0.3 * th * rng.random(ne)).astype(np.float32), asc=rng.uniform(-2, 2, (2, ne)).astype(np.float32),
+              y1=rng.uniform(0, 0.05, (4, ne)).astype(np.float32), y2=rng.uniform(0, 0.05, (4, ne)).astype(np.float32))
+    v = {k: (rng.normal(size=a.shape) * 0.25 * (np.abs(a).mean() + 1e-3)).astype(np.float32) for k, a in x0.items()}
+    u = {k: rng.normal(size=a.shape).astype(np.float32) for k, a in x0.items()}
+
+    def forward(x):
+        sim = Glif3Simulator(n, par, 1.0, batch=batch, resident=False)
+        for k in x:
+            getattr(sim.state, k).copy_(torch.as_tensor(x[k], device="cuda").reshape(getattr(sim.state, k).shape))
+        fwd = sim.run(T, save_state=True)
+        assert int(sim.raster(fwd["bits"]).sum().item()) == 0
+        return sim, fwd, {k: getattr(sim.state, k).double().cpu().numpy().reshape(x[k].shape) for k in x}
+    sim, fwd, a = forward(x0)
+    _, _, b = forward({k: x0[k] + v[k] for k in x0})
+    lhs = sum(float(((b[k] - a[k]) * u[k].astype(np.float64)).sum()) for k in x0)
+    bptt = training.Glif3Bptt(sim, dampening=0.3)
+    for k, t in (("V", bptt.lam_V), ("asc", bptt.lam_asc), ("y1", bptt.lam_y1), ("y2", bptt.lam_y2)):
+        t.copy_(torch.as_tensor(u[k], device="cuda").reshape(t.shape))
+    bptt.backward(fwd, dl_dz=torch.zeros(T, ne, device="cuda"))
+    jt_u = dict(V=bptt.lam_V, asc=bptt.lam_asc, y1=bptt.lam_y1, y2=bptt.lam_y2)
+    rhs = sum(float((jt_u[k].double().cpu().numpy().reshape(v[k].shape) * v[k].astype(np.float64)).sum()) for k in x0)
+    assert abs(lhs) > 1.0
+    assert abs(lhs - rhs) <= 1e-4 * abs(lhs), (lhs, rhs)
