@@ -225,9 +225,16 @@ def bench_bptt(torch, steps=600):
     Poisson inputs at 5 Hz, batch 32, 600 steps; triangular surrogate (dampening 0.3); MSE between
     the rates of 17 random populations and random targets; gradients for every recurrent and input
     weight.  Recurrent weights are scaled by 0.2 and input weights by 2 so that the network settles
-    near 3 Hz (unit weights at this in-degree saturate it)."""
+    near 3 Hz (unit weights at this in-degree saturate it).
+
+    Returns two entries: the training step, and the transposed propagation on its own (the kernel that
+    takes most of the backward pass), timed through bmtk_csr_propagate_bwd on the same table.
+    Rooflines use the bytes that MUST cross HBM: per backward step the packed table once (8 B per synapse),
+    the adjoint ring slots once (L-1 slots x 4 receptors x ne x 4 B), the adjoint state in and out, the
+    forward record (potential and flags) and the input gradient's reads; not the L2 fills the kernels cause by
+    fetching an adjoint row per synapse (those are in `traffic`)."""
     import numpy as np
-    from bmtk_amd import synthetic, training
+    from bmtk_amd import ops, synthetic, training
     from bmtk_amd.simulator import Glif3Simulator
     n, n_in, batch = 51978, 17400, 32
     rng = np.random.default_rng(4)
@@ -237,8 +244,9 @@ def bench_bptt(torch, steps=600):
     in_ptr, in_ev = synthetic.device_poisson_events(n_in, 5.0, 1.0, 2 * steps, batch=batch, seed=5)
     sim = Glif3Simulator(n, par, 1.0, batch=batch, rec=by_src, inp=inp, resident=False)
     sim.set_input_events(in_ptr, in_ev)
-    pop = torch.randint(0, 17, (n,), device="cuda")
-    targets = torch.rand(batch, 17, device="cuda") * 0.01
+    g = torch.Generator(device="cuda").manual_seed(11)
+    pop = torch.randint(0, 17, (n,), device="cuda", generator=g)
+    targets = torch.rand(batch, 17, device="cuda", generator=g) * 0.01
     bptt = training.Glif3Bptt(sim, dampening=0.3)
     res = {}
 
@@ -258,14 +266,48 @@ def bench_bptt(torch, steps=600):
     deg = (sim.rec.indptr[1:] - sim.rec.indptr[:-1]).long()
     spikes = res["counts"].view(n, batch).sum(1)
     events = int((spikes.long() * deg).sum().item())
-    return {"kernel": "sim_step_kernel + pull_kernel (forward), bwd_gather4_kernel + bwd_state_kernel + bwd_rec_grad_kernel + "
-                      "bwd_inp_grad_kernel (backward)",
-            "workload": "BPTT step N=51978 nnz=%d inputs=17400 batch=32 steps=%d" % (sim.rec.nnz, steps),
-            "seconds_per_training_step": t_f + t_b, "forward_s": t_f, "backward_s": t_b,
-            "mean_rate_hz": float(res["counts"].float().mean().item()) / steps * 1e3,
-            "recurrent_events_forward": events, "loss": float(res["loss"]),
-            "weight_grad_events_per_s": events / t_b,
-            "grad_norm_rec": float(bptt.d_rec_w.norm().item()), "grad_norm_inp": float(bptt.d_inp_w.norm().item())}
+    ne, L, nnz, nnz_in = sim.ne, sim.L, sim.rec.nnz, sim.inp.nnz
+    ring_bytes = (L - 1) * 4 * ne * 4
+    # backward, per step: table + adjoint slots (transposed propagation), 11 adjoint state words in and out + the
+    # new slot out + potential and flags in (state adjoint), the input table rows of the step's events
+    bwd_step = nnz * 8 + ring_bytes + ne * (11 * 8 + 16 + 5) + (in_ev.numel() / (2 * steps)) * (nnz_in / n_in) * 8
+    # forward, per step: target-major table once (pull form) + 12 state words in and out + record out
+    fwd_step = nnz * 8 + ne * (12 * 8 + 16 + 5)
+    step_entry = {
+        "kernel": "sim_step_kernel + pull_kernel (forward), bwd_gather4_kernel + bwd_state_kernel + bwd_inp_grad_kernel "
+                  "(backward; the recurrent weight gradient rides in bwd_gather4_kernel)",
+        "workload": "BPTT step N=51978 nnz=%d inputs=17400 batch=32 steps=%d" % (nnz, steps),
+        "seconds_per_training_step": t_f + t_b, "forward_s": t_f, "backward_s": t_b,
+        "mean_rate_hz": float(res["counts"].float().mean().item()) / steps * 1e3,
+        "recurrent_events_forward": events, "loss": float(res["loss"]),
+        "weight_grad_events_per_s": events / t_b,
+        "grad_norm_rec": float(bptt.d_rec_w.norm().item()), "grad_norm_inp": float(bptt.d_inp_w.norm().item()),
+        "roofline": {"bound": "hbm", "achieved": bwd_step * steps / t_b / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bwd_step * steps / t_b / 1e9 / HBM_PEAK_GBS, "what": "backward pass, HBM-compulsory bytes",
+                     "algorithmic_bytes_per_step": bwd_step,
+                     "traffic": profile_traffic("backward_kernels_52k_batch32.txt", "hbm_bytes_per_backward_step")},
+        "roofline_forward": {"bound": "hbm", "achieved": fwd_step * steps / t_f / 1e9, "peak": HBM_PEAK_GBS,
+                             "unit": "GB/s", "frac": fwd_step * steps / t_f / 1e9 / HBM_PEAK_GBS,
+                             "algorithmic_bytes_per_step": fwd_step}}
+    # the transposed propagation alone, every row active
+    lam = torch.randn(L, 4, ne, device="cuda", generator=g)
+    gz = torch.empty(ne, device="cuda")
+    for k in range(5):
+        ops.csr_propagate_bwd(sim.rec, lam, n, batch, k, gz=gz)
+    reps = 50
+    _, dev = time_region(torch, lambda: [ops.csr_propagate_bwd(sim.rec, lam, n, batch, k, gz=gz) for k in range(reps)])
+    per = dev / reps
+    alg = nnz * 8 + ring_bytes + ne * 4
+    gather_entry = {
+        "kernel": "bwd_gather4_kernel", "workload": "transposed propagation N=51978 nnz=%d batch=32, every row" % nnz,
+        "us_per_launch": per * 1e6, "synapse_trials_per_s": nnz * batch / per,
+        "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg / per / 1e9 / HBM_PEAK_GBS, "what": "HBM-compulsory bytes: table + adjoint ring + output once",
+                     "algorithmic_bytes_per_launch": alg,
+                     "traffic": profile_traffic("backward_kernels_52k_batch32.txt", "l2_fill_bytes_per_launch_bwd_gather4"),
+                     "traffic_note": "L2 fills (one 128-byte adjoint row per synapse, served mostly by the memory-side "
+                                     "cache), not HBM bytes"}}
+    return [step_entry, gather_entry]
 
 
 def cpu_baseline(torch, sim, par, class_id, settled, sample_steps):
@@ -450,7 +492,7 @@ def main():
         line["kernels"] = ((bench_state_update(torch) if "state" in want else []) +
                            (bench_compaction(torch) if "compaction" in want else []) +
                            (bench_propagation(torch) if "propagation" in want else []) +
-                           ([bench_bptt(torch)] if "bptt" in want else []))
+                           (bench_bptt(torch) if "bptt" in want else []))
     if args.cpu_steps > 0:
         line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, settled, max(CPU_MIN_STEPS, args.cpu_steps))
     print(json.dumps(line))

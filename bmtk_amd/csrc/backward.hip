@@ -17,6 +17,18 @@ __device__ __forceinline__ float surrogate(float U, float th, float dampening)
     return dampening * fmaxf(0.0f, 1.0f - fabsf(vhat)) / th;
 }
 
+__device__ __forceinline__ unsigned long long trial_mask(const uint64_t *__restrict__ bits, int64_t j, int batch,
+                                                         int tile0, int width)
+{
+    const int64_t bit = j * batch + tile0;
+    const int64_t w = bit >> 6;
+    const int sh = (int)(bit & 63);
+    unsigned long long m = bits[w] >> sh;
+    if (sh + width > 64) m |= bits[w + 1] << (64 - sh);
+    if (width < 64) m &= (1ull << width) - 1ull;
+    return m;
+}
+
 // gz[j*B+b] = sum over out-going synapses (j -> i, w, d, r) of w * lam_ring[(t+d)%L][r][i*B+b]:
 // one wavefront per source neuron and trial tile.  A tile is `bp` trials wide
 // (the batch rounded up to a power of two, at most 64) and the wavefront's 64
@@ -24,6 +36,11 @@ __device__ __forceinline__ float surrogate(float U, float th, float dampening)
 // synapse's adjoint row (bp*4 contiguous bytes per synapse); four such groups
 // are in flight before their products are added.  Rows whose every trial has
 // a zero surrogate derivative in this step are skipped.
+// kGrad (batches of one tile only): the recurrent weight gradient of the step rides along.  The wavefront has a
+// synapse's adjoint row in registers anyway; where the source fired in some trial of this step, the entries of
+// those trials are summed over the row's lanes and added to d_rec_w[p] -- this wavefront is the only writer of
+// its row.  A separate kernel would fetch every such adjoint row a second time to use one or two words of it.
+template <bool kGrad>
 __global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, BwdStep q, int bp)
 {
     const int batch = a.batch;
@@ -46,7 +63,10 @@ __global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, Bw
             active = fabsf((a.save_v[q.row * ne + e] - th) / th) < 1.0f;
         }
     }
-    if (__ballot(active) == 0ull) {
+    // trials in which source j fired in this step (the same in all lanes)
+    const unsigned long long fired = kGrad ? trial_mask(a.spike_bits + q.row * a.spike_bits_stride, j, batch, 0, batch) : 0ull;
+    const bool mine = lane_on && ((fired >> b) & 1ull);
+    if (__ballot(active) == 0ull && fired == 0ull) {
         if (lane_on && sub == 0) a.gz[e] = 0.0f;
         return;
     }
@@ -72,10 +92,19 @@ __global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, Bw
                 slot = slot >= L ? slot - L : slot;
                 const int r = (tdr >> 24) & 3;
                 const int64_t i = tdr & 0xFFFFFFu;
-                v[u] = (active && idx < n_here) ? ring[(int64_t)(slot * GLIF3_NREC + r) * ne + i * batch] : 0.0f;
+                v[u] = ((active || mine) && idx < n_here) ? ring[(int64_t)(slot * GLIF3_NREC + r) * ne + i * batch] : 0.0f;
             }
 #pragma unroll
-            for (int u = 0; u < kInFlight; ++u) acc += w[u] * v[u];
+            for (int u = 0; u < kInFlight; ++u) acc += active ? w[u] * v[u] : 0.0f;
+            if (kGrad && fired != 0ull) {
+#pragma unroll
+                for (int u = 0; u < kInFlight; ++u) {
+                    float g = mine ? v[u] : 0.0f;
+                    for (int off = 1; off < bp; off <<= 1) g += __shfl_xor(g, off, kWave);
+                    const int idx = l0 + u * per + sub;
+                    if (b == 0 && idx < n_here) a.d_rec_w[base + idx] += g;
+                }
+            }
         }
     }
     for (int off = bp; off < kWave; off <<= 1) acc += __shfl_xor(acc, off, kWave);
@@ -86,6 +115,7 @@ __global__ __launch_bounds__(kBlock) void bwd_gather_kernel(bmtk_glif3_bwd a, Bw
 // adjoint row (batch*4 contiguous bytes) is read by lp = bp/4 lanes as 16-byte pieces, so one wavefront
 // instruction covers 64/lp synapses (8 at batch 32) and the address arithmetic and lane exchanges per synapse
 // shrink fourfold.  Partial sums of the 64/lp synapse lanes are folded at the end.
+template <bool kGrad>
 __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, BwdStep q, int lp)
 {
     const int batch = a.batch;
@@ -109,7 +139,10 @@ __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, B
         for (int c = 0; c < 4; ++c)
             if (((f4 >> (8 * c)) & BMTK_F_INTEGRATING) && fabsf((v[c] - th) / th) < 1.0f) act |= 1u << c;
     }
-    if (__ballot(act != 0u) == 0ull) {
+    // trials in which source j fired in this step (the same in all lanes), and this lane's four of them
+    const unsigned long long fired = kGrad ? trial_mask(a.spike_bits + q.row * a.spike_bits_stride, j, batch, 0, batch) : 0ull;
+    const unsigned mine = lane_on ? (unsigned)(fired >> b4) & 0xFu : 0u;
+    if (__ballot(act != 0u) == 0ull && fired == 0ull) {
         if (lane_on && sub == 0) *reinterpret_cast<float4 *>(a.gz + e) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         return;
     }
@@ -136,7 +169,7 @@ __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, B
                 slot = slot >= L ? slot - L : slot;
                 const int r = (tdr >> 24) & 3;
                 const int64_t i = tdr & 0xFFFFFFu;
-                v[u] = (act != 0u && idx < n_here)
+                v[u] = ((act | mine) != 0u && idx < n_here)
                            ? *reinterpret_cast<const float4 *>(ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch)
                            : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             }
@@ -146,6 +179,16 @@ __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, B
                 acc[1] += w[u] * v[u].y;
                 acc[2] += w[u] * v[u].z;
                 acc[3] += w[u] * v[u].w;
+            }
+            if (kGrad && fired != 0ull) {
+#pragma unroll
+                for (int u = 0; u < kInFlight; ++u) {
+                    float g = ((mine & 1u) ? v[u].x : 0.0f) + ((mine & 2u) ? v[u].y : 0.0f) +
+                              ((mine & 4u) ? v[u].z : 0.0f) + ((mine & 8u) ? v[u].w : 0.0f);
+                    for (int off = 1; off < lp; off <<= 1) g += __shfl_xor(g, off, kWave);
+                    const int idx = l0 + u * per + sub;
+                    if (b4 == 0 && idx < n_here) a.d_rec_w[base + idx] += g;
+                }
             }
         }
     }
@@ -219,18 +262,6 @@ __global__ __launch_bounds__(kBlock) void bwd_state_kernel(bmtk_glif3_bwd a, Bwd
         a.lam_y1[k * ne + e] = n1[k];
         a.lam_y2[k * ne + e] = n2[k];
     }
-}
-
-__device__ __forceinline__ unsigned long long trial_mask(const uint64_t *__restrict__ bits, int64_t j, int batch,
-                                                         int tile0, int width)
-{
-    const int64_t bit = j * batch + tile0;
-    const int64_t w = bit >> 6;
-    const int sh = (int)(bit & 63);
-    unsigned long long m = bits[w] >> sh;
-    if (sh + width > 64) m |= bits[w + 1] << (64 - sh);
-    if (width < 64) m &= (1ull << width) - 1ull;
-    return m;
 }
 
 // d_rec_w[p] += sum over trials b in which source j spiked in step t of
@@ -358,14 +389,26 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
     while (bp < a.batch && bp < kWave) bp <<= 1;
     for (int64_t k = n_steps - 1; k >= 0; --k) {
         BwdStep q{step0 + k, k};
-        if (has_rec && a.batch % 4 == 0 && a.batch <= kWave)
-            hipLaunchKernelGGL(bwd_gather4_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q, bp / 4);
-        else if (has_rec)
-            hipLaunchKernelGGL(bwd_gather_kernel, dim3(rows_grid, tiles), dim3(kBlock), 0, st, a, q, bp);
-        else
+        // The recurrent weight gradient of step t reads the adjoint slots t+1 .. t+L-1, which the state adjoint of
+        // this step (it writes slot t) leaves alone: it can ride along with the transposed propagation, which
+        // reads the same slots before the state adjoint runs.  Batches of more than one tile keep the kernel of
+        // their own (several wavefronts would share a row).
+        const bool fused = a.d_rec_w && tiles == 1;
+        if (has_rec && a.batch % 4 == 0 && a.batch <= kWave) {
+            if (fused)
+                hipLaunchKernelGGL(bwd_gather4_kernel<true>, dim3(rows_grid), dim3(kBlock), 0, st, a, q, bp / 4);
+            else
+                hipLaunchKernelGGL(bwd_gather4_kernel<false>, dim3(rows_grid), dim3(kBlock), 0, st, a, q, bp / 4);
+        } else if (has_rec) {
+            if (fused)
+                hipLaunchKernelGGL(bwd_gather_kernel<true>, dim3(rows_grid, tiles), dim3(kBlock), 0, st, a, q, bp);
+            else
+                hipLaunchKernelGGL(bwd_gather_kernel<false>, dim3(rows_grid, tiles), dim3(kBlock), 0, st, a, q, bp);
+        } else {
             hipLaunchKernelGGL(fill_zero_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a.gz, ne);
+        }
         hipLaunchKernelGGL(bwd_state_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q);
-        if (a.d_rec_w) hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
+        if (a.d_rec_w && !fused) hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
         if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(256), dim3(kBlock), 0, st, a, q);
     }
     BMTK_CHECK_LAUNCH("glif3_simulate_bwd");
@@ -396,9 +439,9 @@ extern "C" int bmtk_csr_propagate_bwd(const int32_t *indptr, const bmtk_synapse 
     int bp = 1;
     while (bp < batch && bp < kWave) bp <<= 1;
     if (trials_per_lane == 4 || (trials_per_lane == 0 && can4))
-        hipLaunchKernelGGL(bwd_gather4_kernel, dim3(rows_grid), dim3(kBlock), 0, (hipStream_t)stream, a, q, bp / 4);
+        hipLaunchKernelGGL(bwd_gather4_kernel<false>, dim3(rows_grid), dim3(kBlock), 0, (hipStream_t)stream, a, q, bp / 4);
     else
-        hipLaunchKernelGGL(bwd_gather_kernel, dim3(rows_grid, (unsigned)((batch + kWave - 1) / kWave)), dim3(kBlock), 0,
+        hipLaunchKernelGGL(bwd_gather_kernel<false>, dim3(rows_grid, (unsigned)((batch + kWave - 1) / kWave)), dim3(kBlock), 0,
                            (hipStream_t)stream, a, q, bp);
     BMTK_CHECK_LAUNCH("csr_propagate_bwd");
     return BMTK_OK;
