@@ -195,11 +195,14 @@ def bench_propagation(torch, steps=200, warmup=20):
         events = sum(e for _, _, e in pool_ev) / len(pool_ev)
         hist = torch.stack([pool_bits[k % 4] for k in range(L)])   # spike bits of the last L steps
         syn = torch.zeros(4, ne, device="cuda")
-        for mode in ("scatter", "gather", "pull"):
+        for mode in ("scatter", "gather", "auto", "pull"):
             def one(k):
                 if mode == "scatter":
                     ids, count, _ = pool_ev[k % 4]
                     ops.csr_propagate_scatter(ids, count, t_src, ring, n, batch, k)
+                elif mode == "auto":
+                    ids, count, _ = pool_ev[k % 4]
+                    ops.csr_propagate_auto(ids, count, pool_bits[k % 4], n, t_src, t_tgt, ring, n, batch, k)
                 elif mode == "gather":
                     ops.csr_propagate_gather(pool_bits[k % 4], n, t_tgt, ring, n, batch, k)
                 else:
@@ -210,7 +213,8 @@ def bench_propagation(torch, steps=200, warmup=20):
             wall, dev = time_region(torch, lambda: [one(k) for k in range(steps)])
             per = dev / steps
             alg = events * B_PER_EVENT
-            out.append({"kernel": mode + "_kernel", "workload": "propagation N=51978 nnz=%d batch=64 rate=%gHz" %
+            out.append({"kernel": "scatter_kernel or gather_kernel, chosen on the device" if mode == "auto" else
+                        mode + "_kernel", "workload": "propagation N=51978 nnz=%d batch=64 rate=%gHz" %
                         (t_src.nnz, rate), "events_per_launch": events, "synaptic_events_per_s": events / per,
                         "us_per_launch": per * 1e6,
                         "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS,

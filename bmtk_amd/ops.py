@@ -351,14 +351,38 @@ def csr_propagate_bwd(table, lam_ring, n, batch, step, gz=None, trials_per_lane=
     return gz
 
 
-def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_active=None, zbits=None, n_src=None):
-    """``mode`` "scatter" (source-major table + active list) or "gather"
-    (target-major table + spike bits)."""
+def csr_propagate_auto(active, n_active, zbits, n_src, table_src, table_tgt, ring, n_tgt, batch, step,
+                       scatter_max_active=None, max_active=None):
+    """Delivery with the form chosen on the device (no host synchronisation): the event-driven scatter up to
+    ``scatter_max_active`` active elements, the row-wise gather above.  Default threshold: a fifth of the source
+    rows per 64 trials, the measured break-even of the two kernels on one MI355X."""
+    lib = _lib.load()
+    L = ring.shape[0]
+    if ring.numel() != L * NREC * n_tgt * batch or table_tgt.n_rows != n_tgt or table_src.n_rows != n_src:
+        raise ValueError("ring must be [L, 4, n_tgt*batch]; tables must have one row per source / per target")
+    if scatter_max_active is None:
+        scatter_max_active = max(1, n_src // 5) * max(1, batch // 64)
+    if max_active is None:
+        max_active = active.numel()
+    _lib.check(lib.bmtk_csr_propagate_auto(
+        _p(active, torch.int32, None, "active"), _p(n_active, torch.int32, 1, "n_active"), max_active,
+        _p(zbits, torch.int64, n_words(n_src * batch) + 1, "zbits"), n_src, batch, *table_src.pointers(),
+        *table_tgt.pointers(), _p(ring, torch.float32), L, n_tgt, int(step), int(scatter_max_active), _stream()))
+
+
+def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_active=None, zbits=None, n_src=None,
+                      table_tgt=None, scatter_max_active=None):
+    """``mode`` "scatter" (source-major table + active list), "gather" (target-major table + spike bits) or
+    "auto" (``table`` source-major and ``table_tgt`` target-major, active list and spike bits: the device picks
+    by the active count, see ``csr_propagate_auto``)."""
     if mode == "scatter":
         return csr_propagate_scatter(active, n_active, table, ring, n_tgt, batch, step)
     if mode == "gather":
         return csr_propagate_gather(zbits, n_src, table, ring, n_tgt, batch, step)
-    raise ValueError("mode must be 'scatter' or 'gather'")
+    if mode == "auto":
+        return csr_propagate_auto(active, n_active, zbits, n_src, table, table_tgt, ring, n_tgt, batch, step,
+                                  scatter_max_active)
+    raise ValueError("mode must be 'scatter', 'gather' or 'auto'")
 
 
 def unpack_bits(bits, ne):

@@ -209,3 +209,29 @@ def test_table_from_edges_on_the_device_equals_the_host_build():
             assert a.dtype == b.cpu().numpy().dtype
     with pytest.raises(ValueError):
         ops.SynapseTable.from_edges(src, tgt + n_cols, w, d, r, n_rows, n_cols)
+
+
+@pytest.mark.parametrize("batch", [1, 64])
+def test_auto_delivery_picks_a_form_on_the_device_and_both_give_the_oracle_ring(batch):
+    """`csr_propagate_fwd("auto")`: the active count decides on the device between the event-driven and the row-wise
+    form.  Quarter-pA weights: whichever runs, the ring must equal the fp32 oracle's bit for bit -- with a
+    threshold below, at and above the actual count, and with nothing active."""
+    rng = np.random.default_rng(33)
+    n, L = 500, 6
+    src, tgt, w, d, r = _edges(rng, n, n, 30000)
+    w = (np.round(w * 4) / 4 + np.sign(w) * 0.25).astype(np.float32)
+    by_src = net.coo_to_csr(src, tgt, w, d, r, n_rows=n, major="source")
+    by_tgt = net.csr_transpose(by_src, n)
+    t_src, t_tgt = ops.SynapseTable.from_numpy(by_src), ops.SynapseTable.from_numpy(by_tgt)
+    comp = ops.SpikeCompactor(n * batch)
+    for p in (0.0, 0.01, 0.2):
+        z = (rng.random(n * batch) < p).astype(np.uint8)
+        count = int(z.sum())
+        want = np.zeros((L, 4, n * batch), np.float32)
+        orc.gather_rows(z, batch, by_tgt, want, n, 4)
+        for thr in (0, max(count - 1, 0), count, count + 1, None):
+            ring = torch.zeros(L, 4, n * batch, device="cuda")
+            ids, cnt = comp(to_dev(z))
+            ops.csr_propagate_fwd("auto", t_src, ring, n, batch, 4, active=ids, n_active=cnt, zbits=to_dev(bits_of(z)),
+                                  n_src=n, table_tgt=t_tgt, scatter_max_active=thr)
+            np.testing.assert_array_equal(ring.cpu().numpy(), want, err_msg="p=%g threshold=%s" % (p, thr))
