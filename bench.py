@@ -58,7 +58,7 @@ def profile_traffic(file_name, key):
 
 def build_v1(torch, steps_total, resident="auto"):
     import numpy as np
-    from bmtk_amd import synthetic
+    from bmtk_amd import ops, synthetic
     from bmtk_amd.simulator import Glif3Simulator
     rng = np.random.default_rng(3)
     par = synthetic.random_cells(rng, N_CLASSES)
@@ -66,7 +66,8 @@ def build_v1(torch, steps_total, resident="auto"):
     by_tgt, by_src, _ = synthetic.device_network(N_V1, MEAN_IN, "lognormal", seed=3)
     del by_tgt
     inp = synthetic.device_input_table(N_IN, N_V1, N_IN_SYN, seed=4, w_scale=IN_W_SCALE)
-    in_ptr, in_ev = synthetic.device_poisson_events(N_IN, IN_RATE_HZ, 1.0, steps_total, seed=5)
+    # exponential inter-spike intervals per source, generated on the device (ops.poisson_events)
+    in_ptr, in_ev = ops.poisson_events(N_IN, IN_RATE_HZ, 1.0, steps_total, seed=5)
     sim = Glif3Simulator(N_V1, par, 1.0, class_id=class_id, rec=by_src, inp=inp, resident=resident)
     sim.set_input_events(in_ptr, in_ev)
     return sim, par, class_id
@@ -245,7 +246,7 @@ def bench_bptt(torch, steps=600):
     par = synthetic.random_cells(rng, n)
     _, by_src, _ = synthetic.device_network(n, 1000, "poisson", seed=2, w_scale=0.2)
     inp = synthetic.device_input_table(n_in, n, 8_000_000, seed=4, w_scale=2.0)
-    in_ptr, in_ev = synthetic.device_poisson_events(n_in, 5.0, 1.0, 2 * steps, batch=batch, seed=5)
+    in_ptr, in_ev = ops.poisson_events(n_in, 5.0, 1.0, 2 * steps, batch=batch, seed=5)
     sim = Glif3Simulator(n, par, 1.0, batch=batch, rec=by_src, inp=inp, resident=False)
     sim.set_input_events(in_ptr, in_ev)
     g = torch.Generator(device="cuda").manual_seed(11)

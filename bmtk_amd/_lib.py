@@ -55,7 +55,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 11  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 12  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -84,6 +84,10 @@ SIGNATURES = {
     "bmtk_csr_pack_wide": (c_int32, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p]),
     "bmtk_csr_segment_offsets": (c_int32, [c_int64, c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p,
                                            c_void_p]),
+    "bmtk_poisson_count": (c_int32, [c_int64, c_int32, c_void_p, c_double, c_double, c_double, c_int64, C.c_uint64,
+                                     c_void_p, c_void_p]),
+    "bmtk_poisson_fill": (c_int32, [c_int64, c_int32, c_void_p, c_double, c_double, c_double, c_int64, C.c_uint64,
+                                    c_void_p, c_void_p, c_void_p, c_void_p]),
     "bmtk_glif3_simulate_fwd": (c_int32, [C.POINTER(Glif3Sim), c_int64, c_int64, c_void_p]),
     "bmtk_glif3_simulate_bwd": (c_int32, [C.POINTER(Glif3Bwd), c_int64, c_int64, c_void_p]),
     "bmtk_csr_propagate_bwd": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int32, c_int64, c_void_p,

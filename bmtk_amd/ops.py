@@ -385,6 +385,43 @@ def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_acti
     raise ValueError("mode must be 'scatter', 'gather' or 'auto'")
 
 
+def poisson_events(n_sources, rate_hz, dt_ms, n_steps, batch=1, seed=1, t_start_ms=0.0, t_stop_ms=None,
+                   return_times=False, device=None):
+    """Homogeneous Poisson spike sources generated on the device (exponential inter-spike intervals per source and
+    trial, as bmtk's ``PoissonSpikeGenerator`` draws them, bmtk/utils/reports/spike_trains/spike_trains.py:166-206;
+    independent streams instead of NumPy's global one) as the per-step event lists a simulation reads:
+    ``(in_ptr int64[n_steps+1], in_events int32[])``, ids = source*batch + trial ascending within each step; a
+    source that fires twice inside one step appears twice.  ``rate_hz``: scalar or one rate per source.
+    ``return_times`` adds ``(step int64[], element int64[], time_ms float64[])`` of every spike, in event order.
+    Nothing passes through host memory."""
+    lib = _lib.load()
+    dev = device or _dev()
+    rates = torch.as_tensor(np.broadcast_to(np.asarray(rate_hz, np.float32), (n_sources,)).copy(), device=dev)
+    if bool((rates < 0).any()):
+        raise ValueError("Firing rates must not be negative.")
+    t_stop_ms = n_steps * dt_ms if t_stop_ms is None else t_stop_ms
+    n_ids = n_sources * batch
+    counts = torch.zeros(n_ids, dtype=torch.int32, device=dev)
+    args = (n_sources, batch, _p(rates), float(t_start_ms), float(t_stop_ms), float(dt_ms), int(n_steps),
+            int(seed) & (2 ** 64 - 1))
+    _lib.check(lib.bmtk_poisson_count(*args, _p(counts), _stream()))
+    offsets = torch.zeros(n_ids + 1, dtype=torch.int64, device=dev)
+    offsets[1:] = torch.cumsum(counts, 0)
+    total = int(offsets[-1].item())
+    keys = torch.empty(max(total, 1), dtype=torch.int64, device=dev)
+    times = torch.empty(max(total, 1), dtype=torch.float64, device=dev) if return_times else None
+    _lib.check(lib.bmtk_poisson_fill(*args, _p(offsets), _p(keys), _p(times), _stream()))
+    keys = keys[:total]
+    order = torch.sort(keys, stable=True).indices if return_times else None
+    keys = keys[order] if return_times else torch.sort(keys).values
+    steps = keys // n_ids
+    in_ptr = torch.searchsorted(steps, torch.arange(n_steps + 1, device=dev, dtype=torch.int64)).to(torch.int64)
+    in_events = (keys - steps * n_ids).to(torch.int32)
+    if return_times:
+        return in_ptr, in_events, (steps, in_events.to(torch.int64), times[:total][order])
+    return in_ptr, in_events
+
+
 def unpack_bits(bits, ne):
     """int64 spike-bit words ``[..., words]`` -> uint8 flags ``[..., ne]`` (host or device)."""
     shifts = torch.arange(64, device=bits.device, dtype=torch.int64)

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 11
+#define BMTK_AMD_ABI_VERSION 12
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -326,6 +326,25 @@ typedef struct bmtk_glif3_sim {
  * into its LDS ring slice with LDS atomics -- no global atomics and no state
  * traffic.  The barrier spins a bounded number of times; see res_sync. */
 int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0, int64_t n_steps, void *stream);
+
+/* Poisson spike sources generated on the device: the homogeneous case of bmtk's
+ * PoissonSpikeGenerator._build_fixed_fr (bmtk/utils/reports/spike_trains/spike_trains.py:166-206) without
+ * refractory thinning -- per element (source, trial), from t_start on, t += -ln(1 - U) / rate until t > t_stop,
+ * every t a spike.  Every element has a random stream of its own (Philox4x32-10, keyed by `seed`), where the
+ * reference draws all sources from NumPy's one global stream; the trains are therefore not the reference's
+ * numbers but independent samples of the same process.  rate_hz holds one rate per source.  A spike at time t is
+ * stamped ceil(t / dt) steps (at least 1) and emitted in step stamp - 1; spikes whose emitting step is n_steps
+ * or later are left out.
+ *   bmtk_poisson_count:  counts[e] = spikes of element e = source*batch + trial.
+ *   bmtk_poisson_fill:   with offsets = the exclusive prefix sum of counts, keys[offsets[e] + k] =
+ *                        step * (n_sources*batch) + e for the k-th spike of element e, and its time in ms in
+ *                        times_ms (may be NULL).  Sorting the keys gives the per-step event lists (in_ptr,
+ *                        in_events) of bmtk_glif3_sim, ascending within each step. */
+int bmtk_poisson_count(int64_t n_sources, int32_t batch, const float *rate_hz, double t_start_ms, double t_stop_ms,
+                       double dt_ms, int64_t n_steps, uint64_t seed, int32_t *counts, void *stream);
+int bmtk_poisson_fill(int64_t n_sources, int32_t batch, const float *rate_hz, double t_start_ms, double t_stop_ms,
+                      double dt_ms, int64_t n_steps, uint64_t seed, const int64_t *offsets, int64_t *keys,
+                      double *times_ms, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Backward pass (reverse-time adjoint) of the forward simulation.
