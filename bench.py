@@ -232,8 +232,10 @@ def bench_bptt(torch, steps=600):
     weight.  Recurrent weights are scaled by 0.2 and input weights by 2 so that the network settles
     near 3 Hz (unit weights at this in-degree saturate it).
 
-    Returns two entries: the training step, and the transposed propagation on its own (the kernel that
-    takes most of the backward pass), timed through bmtk_csr_propagate_bwd on the same table.
+    Returns three entries: the training step, and the transposed propagation on its own (the kernel that
+    takes most of the backward pass) in the two forms the library has: through the table regrouped by target
+    range (bmtk_csr_propagate_bwd_blocked, the form the training step uses at this size) and row by row through
+    the source-major table (bmtk_csr_propagate_bwd).
     Rooflines use the bytes that MUST cross HBM: per backward step the packed table once (8 B per synapse),
     the adjoint ring slots once (L-1 slots x 4 receptors x ne x 4 B), the adjoint state in and out, the
     forward record (potential and flags) and the input gradient's reads; not the L2 fills the kernels cause by
@@ -279,8 +281,9 @@ def bench_bptt(torch, steps=600):
     # forward, per step: target-major table once (pull form) + 12 state words in and out + record out
     fwd_step = nnz * 8 + ne * (12 * 8 + 16 + 5)
     step_entry = {
-        "kernel": "sim_step_kernel + pull_kernel (forward), bwd_gather4_kernel + bwd_state_kernel + bwd_inp_grad_kernel "
-                  "(backward; the recurrent weight gradient rides in bwd_gather4_kernel)",
+        "kernel": "sim_step_kernel + pull_kernel (forward), bwd_gather_blocked_kernel + bwd_state_kernel + "
+                  "bwd_inp_grad_kernel (backward; the recurrent weight gradient rides in bwd_gather_blocked_kernel)",
+        "blocked_table_ranges": bptt.n_blocks if bptt.blk is not None else 0,
         "workload": "BPTT step N=51978 nnz=%d inputs=17400 batch=32 steps=%d" % (nnz, steps),
         "seconds_per_training_step": t_f + t_b, "forward_s": t_f, "backward_s": t_b,
         "mean_rate_hz": float(res["counts"].float().mean().item()) / steps * 1e3,
@@ -296,23 +299,38 @@ def bench_bptt(torch, steps=600):
                              "algorithmic_bytes_per_step": fwd_step}}
     # the transposed propagation alone, every row active
     lam = torch.randn(L, 4, ne, device="cuda", generator=g)
-    gz = torch.empty(ne, device="cuda")
-    for k in range(5):
-        ops.csr_propagate_bwd(sim.rec, lam, n, batch, k, gz=gz)
-    reps = 50
-    _, dev = time_region(torch, lambda: [ops.csr_propagate_bwd(sim.rec, lam, n, batch, k, gz=gz) for k in range(reps)])
-    per = dev / reps
+    gz = torch.empty(8, ne, device="cuda")
     alg = nnz * 8 + ring_bytes + ne * 4
-    gather_entry = {
-        "kernel": "bwd_gather4_kernel", "workload": "transposed propagation N=51978 nnz=%d batch=32, every row" % nnz,
-        "us_per_launch": per * 1e6, "synapse_trials_per_s": nnz * batch / per,
-        "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": alg / per / 1e9 / HBM_PEAK_GBS, "what": "HBM-compulsory bytes: table + adjoint ring + output once",
-                     "algorithmic_bytes_per_launch": alg,
-                     "traffic": profile_traffic("backward_kernels_52k_batch32.txt", "l2_fill_bytes_per_launch_bwd_gather4"),
-                     "traffic_note": "L2 fills (one 128-byte adjoint row per synapse, served mostly by the memory-side "
-                                     "cache), not HBM bytes"}}
-    return [step_entry, gather_entry]
+    reps = 50
+
+    def gather_entry(kernel, what, call, traffic_key, traffic_note):
+        for k in range(5):
+            call(k)
+        _, dev = time_region(torch, lambda: [call(k) for k in range(reps)])
+        per = dev / reps
+        return {"kernel": kernel, "workload": "transposed propagation N=51978 nnz=%d batch=32, every row, %s" % (nnz, what),
+                "us_per_launch": per * 1e6, "synapse_trials_per_s": nnz * batch / per,
+                "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": alg / per / 1e9 / HBM_PEAK_GBS,
+                             "what": "HBM-compulsory bytes: table + adjoint ring + output once",
+                             "algorithmic_bytes_per_launch": alg,
+                             "traffic": profile_traffic("backward_kernels_52k_batch32.txt", traffic_key),
+                             "traffic_note": traffic_note}}
+
+    entries = [step_entry]
+    if bptt.blk is not None:
+        entries.append(gather_entry(
+            "bwd_gather_blocked_kernel", "table regrouped into %d target ranges" % bptt.n_blocks,
+            lambda k: ops.csr_propagate_bwd_blocked(bptt.blk, bptt.n_blocks, lam, n, batch, k, gz_parts=gz),
+            "hbm_bytes_per_launch_bwd_gather_blocked",
+            "HBM bytes; the kernel reads one 128-byte adjoint row per synapse (6.6 GB per launch) from the L2s, "
+            "which is what bounds it"))
+    entries.append(gather_entry(
+        "bwd_gather4_kernel", "source-major table row by row",
+        lambda k: ops.csr_propagate_bwd(sim.rec, lam, n, batch, k, gz=gz[0]),
+        "l2_fill_bytes_per_launch_bwd_gather4",
+        "L2 fills (one 128-byte adjoint row per synapse, served mostly by the memory-side cache), not HBM bytes"))
+    return entries
 
 
 def cpu_baseline(torch, sim, par, class_id, settled, sample_steps):

@@ -9,6 +9,7 @@ namespace bmtk {
 struct BwdStep {
     int64_t t;    // absolute step being differentiated
     int64_t row;  // its row in the forward record
+    int parts;    // partial sums gz[parts][ne] that the transposed propagation left (1, or 8 from the blocked form)
 };
 
 __device__ __forceinline__ float surrogate(float U, float th, float dampening)
@@ -200,6 +201,248 @@ __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, B
                                                             (act & 4u) ? acc[2] : 0.0f, (act & 8u) ? acc[3] : 0.0f);
 }
 
+// The same sums through the table regrouped by target range, for networks whose adjoint ring is far larger than an
+// L2.  bwd_gather4_kernel visits the adjoint rows of a source's targets all over the ring: at 52k neurons x 32
+// trials the ring is 133 MB, every 128-byte row misses the 4 MB L2 of its XCD and the kernel runs at the rate the
+// fabric fills L2 lines (6.4 GB per step).  Here the targets are cut into blk_count ranges whose slice of the ring
+// (all slots and receptors) fits an L2, and the table holds, range after range, a CSR over the sources of the
+// synapses into that range.  Workgroup b runs on XCD b % 8 (workgroups are dealt to the XCDs in turn) and takes
+// the ranges x*P .. x*P+P-1, one after the other, over a fixed share of the source rows, so that while an XCD
+// works through a range its L2 holds that slice and each adjoint row is fetched from memory once per sweep
+// instead of once per synapse.  A lane group of lp lanes (4 trials each) owns one source row; its partial sum
+// over the ranges seen so far waits in LDS (16 bytes per lane and row, lane-private, so no barriers), which is
+// what bounds the rows of a sweep: 16 wavefronts x gpw row groups x 64/lp rows.  The eight XCDs each see every
+// row for their own ranges and write a partial sum of their own, gz[x][ne]; the state adjoint adds the eight.
+constexpr int kBlkThreads = 1024;
+constexpr int kBlkWaves = kBlkThreads / kWave;
+constexpr int kBlkMaxGroups = 8;  // row groups per wavefront and sweep: one byte of trial masks each in a 64-bit register
+constexpr int kBlkInFlight = 8;   // synapses of a row in flight
+static_assert(kBlkInFlight % 8 == 0 && 2 * kBlkInFlight <= BMTK_BLOCKED_PAD, "the kernel reads up to 2*kBlkInFlight - 1 records past a row's end");
+
+// 24-bit multiplies (full rate; the compiler turns __umul24 with a uniform operand into the quarter-rate 32-bit
+// multiply).  Only bits 0-23 of a and b count.
+__device__ __forceinline__ unsigned mul_u24(unsigned a, unsigned b)
+{
+    unsigned r;
+    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ unsigned mad_u24(unsigned a, unsigned b, unsigned c)
+{
+    unsigned r;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// the value of `x` in the lane a data-parallel-primitive control word names (all of the ones used here have a source)
+template <int kCtrl>
+__device__ __forceinline__ float dpp_move(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), kCtrl, 0xF, 0xF, false));
+}
+
+// kNe24: n_neurons*batch < 2^24, so that the cell arithmetic can use 24-bit multiplies; kWide: lp >= 8
+template <bool kGrad, bool kNe24, bool kWide>
+__global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_glif3_bwd a, BwdStep q, int lp, int rows_cu,
+                                                                         int sweeps, int gpw)
+{
+    extern __shared__ float4 blk_acc[];  // [kBlkWaves][gpw][kWave]
+    constexpr int kF = kBlkInFlight;
+    const int batch = a.batch;
+    const int64_t n = a.n_neurons, ne = n * batch;
+    const int L = a.ring_slots;
+    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    const int x = blockIdx.x & 7;
+    const int P = a.blk_count >> 3;
+    const int per = kWave / lp;  // rows a wavefront works on side by side
+    const int grp = lane / lp, b4 = (lane - grp * lp) * 4;
+    const bool lane_on = b4 < batch;
+    const unsigned long long grp_lanes = (lp == kWave ? ~0ull : ((1ull << lp) - 1ull)) << (grp * lp);
+    const int64_t row_lo = (int64_t)(blockIdx.x >> 3) * rows_cu;
+    const int64_t row_hi = row_lo + rows_cu < n ? row_lo + rows_cu : n;
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.blk_packed);
+    // byte offset of a synapse's adjoint cell from the start of the ring, in 32 bits: the record's upper byte is
+    // delay*4 + receptor, so (slot0 + delay) % L * 4 + receptor = min(u, u - 4L) with u = slot0*4 + that byte
+    const char *__restrict__ ring = reinterpret_cast<const char *>(a.lam_ring);
+    const unsigned lane_off = (unsigned)b4 * 4u;
+    const unsigned q_lo = (unsigned)(q.t % L) * 4u, q_wrap = q_lo - 4u * (unsigned)L;
+    const unsigned ne32 = (unsigned)ne, batch32 = (unsigned)batch;
+    auto cell_off = [&](unsigned tdr) -> unsigned {
+        const unsigned dq = tdr >> 24;
+        const unsigned plane = min(dq + q_lo, dq + q_wrap);
+        const unsigned elem = mad_u24(tdr, batch32, kNe24 ? mul_u24(plane, ne32) : plane * ne32);  // bits 24-31 of tdr do not count
+        return (elem << 2) + lane_off;
+    };
+    float4 *acc = blk_acc + (size_t)wave * gpw * kWave + lane;
+    for (int sw = 0; sw < sweeps; ++sw) {
+        const int64_t jw = row_lo + ((int64_t)sw * kBlkWaves + wave) * gpw * per + grp;  // this lane's row of group 0
+        // per row group one byte: bits 0-3 the lane's trials with a non-zero surrogate derivative in this step,
+        // bits 4-7 those in which the source fired (kGrad)
+        unsigned long long masks = 0ull;
+        for (int k = 0; k < gpw; ++k) {
+            const int64_t j = jw + (int64_t)k * per;
+            unsigned act = 0u, mine = 0u;
+            if (j < row_hi && lane_on) {
+                const int64_t e = j * batch + b4;
+                if (a.save_flags) {
+                    const uint32_t f4 = *reinterpret_cast<const uint32_t *>(a.save_flags + q.row * ne + e);
+                    const float4 v4 = *reinterpret_cast<const float4 *>(a.save_v + q.row * ne + e);
+                    const int64_t col = a.class_id ? (int64_t)a.class_id[j] : j;
+                    const float th = a.prop[GLIF3_TH * a.prop_stride + col];
+                    const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        if (((f4 >> (8 * c)) & BMTK_F_INTEGRATING) && fabsf((v[c] - th) / th) < 1.0f) act |= 1u << c;
+                } else {
+                    act = 0xFu;
+                }
+                if (kGrad)
+                    mine = (unsigned)(trial_mask(a.spike_bits + q.row * a.spike_bits_stride, j, batch, 0, batch) >> b4) & 0xFu;
+            }
+            masks |= (unsigned long long)(act | (mine << 4)) << (8 * k);
+            acc[k * kWave] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+        // the synapses this lane's row of group k sends into range ph: [p, p1); empty for rows none of whose
+        // trials needs them, and for rows past the end
+        auto row_range = [&](int ph, int k, int &p, int &p1) {
+            p = p1 = 0;
+            if (ph >= P) return;
+            const bool want = ((masks >> (8 * k)) & 0xFFull) != 0ull;
+            const int64_t j = jw + (int64_t)k * per;
+            if ((__ballot(want) & grp_lanes) != 0ull && j < row_hi) {
+                const int32_t *__restrict__ ip = a.blk_indptr + (int64_t)(x * P + ph) * n + j;
+                p = ip[0];
+                p1 = ip[1];
+            }
+        };
+        int p_next, p1_next;
+        row_range(0, 0, p_next, p1_next);
+        for (int ph = 0; ph < P; ++ph) {
+            for (int k = 0; k < gpw; ++k) {
+                int p = p_next;
+                const int p1 = p1_next;
+                row_range(k + 1 < gpw ? ph : ph + 1, k + 1 < gpw ? k + 1 : 0, p_next, p1_next);  // asked for a visit ahead
+                if (__ballot(p < p1) == 0ull) continue;
+                const unsigned mine = (unsigned)(masks >> (8 * k + 4)) & 0xFu;
+                const int p1_lane = ((masks >> (8 * k)) & 0xFFull) != 0ull ? p1 : 0;  // lanes none of whose trials counts stay idle
+                const bool row_fired = kGrad && (__ballot(mine != 0u) & grp_lanes) != 0ull;
+                const float fired_f[4] = {(mine & 1u) ? 1.0f : 0.0f, (mine & 2u) ? 1.0f : 0.0f, (mine & 4u) ? 1.0f : 0.0f,
+                                          (mine & 8u) ? 1.0f : 0.0f};
+                const int in_row = lane - grp * lp;  // this lane's place among its row's lanes
+                float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                // kF synapses of the row at a time: their adjoint rows are asked for, then the row's next kF
+                // records (which arrive while the adjoint rows are on their way), then the products are added.
+                // Lanes past the row's end read the ring's first cell with weight 0 -- no branches around loads.
+                auto visit = [&](auto fetch, auto record) {
+                    auto cur = fetch(0), nxt = cur;
+                    auto work = [&](const decltype(cur) &have, decltype(cur) &ahead) {
+                        float4 v[kF];
+                        float w[kF];
+#pragma unroll
+                        for (int u = 0; u < kF; ++u) {
+                            const uint2 sy = record(have, u);
+                            const bool valid = p + u < p1_lane;
+                            const unsigned off = valid ? cell_off(sy.x) : lane_off;
+                            w[u] = valid ? __uint_as_float(sy.y) : 0.0f;
+                            v[u] = *reinterpret_cast<const float4 *>(ring + off);
+                        }
+                        ahead = fetch(kF);
+#pragma unroll
+                        for (int u = 0; u < kF; ++u) {
+                            s.x = fmaf(w[u], v[u].x, s.x);
+                            s.y = fmaf(w[u], v[u].y, s.y);
+                            s.z = fmaf(w[u], v[u].z, s.z);
+                            s.w = fmaf(w[u], v[u].w, s.w);
+                        }
+                        if (kGrad && __ballot(row_fired && p < p1) != 0ull) {
+                            if (kWide) {
+                                // the gradient of record u is the sum, over the row's lanes, of the adjoint entries of
+                                // the trials in which the source fired; every lane gets every sum (data-parallel
+                                // moves within quads, half rows and rows of 16 lanes) and keeps the one of the
+                                // record it then updates: one read-modify-write for the kF records of all rows
+                                float keep = 0.0f;
+#pragma unroll
+                                for (int u = 0; u < kF; ++u) {
+                                    float g = fmaf(fired_f[3], v[u].w, fmaf(fired_f[2], v[u].z, fmaf(fired_f[1], v[u].y, fired_f[0] * v[u].x)));
+                                    g += dpp_move<0xB1>(g);   // quad_perm [1,0,3,2]
+                                    g += dpp_move<0x4E>(g);   // quad_perm [2,3,0,1]
+                                    g += dpp_move<0x141>(g);  // row_half_mirror: the other quad of these eight lanes
+                                    if (lp > 8) g += dpp_move<0x140>(g);  // row_mirror: the other eight of these sixteen
+                                    keep = in_row == u ? g : keep;
+                                }
+                                if (row_fired && in_row < kF && p + in_row < p1) a.d_blk_w[p + in_row] += keep;
+                            } else {
+#pragma unroll
+                                for (int u = 0; u < kF; ++u) {
+                                    float g = ((mine & 1u) ? v[u].x : 0.0f) + ((mine & 2u) ? v[u].y : 0.0f) +
+                                              ((mine & 4u) ? v[u].z : 0.0f) + ((mine & 8u) ? v[u].w : 0.0f);
+                                    for (int off = 1; off < lp; off <<= 1) g += __shfl_xor(g, off, kWave);
+                                    if (row_fired && b4 == 0 && p + u < p1) a.d_blk_w[p + u] += g;
+                                }
+                            }
+                        }
+                        p += kF;
+                    };
+                    while (true) {
+                        work(cur, nxt);
+                        if (__ballot(p < p1) == 0ull) break;
+                        work(nxt, cur);
+                        if (__ballot(p < p1) == 0ull) break;
+                    }
+                };
+                if (kWide) {
+                    // a row's first eight lanes fetch one record in eight each (one wavefront instruction for eight
+                    // records of every row) and pass them round; eight lanes fetching the same record eight times
+                    // over kept the address unit busier than the adjoint rows did
+                    struct Shared {
+                        uint2 r[kF / 8];
+                    };
+                    const int c = (lane - grp * lp) & 7, first = grp * lp;
+                    visit(
+                        [&](int ahead) {
+                            Shared f;
+#pragma unroll
+                            for (int i = 0; i < kF / 8; ++i) f.r[i] = rows[p + ahead + 8 * i + c];
+                            return f;
+                        },
+                        [&](const Shared &have, int u) {
+                            return make_uint2((unsigned)__shfl((int)have.r[u / 8].x, first + (u & 7), kWave),
+                                              (unsigned)__shfl((int)have.r[u / 8].y, first + (u & 7), kWave));
+                        });
+                } else {
+                    struct Records {
+                        uint2 r[kF];
+                    };
+                    visit(
+                        [&](int ahead) {
+                            Records f;
+#pragma unroll
+                            for (int u = 0; u < kF; ++u) f.r[u] = rows[p + ahead + u];
+                            return f;
+                        },
+                        [&](const Records &have, int u) { return have.r[u]; });
+                }
+                float4 t = acc[k * kWave];
+                t.x += s.x;
+                t.y += s.y;
+                t.z += s.z;
+                t.w += s.w;
+                acc[k * kWave] = t;
+            }
+        }
+        for (int k = 0; k < gpw; ++k) {
+            const int64_t j = jw + (int64_t)k * per;
+            if (j < row_hi && lane_on) {
+                const unsigned act = (unsigned)(masks >> (8 * k)) & 0xFu;
+                const float4 t = acc[k * kWave];
+                *reinterpret_cast<float4 *>(a.gz + (int64_t)x * ne + j * batch + b4) =
+                    make_float4((act & 1u) ? t.x : 0.0f, (act & 2u) ? t.y : 0.0f, (act & 4u) ? t.z : 0.0f,
+                                (act & 8u) ? t.w : 0.0f);
+            }
+        }
+    }
+}
+
 // state adjoint of one step, one thread per element; writes the adjoint of
 // this step's arrivals into ring slot t
 __global__ __launch_bounds__(kBlock) void bwd_state_kernel(bmtk_glif3_bwd a, BwdStep q)
@@ -233,6 +476,7 @@ __global__ __launch_bounds__(kBlock) void bwd_state_kernel(bmtk_glif3_bwd a, Bwd
     float nV, nA[GLIF3_NASC];
     if (f & BMTK_F_INTEGRATING) {
         float g = a.gz[e];
+        for (int x = 1; x < q.parts; ++x) g += a.gz[(int64_t)x * ne + e];
         if (a.dl_dz) g += a.dl_dz[q.row * ne + e];
         if (a.dl_dz_const) g += a.dl_dz_const[e];
         const float lU = lV + surrogate(a.save_v[q.row * ne + e], p.th, a.dampening) * g;
@@ -358,6 +602,97 @@ __global__ __launch_bounds__(kBlock) void spike_counts_kernel(const uint64_t *__
 
 using namespace bmtk;
 
+namespace {
+
+const void *blocked_variant(bool grad, bool ne24, bool wide)
+{
+#define BMTK_BLK(g, n, w) reinterpret_cast<const void *>(bwd_gather_blocked_kernel<g, n, w>)
+    if (grad) {
+        if (ne24) return wide ? BMTK_BLK(true, true, true) : BMTK_BLK(true, true, false);
+        return wide ? BMTK_BLK(true, false, true) : BMTK_BLK(true, false, false);
+    }
+    if (ne24) return wide ? BMTK_BLK(false, true, true) : BMTK_BLK(false, true, false);
+    return wide ? BMTK_BLK(false, false, true) : BMTK_BLK(false, false, false);
+#undef BMTK_BLK
+}
+
+// launch geometry of bwd_gather_blocked_kernel for a network on the current device
+struct BlockedPlan {
+    unsigned grid;
+    int lp, rows_cu, sweeps, gpw;
+    size_t lds;
+};
+
+int blocked_plan(const bmtk_glif3_bwd &a, BlockedPlan &pl)
+{
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    static int cu_count[64];
+    int n_cu = (dev >= 0 && dev < 64) ? cu_count[dev] : 0;
+    if (n_cu <= 0) {
+        n_cu = 256;
+        (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (dev >= 0 && dev < 64) cu_count[dev] = n_cu;
+    }
+    const int cus = n_cu >= 8 ? n_cu / 8 : 1;  // workgroups per XCD, one per compute unit
+    int bp = 4;
+    while (bp < a.batch) bp <<= 1;
+    pl.lp = bp / 4;
+    const int per = kWave / pl.lp;
+    int64_t rows_cu = (a.n_neurons + cus - 1) / cus;
+    rows_cu = (rows_cu + per - 1) / per * per;
+    const int64_t cap = (int64_t)kBlkWaves * kBlkMaxGroups * per;  // rows of one sweep
+    pl.sweeps = (int)((rows_cu + cap - 1) / cap);
+    pl.gpw = (int)((rows_cu + (int64_t)pl.sweeps * kBlkWaves * per - 1) / ((int64_t)pl.sweeps * kBlkWaves * per));
+    pl.rows_cu = (int)rows_cu;
+    pl.grid = (unsigned)cus * 8u;
+    pl.lds = (size_t)kBlkWaves * pl.gpw * kWave * sizeof(float4);
+    static bool asked[8][64];
+    const void *variants[8];
+    for (int g = 0; g < 8; ++g) variants[g] = blocked_variant(g & 4, g & 2, g & 1);
+    for (int g = 0; g < 8; ++g) {
+        if (dev < 0 || dev >= 64 || asked[g][dev]) continue;
+        const hipError_t err = hipFuncSetAttribute(
+            variants[g], hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kBlkWaves * kBlkMaxGroups * kWave * sizeof(float4)));
+        if (err != hipSuccess) {
+            set_error("transposed propagation: cannot reserve LDS: %s", hipGetErrorString(err));
+            return BMTK_E_LAUNCH;
+        }
+        asked[g][dev] = true;
+    }
+    return BMTK_OK;
+}
+
+// what the blocked form of the table must satisfy
+int blocked_check(const bmtk_glif3_bwd &a, const char *who)
+{
+    BMTK_REQUIRE(a.blk_count > 0 && a.blk_count % 8 == 0 && a.blk_indptr && a.blk_packed,
+                 "%s: the blocked table needs blk_count (a multiple of 8), blk_indptr and blk_packed", who);
+    BMTK_REQUIRE(a.batch % 4 == 0 && a.batch <= kWave, "%s: the blocked table serves batches that are a multiple of 4 up to 64",
+                 who);
+    BMTK_REQUIRE((int64_t)a.ring_slots * GLIF3_NREC * a.n_neurons * a.batch < (1ll << 30),
+                 "%s: the adjoint ring must stay below 4 GB for the blocked table", who);
+    return BMTK_OK;
+}
+
+int blocked_launch(const bmtk_glif3_bwd &a, const BwdStep &q, const BlockedPlan &pl, bool grad, hipStream_t st)
+{
+    const bool ne24 = a.n_neurons * (int64_t)a.batch < (1ll << 24);
+    bmtk_glif3_bwd args = a;
+    BwdStep step = q;
+    int lp = pl.lp, rows_cu = pl.rows_cu, sweeps = pl.sweeps, gpw = pl.gpw;
+    void *params[] = {&args, &step, &lp, &rows_cu, &sweeps, &gpw};
+    const hipError_t err = hipLaunchKernel(blocked_variant(grad, ne24, pl.lp >= 8), dim3(pl.grid), dim3(kBlkThreads),
+                                           params, pl.lds, st);
+    if (err != hipSuccess) {
+        set_error("transposed propagation: launch failed: %s", hipGetErrorString(err));
+        return BMTK_E_LAUNCH;
+    }
+    return BMTK_OK;
+}
+
+}  // namespace
+
 extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_steps, void *stream)
 {
     BMTK_REQUIRE(bwd != nullptr, "glif3_simulate_bwd: bwd is null");
@@ -374,9 +709,17 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
     BMTK_REQUIRE(a.lam_V && a.lam_asc && a.lam_y1 && a.lam_y2 && a.lam_ring && a.gz,
                  "glif3_simulate_bwd: adjoint state pointers must be non-null");
     BMTK_REQUIRE(!(a.dl_dz && a.dl_dz_const), "glif3_simulate_bwd: give dl_dz or dl_dz_const, not both");
+    const bool blocked = a.blk_count != 0;
+    BlockedPlan pl{};
+    if (blocked) {
+        int rc = blocked_check(a, "glif3_simulate_bwd");
+        if (rc == BMTK_OK) rc = blocked_plan(a, pl);
+        if (rc != BMTK_OK) return rc;
+    }
     const bool has_rec = a.rec_indptr != nullptr;
     BMTK_REQUIRE(!has_rec || a.rec_packed, "glif3_simulate_bwd: recurrent table needs rec_packed");
     BMTK_REQUIRE(!a.d_rec_w || has_rec, "glif3_simulate_bwd: d_rec_w without a recurrent table");
+    BMTK_REQUIRE(!a.d_blk_w || blocked, "glif3_simulate_bwd: d_blk_w without the blocked table");
     const bool inp_grad = a.d_inp_w != nullptr;
     BMTK_REQUIRE(!inp_grad || (a.in_ptr && a.in_events && a.inp_indptr && a.inp_packed),
                  "glif3_simulate_bwd: d_inp_w needs the input events and the input table");
@@ -388,13 +731,16 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
     int bp = 1;  // trial-tile width: the batch rounded up to a power of two, at most one wavefront
     while (bp < a.batch && bp < kWave) bp <<= 1;
     for (int64_t k = n_steps - 1; k >= 0; --k) {
-        BwdStep q{step0 + k, k};
+        BwdStep q{step0 + k, k, blocked ? 8 : 1};
         // The recurrent weight gradient of step t reads the adjoint slots t+1 .. t+L-1, which the state adjoint of
         // this step (it writes slot t) leaves alone: it can ride along with the transposed propagation, which
         // reads the same slots before the state adjoint runs.  Batches of more than one tile keep the kernel of
         // their own (several wavefronts would share a row).
-        const bool fused = a.d_rec_w && tiles == 1;
-        if (has_rec && a.batch % 4 == 0 && a.batch <= kWave) {
+        const bool fused = blocked ? a.d_blk_w != nullptr : (a.d_rec_w && tiles == 1);
+        if (blocked) {
+            const int rc = blocked_launch(a, q, pl, fused, st);
+            if (rc != BMTK_OK) return rc;
+        } else if (has_rec && a.batch % 4 == 0 && a.batch <= kWave) {
             if (fused)
                 hipLaunchKernelGGL(bwd_gather4_kernel<true>, dim3(rows_grid), dim3(kBlock), 0, st, a, q, bp / 4);
             else
@@ -434,7 +780,7 @@ extern "C" int bmtk_csr_propagate_bwd(const int32_t *indptr, const bmtk_synapse 
     a.rec_packed = packed;
     a.lam_ring = const_cast<float *>(lam_ring);
     a.gz = gz;
-    BwdStep q{step, 0};
+    BwdStep q{step, 0, 1};
     const unsigned rows_grid = (unsigned)((n_neurons + kBlock / kWave - 1) / (kBlock / kWave));
     int bp = 1;
     while (bp < batch && bp < kWave) bp <<= 1;
@@ -444,6 +790,35 @@ extern "C" int bmtk_csr_propagate_bwd(const int32_t *indptr, const bmtk_synapse 
         hipLaunchKernelGGL(bwd_gather_kernel<false>, dim3(rows_grid, (unsigned)((batch + kWave - 1) / kWave)), dim3(kBlock), 0,
                            (hipStream_t)stream, a, q, bp);
     BMTK_CHECK_LAUNCH("csr_propagate_bwd");
+    return BMTK_OK;
+}
+
+extern "C" int bmtk_csr_propagate_bwd_blocked(const int32_t *blk_indptr, const bmtk_synapse *blk_packed, int32_t blk_count,
+                                              int64_t n_neurons, int32_t batch, const float *lam_ring, int32_t L,
+                                              int64_t step, float *gz_parts, void *stream)
+{
+    BMTK_REQUIRE(lam_ring && gz_parts, "csr_propagate_bwd_blocked: pointers must be non-null");
+    BMTK_REQUIRE(n_neurons > 0 && batch > 0 && step >= 0, "csr_propagate_bwd_blocked: bad sizes or step");
+    BMTK_REQUIRE(n_neurons * (int64_t)batch < (1ll << 31) && n_neurons < (1ll << 24),
+                 "csr_propagate_bwd_blocked: network too large");
+    BMTK_REQUIRE(L > 1 && L <= 64, "csr_propagate_bwd_blocked: L must lie in 2..64");
+    bmtk_glif3_bwd a{};
+    a.n_neurons = n_neurons;
+    a.batch = batch;
+    a.ring_slots = L;
+    a.blk_count = blk_count;
+    a.blk_indptr = blk_indptr;
+    a.blk_packed = blk_packed;
+    a.lam_ring = const_cast<float *>(lam_ring);
+    a.gz = gz_parts;
+    BlockedPlan pl{};
+    int rc = blocked_check(a, "csr_propagate_bwd_blocked");
+    if (rc == BMTK_OK) rc = blocked_plan(a, pl);
+    if (rc != BMTK_OK) return rc;
+    BwdStep q{step, 0, 8};
+    rc = blocked_launch(a, q, pl, false, (hipStream_t)stream);
+    if (rc != BMTK_OK) return rc;
+    BMTK_CHECK_LAUNCH("csr_propagate_bwd_blocked");
     return BMTK_OK;
 }
 

@@ -155,6 +155,9 @@ def spikes_compact(z):
     return ids[:int(count.item())].clone()
 
 
+BLOCKED_PAD = 16  # BMTK_BLOCKED_PAD of include/bmtk_amd.h
+
+
 @dataclass
 class SynapseTable:
     """Device copy of a synapse table (see ``bmtk_amd.network``)."""
@@ -268,6 +271,25 @@ class SynapseTable:
                             self.delays[order].contiguous(), self.receptors[order].contiguous(), n_rows=n_cols,
                             max_row=int(counts.max().item()) if counts.numel() else 0)
 
+    def blocked(self, n_cols, n_blocks):
+        """The table regrouped by column range for the transposed propagation of the backward pass
+        (``bmtk_glif3_bwd.blk_*`` of include/bmtk_amd.h): columns are cut into ``n_blocks`` equal ranges and the
+        records are ordered by (range, row, position in the row).  Returns (indptr int32 [n_blocks*n_rows + 1],
+        packed records in the new order followed by ``BLOCKED_PAD`` zero records, order int64 [nnz]: new position ->
+        position in this table)."""
+        dev = self.indices.device
+        span = -(-n_cols // n_blocks)
+        rows = torch.repeat_interleave(torch.arange(self.n_rows, device=dev),
+                                       (self.indptr[1:] - self.indptr[:-1]).long())
+        key = torch.div(self.indices.long(), span, rounding_mode="floor") * self.n_rows + rows
+        order = torch.sort(key, stable=True).indices
+        counts = torch.bincount(key, minlength=n_blocks * self.n_rows)
+        indptr = torch.zeros(n_blocks * self.n_rows + 1, dtype=torch.int32, device=dev)
+        indptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+        packed = torch.zeros(self.nnz + BLOCKED_PAD, 2, dtype=torch.int32, device=dev)
+        packed[:self.nnz] = self.packed()[:self.nnz][order]
+        return indptr, packed, order
+
     def segment_offsets(self, span, n_groups):
         """uint32 [n_rows, n_groups+1] offsets of the first synapse per row whose index is >= g*span
         (stored in an int32 tensor).  Raises if a row is not sorted by index."""
@@ -349,6 +371,32 @@ def csr_propagate_bwd(table, lam_ring, n, batch, step, gz=None, trials_per_lane=
                                           _p(lam_ring, torch.float32), L, int(step),
                                           _p(gz, torch.float32, n * batch, "gz"), int(trials_per_lane), _stream()))
     return gz
+
+
+def blocked_table_blocks(n, batch, ring_slots, slice_bytes=8 << 20):
+    """Number of column ranges (a multiple of 8) that keeps one range's share of an adjoint ring
+    [ring_slots, 4, n*batch] fp32 at about ``slice_bytes``.  The default, twice an XCD's 4 MB L2, is where the
+    kernel was fastest at 52k neurons x 32 trials (16 to 32 ranges; three quarters of the reads hit the L2):
+    fewer, longer row segments outweigh the better hit rate of smaller slices."""
+    total = ring_slots * NREC * n * batch * 4
+    return 8 * max(1, -(-total // (8 * slice_bytes)))
+
+
+def csr_propagate_bwd_blocked(blk, n_blocks, lam_ring, n, batch, step, gz_parts=None):
+    """Transposed propagation through the blocked form ``blk = table.blocked(n, n_blocks)`` of a source-major
+    table: returns the eight partial sums ``gz_parts`` [8, n*batch]; their sum over the first axis is what
+    ``csr_propagate_bwd`` returns (up to the order of the additions)."""
+    lib = _lib.load()
+    L = lam_ring.shape[0]
+    indptr, packed = blk[0], blk[1]
+    if indptr.numel() != n_blocks * n + 1 or lam_ring.numel() != L * NREC * n * batch:
+        raise ValueError("blocked table must have n_blocks*n + 1 offsets and lam_ring must be [L, 4, n*batch]")
+    if gz_parts is None:
+        gz_parts = torch.empty(8, n * batch, device=lam_ring.device)
+    _lib.check(lib.bmtk_csr_propagate_bwd_blocked(_p(indptr, torch.int32), _p(packed), n_blocks, n, batch,
+                                                  _p(lam_ring, torch.float32), L, int(step),
+                                                  _p(gz_parts, torch.float32, 8 * n * batch, "gz_parts"), _stream()))
+    return gz_parts
 
 
 def csr_propagate_auto(active, n_active, zbits, n_src, table_src, table_tgt, ring, n_tgt, batch, step,

@@ -47,7 +47,13 @@ class Glif3Bptt:
     """Reverse-time adjoint over a recorded forward run of a ``Glif3Simulator``
     built with ``resident=False``."""
 
-    def __init__(self, sim, dampening=0.3):
+    # adjoint rings above this size use the table regrouped by target range (the ring no longer fits the L2s)
+    BLOCKED_MIN_RING_BYTES = 32 << 20
+
+    def __init__(self, sim, dampening=0.3, blocked=None, n_blocks=None):
+        """``blocked``: use the recurrent table regrouped by target range for the transposed propagation (None:
+        when the adjoint ring exceeds ``BLOCKED_MIN_RING_BYTES`` and the batch allows it); ``n_blocks``: number of
+        target ranges, a multiple of 8 (None: ``ops.blocked_table_blocks``)."""
         if sim.res_span or sim.delay_offset:
             raise ValueError("the backward pass needs a simulator built with resident=False and delay_offset 0")
         self.sim, self.dampening = sim, float(dampening)
@@ -58,8 +64,21 @@ class Glif3Bptt:
         self.lam_y1 = torch.zeros(NREC, ne, device=dev)
         self.lam_y2 = torch.zeros(NREC, ne, device=dev)
         self.lam_ring = torch.zeros(sim.L, NREC, ne, device=dev)
-        self.gz = torch.zeros(ne, device=dev)
         self.d_rec_w = torch.zeros(sim.rec.nnz, device=dev) if sim.rec is not None else None
+        can_block = sim.rec is not None and sim.batch % 4 == 0 and sim.batch <= 64 and sim.L * NREC * ne < (1 << 32)
+        if blocked is None:
+            blocked = can_block and sim.L * NREC * ne * 4 > self.BLOCKED_MIN_RING_BYTES
+        elif blocked and not can_block:
+            raise ValueError("the blocked table needs a recurrent table and a batch that is a multiple of 4 up to 64")
+        self.blk = None
+        if blocked:
+            from . import ops
+            self.n_blocks = int(n_blocks or ops.blocked_table_blocks(sim.n, sim.batch, sim.L))
+            if self.n_blocks % 8:
+                raise ValueError("n_blocks must be a multiple of 8")
+            self.blk = sim.rec.blocked(sim.n, self.n_blocks)
+            self.d_blk_w = torch.zeros(sim.rec.nnz, device=dev)
+        self.gz = torch.zeros(8 * ne if blocked else ne, device=dev)
         self.d_inp_w = torch.zeros(sim.inp.nnz, device=dev) if sim.inp is not None and sim.in_ptr is not None else None
 
     def zero(self):
@@ -82,7 +101,11 @@ class Glif3Bptt:
         a.spike_bits, a.spike_bits_stride = _p(bits, torch.int64), bits.shape[1]
         if sim.rec is not None:
             a.rec_indptr, a.rec_packed = _p(sim.rec.indptr), _p(sim.rec.packed())
-            a.d_rec_w = _p(self.d_rec_w)
+            if self.blk is None:
+                a.d_rec_w = _p(self.d_rec_w)
+            else:
+                a.blk_count, a.blk_indptr, a.blk_packed = self.n_blocks, _p(self.blk[0]), _p(self.blk[1])
+                a.d_blk_w = _p(self.d_blk_w)
         if self.d_inp_w is not None:
             a.in_ptr, a.in_events = _p(sim.in_ptr), _p(sim.in_events)
             a.inp_indptr, a.inp_packed = _p(sim.inp.indptr), _p(sim.inp.packed())
@@ -92,3 +115,6 @@ class Glif3Bptt:
         a.lam_V, a.lam_asc, a.lam_y1, a.lam_y2 = (_p(x) for x in (self.lam_V, self.lam_asc, self.lam_y1, self.lam_y2))
         a.lam_ring, a.gz = _p(self.lam_ring), _p(self.gz)
         _lib.check(self.lib.bmtk_glif3_simulate_bwd(C.byref(a), saved["step0"], n_steps, _stream()))
+        if self.blk is not None:  # the blocked kernel accumulates in its table's order: back to the order of sim.rec
+            self.d_rec_w.index_add_(0, self.blk[2], self.d_blk_w)
+            self.d_blk_w.zero_()

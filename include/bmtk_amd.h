@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 12
+#define BMTK_AMD_ABI_VERSION 13
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -364,6 +364,7 @@ int bmtk_poisson_fill(int64_t n_sources, int32_t batch, const float *rate_hz, do
  * Outputs: gradients with respect to every weight of the recurrent and input
  * tables, in packed-table order, accumulated (+=) into d_rec_w / d_inp_w.
  */
+#define BMTK_BLOCKED_PAD 16
 typedef struct bmtk_glif3_bwd {
     int64_t n_neurons;
     int32_t batch;
@@ -391,10 +392,24 @@ typedef struct bmtk_glif3_bwd {
     /* adjoint state, in/out (zero before the last step of the whole run) */
     float *lam_V, *lam_asc, *lam_y1, *lam_y2; /* [ne], [2][ne], [4][ne], [4][ne] */
     float *lam_ring;               /* [L][4][ne]: adjoint of the arrivals of the steps still ahead */
-    float *gz;                     /* [ne] scratch */
+    float *gz;                     /* [ne] scratch; [8][ne] when the blocked table is given */
     /* outputs */
     float *d_rec_w;                /* [rec nnz] or NULL */
     float *d_inp_w;                /* [inp nnz] or NULL */
+    /* Optional, for batches that are a multiple of 4 up to 64: the recurrent table regrouped by target range,
+     * which the transposed propagation then uses instead of rec_indptr / rec_packed.  The targets are cut into
+     * blk_count equal ranges (a multiple of 8; range s holds targets s*span .. (s+1)*span-1) small enough that a
+     * range's part of lam_ring fits one L2 (a few MB), and the table is, range after range, a CSR over the
+     * SOURCES of the synapses into that range: blk_indptr[s*n_neurons + j] .. [s*n_neurons + j + 1] delimit the
+     * synapses source j sends into range s (one flat array of blk_count*n_neurons + 1 offsets), blk_packed holds
+     * the records in that order FOLLOWED BY BMTK_BLOCKED_PAD more records of any content (the kernel reads up to
+     * that many records past a row's end and ignores them).  Needs a lam_ring below 4 GB. */
+    int32_t blk_count;             /* 0 = no blocked table */
+    int32_t reserved0;
+    const int32_t *blk_indptr;
+    const bmtk_synapse *blk_packed;
+    float *d_blk_w;                /* [rec nnz] recurrent weight gradient in the order of blk_packed, accumulated,
+                                      or NULL (then d_rec_w, if given, is filled through rec_indptr / rec_packed) */
 } bmtk_glif3_bwd;
 
 /* Differentiate steps step0+n_steps-1 down to step0 (three launches per step:
@@ -412,6 +427,13 @@ int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_
 int bmtk_csr_propagate_bwd(const int32_t *indptr, const bmtk_synapse *packed, int64_t n_neurons, int32_t batch,
                            const float *lam_ring, int32_t L, int64_t step, float *gz, int32_t trials_per_lane,
                            void *stream);
+
+/* The same sums through the blocked form of the table (bmtk_glif3_bwd: blk_count, blk_indptr, blk_packed), as
+ * eight partial sums gz_parts[8][n_neurons*batch] whose sum over the first index is gz.  Batches that are a
+ * multiple of 4 up to 64; every element counts. */
+int bmtk_csr_propagate_bwd_blocked(const int32_t *blk_indptr, const bmtk_synapse *blk_packed, int32_t blk_count,
+                                   int64_t n_neurons, int32_t batch, const float *lam_ring, int32_t L, int64_t step,
+                                   float *gz_parts, void *stream);
 
 /* Number of spikes of every element over n_steps rows of spike bits: counts[e] (int32). */
 int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_steps, int64_t ne, int32_t *counts,

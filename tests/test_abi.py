@@ -71,6 +71,18 @@ def test_argument_validation_needs_no_gpu():
     assert lib.bmtk_spikes_compact_noalloc(None, _lib.COMPACT_NOALLOC_MAX_N + 1, None, None, None) == -1
     assert b"exceeds" in lib.bmtk_amd_last_error()
     assert lib.bmtk_spikes_compact_noalloc(None, 16, None, None, None) == -1      # null pointers
+    # the blocked transposed propagation: range count, batch and padding constants
+    assert lib.bmtk_csr_propagate_bwd_blocked(None, None, 12, 100, 32, None, 6, 0, None, None) == -1    # null pointers
+    import ctypes
+    buf = ctypes.create_string_buffer(64)
+    ptr = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.bmtk_csr_propagate_bwd_blocked(ptr, ptr, 12, 100, 32, ptr, 6, 0, ptr, None) == -1
+    assert b"multiple of 8" in lib.bmtk_amd_last_error()
+    assert lib.bmtk_csr_propagate_bwd_blocked(ptr, ptr, 16, 100, 6, ptr, 6, 0, ptr, None) == -1
+    assert b"multiple of 4" in lib.bmtk_amd_last_error()
+    from bmtk_amd import ops
+    pad = int(re.search(r"#define BMTK_BLOCKED_PAD (\d+)", open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()).group(1))
+    assert ops.BLOCKED_PAD == pad
     limit = int(re.search(r"#define BMTK_COMPACT_NOALLOC_MAX_N \(1ll << (\d+)\)",
                           open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()).group(1))
     assert _lib.COMPACT_NOALLOC_MAX_N == 1 << limit

@@ -32,9 +32,12 @@ def _rel(got, want):
     return float(np.max(np.abs(got - want)) / max(np.max(np.abs(want)), 1e-30))
 
 
-@pytest.mark.parametrize("batch,seed,loss_kind", [(1, 2, "per_step"), (3, 4, "per_step"), (1, 5, "rates"), (4, 6, "rates"),
-                                                  (8, 8, "per_step"), (32, 9, "rates")])  # multiples of 4: four trials per lane
-def test_weight_gradients_match_autograd(batch, seed, loss_kind):
+@pytest.mark.parametrize("batch,seed,loss_kind,n_blocks",
+                         [(1, 2, "per_step", 0), (3, 4, "per_step", 0), (1, 5, "rates", 0), (4, 6, "rates", 0),
+                          (8, 8, "per_step", 0), (32, 9, "rates", 0),  # multiples of 4: four trials per lane
+                          # the recurrent table regrouped into n_blocks target ranges (more ranges than fit: empty ones)
+                          (8, 8, "per_step", 8), (32, 9, "rates", 16), (4, 6, "per_step", 64), (64, 3, "per_step", 8)])
+def test_weight_gradients_match_autograd(batch, seed, loss_kind, n_blocks):
     cfg = _net(batch, seed)
     n, T, h = cfg["n"], cfg["steps"], cfg["h"]
     ne = n * batch
@@ -45,7 +48,8 @@ def test_weight_gradients_match_autograd(batch, seed, loss_kind):
     sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
     fwd = sim.run(T, save_state=True)
     ras = sim.raster(fwd["bits"]).cpu().numpy()
-    bptt = training.Glif3Bptt(sim, dampening=0.3)
+    bptt = training.Glif3Bptt(sim, dampening=0.3, blocked=n_blocks > 0, n_blocks=n_blocks or None)
+    assert (bptt.blk is not None) == (n_blocks > 0)
     if loss_kind == "per_step":
         a = rng.normal(size=(T, ne))
         loss_fn = lambda z: (z * torch.as_tensor(a)).sum()

@@ -116,7 +116,8 @@ def _adjoint_ring(rng, L, ne):
 @pytest.mark.parametrize("batch", [32, 64, 8])
 def test_transposed_propagation_at_12k_neurons(batch):
     """12,000 source rows of ~400 synapses at batch 32 (the training configuration's batch), 64 and 8:
-      - four trials per lane == one trial per lane, bit for bit (exact operands);
+      - four trials per lane == one trial per lane == the blocked table's partial sums added up, bit for bit
+        (exact operands);
       - both equal W^T lambda computed on the host from the transposed table;
       - the adjoint identity <deliver(z), lambda> = <z, W^T lambda> against the forward gather kernel."""
     n, L, step = 12000, 6, 3
@@ -129,6 +130,10 @@ def test_transposed_propagation_at_12k_neurons(batch):
     g4 = ops.csr_propagate_bwd(t_src, lam_d, n, batch, step, trials_per_lane=4)
     g0 = ops.csr_propagate_bwd(t_src, lam_d, n, batch, step)
     assert torch.equal(g1, g4) and torch.equal(g0, g4)
+    # the table regrouped into target ranges: eight partial sums, exact like the rest
+    for n_blocks in (8, 24):
+        parts = ops.csr_propagate_bwd_blocked(t_src.blocked(n, n_blocks), n_blocks, lam_d, n, batch, step)
+        assert torch.equal(parts.sum(0), g4)
     # host: gz[j, b] = sum over synapses (j -> i) of w * lam[(step + d) % L, r, i, b], from the target-major copy
     indptr, src, w, d, r = host_tgt
     tgt = np.repeat(np.arange(n), np.diff(indptr))
@@ -187,6 +192,7 @@ def test_weight_gradients_match_autograd_over_many_rows_and_long_event_lists():
 def test_backward_at_10k_neurons_batch_32_chunked_equals_one_call():
     """10,000 neurons x batch 32, ~100 synapses per row, 40 steps: the backward pass in one call and as three chunks
     in reverse time order give the same gradients (to 1e-6 of the largest; the additions happen in the same order),
+    the recurrent table regrouped into 16 target ranges gives them to 1e-5,
     and the forward run they differentiate is the fp32 oracle's, spike for spike."""
     n, batch, T = 10000, 32, 40
     cfg = _net_cfg(n=n, n_in=2000, batch=batch, steps=T, seed=17, in_rate=60.0, in_w=4.0, w_scale=2.0,
@@ -201,7 +207,7 @@ def test_backward_at_10k_neurons_batch_32_chunked_equals_one_call():
     assert want["count"] > 20 * batch
     a = torch.as_tensor(np.random.default_rng(1).normal(size=(T, ne)).astype(np.float32), device="cuda")
     grads = []
-    for chunks in ([T], [15, 14, 11]):
+    for chunks, n_blocks in (([T], 0), ([15, 14, 11], 0), ([15, 14, 11], 16)):
         sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"],
                              ring_slots=cfg["L"], resident=False)
         sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
@@ -211,10 +217,12 @@ def test_backward_at_10k_neurons_batch_32_chunked_equals_one_call():
             k0 += c
         ras = np.concatenate([sim.raster(f["bits"]).cpu().numpy() for f, _, _ in runs])
         np.testing.assert_array_equal(ras, want["raster"])
-        bptt = training.Glif3Bptt(sim)
+        bptt = training.Glif3Bptt(sim, blocked=n_blocks > 0, n_blocks=n_blocks or None)
         for f, k0, c in reversed(runs):
             bptt.backward(f, dl_dz=a[k0:k0 + c].contiguous())
         grads.append((bptt.d_rec_w.cpu().numpy(), bptt.d_inp_w.cpu().numpy()))
-    for one, three in zip(grads[0], grads[1]):
+    for one, three, blocked in zip(*grads):
         assert np.abs(one).max() > 0
         np.testing.assert_allclose(one, three, rtol=0, atol=1e-6 * np.abs(one).max())
+        # the blocked table adds a row's synapses range by range: another order, the same sums to rounding
+        np.testing.assert_allclose(one, blocked, rtol=0, atol=1e-5 * np.abs(one).max())
