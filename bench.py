@@ -166,7 +166,10 @@ def bench_compaction(torch, steps=200, warmup=20):
     return out
 
 
-def bench_propagation(torch, steps=200, warmup=20):
+PROPAGATION_MODES = ("scatter", "gather", "auto", "pull")
+
+
+def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES):
     """Isolated spike propagation: 51,978 neurons, Poisson(1000) in-degree
     (~52 M synapses), batch 64, Bernoulli spikes at 1, 5 and 20 Hz."""
     from bmtk_amd import ops, synthetic
@@ -196,7 +199,7 @@ def bench_propagation(torch, steps=200, warmup=20):
         events = sum(e for _, _, e in pool_ev) / len(pool_ev)
         hist = torch.stack([pool_bits[k % 4] for k in range(L)])   # spike bits of the last L steps
         syn = torch.zeros(4, ne, device="cuda")
-        for mode in ("scatter", "gather", "auto", "pull"):
+        for mode in modes:
             def one(k):
                 if mode == "scatter":
                     ids, count, _ = pool_ev[k % 4]
@@ -417,6 +420,12 @@ def main():
     ap.add_argument("--no-kernels", action="store_true", help="skip the isolated-kernel measurements")
     ap.add_argument("--kernels", default="state,compaction,propagation,bptt",
                     help="which isolated-kernel measurements to run (comma-separated)")
+    ap.add_argument("--propagation-modes", default=",".join(PROPAGATION_MODES),
+                    help="delivery forms the propagation group times (profiler runs leave out 'auto', which launches "
+                         "the scatter and gather kernels too and would be pooled with them)")
+    ap.add_argument("--only-kernels", action="store_true",
+                    help="run only the isolated-kernel measurements of --kernels (for profiler runs); prints a line "
+                         "with just their entries")
     ap.add_argument("--per-step", action="store_true", help="force one launch per step instead of resident mode")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy 10 times (reference for scaling the FETCH_SIZE / "
@@ -438,6 +447,19 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "copies": 10}))
+        return
+
+    modes = tuple(m for m in args.propagation_modes.split(",") if m)
+    if set(modes) - set(PROPAGATION_MODES):
+        sys.exit("bench.py: --propagation-modes takes %s" % ", ".join(PROPAGATION_MODES))
+    groups = {"state": bench_state_update, "compaction": bench_compaction,
+              "propagation": lambda t: bench_propagation(t, modes=modes), "bptt": bench_bptt}
+    want = [g for g in args.kernels.split(",") if g]
+    unknown = set(want) - set(groups)
+    if unknown:
+        sys.exit("bench.py: unknown --kernels entries: %s" % ", ".join(sorted(unknown)))
+    if args.only_kernels:
+        print(json.dumps({"only_kernels": True, "kernels": sum((groups[g](torch) for g in groups if g in want), [])}))
         return
 
     K, W, S = args.steps, args.warmup, args.sim_steps
@@ -507,15 +529,8 @@ def main():
                      "frac_at_the_margin": alg_step / slope / 1e9 / HBM_PEAK_GBS},
     }
     if not args.no_kernels:
-        want = set(args.kernels.split(","))
-        unknown = want - {"state", "compaction", "propagation", "bptt"}
-        if unknown:
-            sys.exit("bench.py: unknown --kernels entries: %s" % ", ".join(sorted(unknown)))
         del passes
-        line["kernels"] = ((bench_state_update(torch) if "state" in want else []) +
-                           (bench_compaction(torch) if "compaction" in want else []) +
-                           (bench_propagation(torch) if "propagation" in want else []) +
-                           (bench_bptt(torch) if "bptt" in want else []))
+        line["kernels"] = sum((groups[g](torch) for g in groups if g in want), [])
     if args.cpu_steps > 0:
         line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, settled, max(CPU_MIN_STEPS, args.cpu_steps))
     print(json.dumps(line))
