@@ -219,21 +219,6 @@ constexpr int kBlkMaxGroups = 8;  // row groups per wavefront and sweep: one byt
 constexpr int kBlkInFlight = 8;   // synapses of a row in flight
 static_assert(kBlkInFlight % 8 == 0 && 2 * kBlkInFlight <= BMTK_BLOCKED_PAD, "the kernel reads up to 2*kBlkInFlight - 1 records past a row's end");
 
-// 24-bit multiplies (full rate; the compiler turns __umul24 with a uniform operand into the quarter-rate 32-bit
-// multiply).  Only bits 0-23 of a and b count.
-__device__ __forceinline__ unsigned mul_u24(unsigned a, unsigned b)
-{
-    unsigned r;
-    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return r;
-}
-__device__ __forceinline__ unsigned mad_u24(unsigned a, unsigned b, unsigned c)
-{
-    unsigned r;
-    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
-
 // the value of `x` in the lane a data-parallel-primitive control word names (all of the ones used here have a source)
 template <int kCtrl>
 __device__ __forceinline__ float dpp_move(float x)

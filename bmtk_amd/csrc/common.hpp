@@ -52,20 +52,36 @@ __device__ __forceinline__ unsigned long long bcast_u64(unsigned long long v, in
     return ((unsigned long long)hi << 32) | lo;
 }
 
+// 24-bit multiplies (full rate; the compiler turns __umul24 with a uniform operand into the quarter-rate 32-bit
+// multiply).  Only bits 0-23 of a and b count.
+__device__ __forceinline__ unsigned mul_u24(unsigned a, unsigned b)
+{
+    unsigned r;
+    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ unsigned mad_u24(unsigned a, unsigned b, unsigned c)
+{
+    unsigned r;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // inclusive prefix sum over the 64 lanes, with data-parallel-primitive moves (no LDS round trips): sums of 4
 // by three one-lane shifts within a row of 16, then shifts by 4 and 8 confined to the lanes that have such a
 // neighbour, then the last lane of row 0 (2) is added to row 1 (3) and lane 31 to the upper half
-#define BMTK_DPP(src, ctrl, row_mask, bank_mask) \
-    ((unsigned)__builtin_amdgcn_update_dpp(0, (int)(src), (ctrl), (row_mask), (bank_mask), false))
+#define BMTK_DPP(src, ctrl, row_mask, bank_mask, bound) \
+    ((unsigned)__builtin_amdgcn_update_dpp(0, (int)(src), (ctrl), (row_mask), (bank_mask), (bound)))
 __device__ __forceinline__ unsigned wave_inclusive_scan(unsigned v)
 {
-    unsigned t = v + BMTK_DPP(v, 0x111, 0xF, 0xF);  // row_shr:1
-    t += BMTK_DPP(v, 0x112, 0xF, 0xF);              // row_shr:2
-    t += BMTK_DPP(v, 0x113, 0xF, 0xF);              // row_shr:3
-    t += BMTK_DPP(t, 0x114, 0xF, 0xE);              // row_shr:4, lanes 4..15 of each row
-    t += BMTK_DPP(t, 0x118, 0xF, 0xC);              // row_shr:8, lanes 8..15
-    t += BMTK_DPP(t, 0x142, 0xA, 0xF);              // row_bcast:15 into rows 1 and 3
-    t += BMTK_DPP(t, 0x143, 0xC, 0xF);              // row_bcast:31 into rows 2 and 3
+    // lanes without a source read 0 (bound_ctrl), which lets the compiler fold each move into its addition
+    unsigned t = v + BMTK_DPP(v, 0x111, 0xF, 0xF, true);  // row_shr:1
+    t += BMTK_DPP(v, 0x112, 0xF, 0xF, true);              // row_shr:2
+    t += BMTK_DPP(v, 0x113, 0xF, 0xF, true);              // row_shr:3
+    t += BMTK_DPP(t, 0x114, 0xF, 0xE, false);             // row_shr:4, lanes 4..15 of each row
+    t += BMTK_DPP(t, 0x118, 0xF, 0xC, false);             // row_shr:8, lanes 8..15
+    t += BMTK_DPP(t, 0x142, 0xA, 0xF, false);             // row_bcast:15 into rows 1 and 3
+    t += BMTK_DPP(t, 0x143, 0xC, 0xF, false);             // row_bcast:31 into rows 2 and 3
     return t;
 }
 #undef BMTK_DPP

@@ -112,19 +112,20 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
     // part -- the first two synapses of the segments -- the addition is therefore a compare-and-swap loop (a
     // lane repeats only if another thread changed its cell in between, which is rare among 23,000 cells); the
     // thinly populated later ones keep the float atomic.  The sum is the same either way.
+    // ring cell of a synapse: the record's upper byte is delay*4 + receptor, so (slot0 + delay) % L * 4 + receptor
+    // = min(u, u - 4L) with u = slot0*4 + that byte (unsigned), times the span, plus the target's place in it
+    const unsigned q_lo = (unsigned)slot0 * 4u, q_wrap = q_lo - 4u * (unsigned)L;
     auto add = [&](const uint2 sy, bool crowded) {
-        int slot = slot0 + (int)(sy.x >> 26);
-        slot = slot >= L ? slot - L : slot;
-        const int r = (sy.x >> 24) & 3;
-        const int i = (int)(sy.x & 0xFFFFFFu) - e0;
-        float *cell = ring_l + (slot * GLIF3_NREC + r) * span + i;
+        const unsigned dq = sy.x >> 24;
+        const unsigned plane = min(dq + q_lo, dq + q_wrap);
+        float *cell = ring_l + (mul_u24(plane, (unsigned)span) + (sy.x & 0xFFFFFFu) - (unsigned)e0);
         const float w = __uint_as_float(sy.y);
         if (!crowded) {
             atomicAdd(cell, w);
             return;
         }
         unsigned *bits = reinterpret_cast<unsigned *>(cell);
-        unsigned old = *reinterpret_cast<volatile unsigned *>(bits);
+        unsigned old = *bits;  // only seeds the loop: a stale value costs one more round
         while (true) {
             const unsigned seen = atomicCAS(bits, old, __float_as_uint(__uint_as_float(old) + w));
             if (seen == old) break;
@@ -174,10 +175,17 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
         PROF_T(p0);
         unsigned long long v[kScanWords];
         unsigned cnt = 0;
+        // words past the end are read from the row's last word, which nothing ever writes (it stays zero):
+        // no branch round the loads
+        if (has_rec) {
 #pragma unroll
-        for (int u = 0; u < kScanWords; ++u) {
-            const int64_t w = w0 + (int64_t)u * kResBlock + tid;
-            v[u] = w < n_words ? __hip_atomic_load(bits + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+            for (int u = 0; u < kScanWords; ++u) {
+                const unsigned w = min((unsigned)w0 + (unsigned)(u * kResBlock + tid), (unsigned)words);
+                v[u] = __hip_atomic_load(bits + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kScanWords; ++u) v[u] = 0ull;
         }
         const int64_t ke = k0 + round * kResBlock + tid;
         const bool has_event = ke < k1;

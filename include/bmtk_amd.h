@@ -222,7 +222,8 @@ typedef struct bmtk_glif3_sim {
     const float *i_ext;          /* [ne] constant external current or NULL */
     uint64_t *work_bits;         /* history of spike bits, hist_slots rows of ceil(ne/64)+1 words: the spikes
                                   * of step t live in row t % hist_slots.  Zero it before the first run and
-                                  * leave it alone between runs that continue one another. */
+                                  * leave it alone between runs that continue one another (the last word of
+                                  * every row is never written and must stay zero). */
     /* Long delays.  NEST networks have a minimum delay, often far above one step (1-2 ms at a 0.001-0.1 ms
      * resolution).  With delay_offset = B every delay stored in the two tables is the true delay minus B steps
      * (still >= 1) and the spikes and input events of step u are handed to the tables B steps late, from the
