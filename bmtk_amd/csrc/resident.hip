@@ -254,10 +254,15 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
     }
 }
 
-// kLate: the run has slack (S > 0), see the loop body
-template <bool kLate>
+// kLate: the run has slack (S > 0), see the loop body.  kExtras: membrane potential probes or a spike list are
+// asked for; without them their pointers and counters are out of the loop, which is short of scalar registers.
+template <bool kLate, bool kExtras>
 __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim s, Resident r)
 {
+    if (!kExtras) {
+        s.probe_col = nullptr;
+        s.spike_count = nullptr;
+    }
     extern __shared__ float ring_l[];  // [L*4][span], then the active-row list
     __shared__ int go_on;
     __shared__ unsigned scan_l[kResBlock / kWave];
@@ -313,6 +318,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     // next step is fetched a step ahead.  Steps before 0 have no events (in_ptr[0] = 0).
     const int B = r.offset;
     auto in_bound = [&](int64_t i) -> int64_t { return (s.in_ptr && i > 0) ? s.in_ptr[i] : 0; };
+    int opaque_zero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(opaque_zero));
     int64_t ka = 0, kb = in_bound(r.step0 - B);
 #ifdef BMTK_RES_PROFILE
     long long prof_prev = 0, prof_c1 = 0;
@@ -375,7 +382,12 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
 #ifdef BMTK_RES_PROFILE
         if (k > 0) PROF_ADD(1, prof_prev, c0);
 #endif
-        const int64_t kn = in_bound(t + 1 - B);
+        // The bound of the next step's events is asked for now and looked at after the pull.  The address gets a
+        // zero the compiler cannot see through: a load it knows to be the same in every lane is moved to a scalar
+        // register on the spot, and every wavefront would wait for the answer here, at the top of the step.
+        const int64_t in_next = t + 1 - B;
+        long long kn_lanes = 0;
+        if (s.in_ptr && in_next > 0) kn_lanes = s.in_ptr[in_next + opaque_zero];
         if (defer && k > 0 && tid == kLooker) go_on = poll(k - 1);
         // 1. fold the arrivals of slot t-1 and update
         bool spike = false;
@@ -456,7 +468,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         if (k > 0 && t - 1 - B >= 0 && mine > 0)
             pull_step(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb);
         ka = kb;
-        kb = kn;
+        kb = ((int64_t)__builtin_amdgcn_readfirstlane((int)(kn_lanes >> 32)) << 32) |
+             (int64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)kn_lanes);
         if (late) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __syncthreads();
@@ -565,8 +578,12 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     slack = slack < kMaxSlack ? slack : kMaxSlack;
     Resident r{step0, n_steps, s.res_span, s.res_groups, s.delay_offset, hist, slack, slack / 2 + 1};
     const size_t lds = (size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) + kActCap * sizeof(int);
-    const void *kernel = slack > 0 ? reinterpret_cast<const void *>(sim_resident_kernel<true>)
-                                   : reinterpret_cast<const void *>(sim_resident_kernel<false>);
+    const bool extras = s.probe_col != nullptr || s.spike_count != nullptr;
+    const void *kernel =
+        slack > 0 ? (extras ? reinterpret_cast<const void *>(sim_resident_kernel<true, true>)
+                            : reinterpret_cast<const void *>(sim_resident_kernel<true, false>))
+                  : (extras ? reinterpret_cast<const void *>(sim_resident_kernel<false, true>)
+                            : reinterpret_cast<const void *>(sim_resident_kernel<false, false>));
     hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) {
         set_error("glif3_simulate_fwd: resident mode needs %zu bytes of LDS: %s", lds, hipGetErrorString(err));
@@ -577,10 +594,7 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     int dev = 0, n_cu = 0, per_cu = 0;
     (void)hipGetDevice(&dev);
     (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
-    if (slack > 0)
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, sim_resident_kernel<true>, kResBlock, lds);
-    else
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, sim_resident_kernel<false>, kResBlock, lds);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kResBlock, lds);
     if ((int64_t)per_cu * n_cu < (int64_t)grid) {
         set_error("glif3_simulate_fwd: %u resident workgroups do not fit the device (%d compute units x %d)", grid,
                   n_cu, per_cu);
@@ -591,16 +605,11 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     // BMTK_AMD_PLAIN_LAUNCH=1 uses an ordinary launch (co-residency then rests on the occupancy check
     // above and an otherwise idle device); for tools that cannot follow cooperative launches.
     const char *plain = getenv("BMTK_AMD_PLAIN_LAUNCH");
-    if (plain && plain[0] == '1') {
-        if (slack > 0)
-            hipLaunchKernelGGL(sim_resident_kernel<true>, dim3(grid), dim3(kResBlock), lds, stream, s_copy, r);
-        else
-            hipLaunchKernelGGL(sim_resident_kernel<false>, dim3(grid), dim3(kResBlock), lds, stream, s_copy, r);
-        err = hipGetLastError();
-    } else {
-        void *args[] = {&s_copy, &r};
+    void *args[] = {&s_copy, &r};
+    if (plain && plain[0] == '1')
+        err = hipLaunchKernel(kernel, dim3(grid), dim3(kResBlock), args, lds, stream);
+    else
         err = hipLaunchCooperativeKernel(kernel, dim3(grid), dim3(kResBlock), args, lds, stream);
-    }
     if (err != hipSuccess) {
         set_error("glif3_simulate_fwd: launch of %u resident workgroups failed: %s", grid, hipGetErrorString(err));
         return BMTK_E_LAUNCH;
