@@ -156,6 +156,9 @@ constexpr unsigned kInputTag = 0x80000000u;
 // event (independent loads), a workgroup-wide prefix sum packs the rows that
 // fired into one LDS list, then one thread per listed row pulls this
 // workgroup's segment of it.  Must be called by all threads of the workgroup.
+// kUnified: the input rows follow the recurrent rows in ONE table (inp_seg = rec_seg + n_neurons*(n_groups+1), both
+// sets of offsets index rec_packed), so a listed row needs no choice between two tables.
+template <bool kUnified>
 __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int hist_row, int slot0,
                                           float *ring_l, unsigned *act, unsigned *scan_l, int e0, int64_t words,
                                           int64_t k0, int64_t k1)
@@ -214,7 +217,7 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
                     act[pos++] = j0 + (unsigned)bit;
                 }
             }
-            if (has_event) act[pos] = event_row | kInputTag;
+            if (has_event) act[pos] = kUnified ? event_row + (unsigned)s.n_neurons : event_row | kInputTag;
         } else {
             // more rows than the list holds: every thread pulls what it found itself, unbalanced but correct
             for (int u = 0; u < kScanWords; ++u) {
@@ -227,9 +230,14 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
                                  slot0);
                 }
             }
-            if (has_event)
-                pull_segment(s.inp_seg + (int64_t)event_row * (r.n_groups + 1), g, s.inp_packed, ring_l, r.span, e0,
-                             L, slot0);
+            if (has_event) {
+                if (kUnified)
+                    pull_segment(s.rec_seg + (s.n_neurons + (int64_t)event_row) * (r.n_groups + 1), g, s.rec_packed, ring_l,
+                                 r.span, e0, L, slot0);
+                else
+                    pull_segment(s.inp_seg + (int64_t)event_row * (r.n_groups + 1), g, s.inp_packed, ring_l, r.span, e0,
+                                 L, slot0);
+            }
         }
         __syncthreads();
         PROF_T(p2);
@@ -238,11 +246,16 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
                 // one code path for both kinds of rows: a wavefront nearly always holds some of each, and a
                 // branch would make it walk the two chains of dependent loads one after the other
                 const unsigned entry = act[a];
-                const int64_t row = entry & ~kInputTag;
-                const bool is_input = (entry & kInputTag) != 0u;
-                const uint32_t *seg = is_input ? s.inp_seg : s.rec_seg;
-                const bmtk_synapse *tab = is_input ? s.inp_packed : s.rec_packed;
-                pull_segment(seg + row * (r.n_groups + 1), g, tab, ring_l, r.span, e0, L, slot0);
+                if (kUnified) {  // rows * (n_groups + 1) stays below 2^32 (checked before the launch)
+                    pull_segment(s.rec_seg + mul_u24(entry, (unsigned)(r.n_groups + 1)), g, s.rec_packed, ring_l, r.span,
+                                 e0, L, slot0);
+                } else {
+                    const int64_t row = entry & ~kInputTag;
+                    const bool is_input = (entry & kInputTag) != 0u;
+                    const uint32_t *seg = is_input ? s.inp_seg : s.rec_seg;
+                    const bmtk_synapse *tab = is_input ? s.inp_packed : s.rec_packed;
+                    pull_segment(seg + row * (r.n_groups + 1), g, tab, ring_l, r.span, e0, L, slot0);
+                }
             }
         }
         __syncthreads();
@@ -254,14 +267,17 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
     }
 }
 
-// kLate: the run has slack (S > 0), see the loop body.  kExtras: membrane potential probes or a spike list are
-// asked for; without them their pointers and counters are out of the loop, which is short of scalar registers.
-template <bool kLate, bool kExtras>
+// kLate: the run has slack (S > 0), see the loop body.  kLean: no membrane potential probes and no spike list are
+// asked for and the two tables are one (pull_step); their pointers and counters are then out of the loop, which is
+// short of scalar registers (98 spilled in the general form; every use in the loop is a lane read).
+template <bool kLate, bool kLean>
 __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim s, Resident r)
 {
-    if (!kExtras) {
+    if (kLean) {
         s.probe_col = nullptr;
         s.spike_count = nullptr;
+        s.inp_seg = nullptr;
+        s.inp_packed = nullptr;
     }
     extern __shared__ float ring_l[];  // [L*4][span], then the active-row list
     __shared__ int go_on;
@@ -466,7 +482,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         // 3. pull the spikes and input events of step t-1-B while the barrier fills (the first step of a
         //    call pulls nothing: the call before it closed with that pull)
         if (k > 0 && t - 1 - B >= 0 && mine > 0)
-            pull_step(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb);
+            pull_step<kLean>(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb);
         ka = kb;
         kb = ((int64_t)__builtin_amdgcn_readfirstlane((int)(kn_lanes >> 32)) << 32) |
              (int64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)kn_lanes);
@@ -508,7 +524,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         // closing: spikes and inputs of the last step (less the delay offset), then fold the last slot
         const int64_t tl = r.step0 + done - 1;
         if (tl - B >= 0 && mine > 0)
-            pull_step(s, r, g, wrap(tl - B, r.hist), wrap(tl, L), ring_l, act, scan_l, e0, words, ka, kb);
+            pull_step<kLean>(s, r, g, wrap(tl - B, r.hist), wrap(tl, L), ring_l, act, scan_l, e0, words, ka, kb);
         __syncthreads();
         if (own) {
             float *prev = ring_l + (int)(tl % L) * GLIF3_NREC * span + tid;
@@ -578,12 +594,18 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     slack = slack < kMaxSlack ? slack : kMaxSlack;
     Resident r{step0, n_steps, s.res_span, s.res_groups, s.delay_offset, hist, slack, slack / 2 + 1};
     const size_t lds = (size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) + kActCap * sizeof(int);
-    const bool extras = s.probe_col != nullptr || s.spike_count != nullptr;
+    // the lean form: nothing asked for beyond spike bits, and one table for recurrent and input rows
+    const bool has_inputs = s.in_ptr != nullptr;
+    const int64_t rows = s.n_neurons + (has_inputs ? s.n_inputs : 0);
+    const bool unified = s.rec_seg != nullptr && rows < (1ll << 24) && rows * (s.res_groups + 1) < (1ll << 32) &&
+                         (!has_inputs || (s.inp_packed == s.rec_packed &&
+                                          s.inp_seg == s.rec_seg + s.n_neurons * (int64_t)(s.res_groups + 1)));
+    const bool lean = unified && s.probe_col == nullptr && s.spike_count == nullptr;
     const void *kernel =
-        slack > 0 ? (extras ? reinterpret_cast<const void *>(sim_resident_kernel<true, true>)
-                            : reinterpret_cast<const void *>(sim_resident_kernel<true, false>))
-                  : (extras ? reinterpret_cast<const void *>(sim_resident_kernel<false, true>)
-                            : reinterpret_cast<const void *>(sim_resident_kernel<false, false>));
+        slack > 0 ? (lean ? reinterpret_cast<const void *>(sim_resident_kernel<true, true>)
+                          : reinterpret_cast<const void *>(sim_resident_kernel<true, false>))
+                  : (lean ? reinterpret_cast<const void *>(sim_resident_kernel<false, true>)
+                          : reinterpret_cast<const void *>(sim_resident_kernel<false, false>));
     hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) {
         set_error("glif3_simulate_fwd: resident mode needs %zu bytes of LDS: %s", lds, hipGetErrorString(err));

@@ -150,7 +150,7 @@ class Glif3Simulator:
             raise ValueError("the packed synapse tables index at most 2^24 neurons")
         self.res_sync = torch.zeros(_lib.RES_SYNC_WORDS, dtype=torch.int32, device=self.dev)
         self.res_span = self.res_groups = 0
-        self.rec_seg = self.inp_seg = None
+        self.rec_seg = self.inp_seg = self.res_unified = None
         self._pending_check = False
         self.probe_ids = self.probe_col = None
         self.probe_every = 1
@@ -199,6 +199,21 @@ class Glif3Simulator:
         if self.inp is not None:
             self.inp = self.inp.sorted_by_index()
             self.inp_seg = self.inp.segment_offsets(span, groups)
+        self.res_unified = None
+        if self.rec is not None and self.inp is not None and self.rec.nnz + self.inp.nnz < (1 << 32):
+            # One table for both kinds of rows, the input rows behind the recurrent ones: the kernel then needs no
+            # choice between two tables per listed row (and fewer of its scarce scalar registers).  The packed
+            # records of the two tables become views of the joint array; the input offsets count from its start.
+            nr, ni = self.rec.nnz, self.inp.nnz
+            packed = torch.empty(max(nr + ni, 1), 2, dtype=torch.int32, device=self.dev)
+            packed[:nr] = self.rec.packed()[:nr]
+            packed[nr:nr + ni] = self.inp.packed()[:ni]
+            self.rec._packed, self.inp._packed = packed[:nr], packed[nr:nr + ni]
+            seg = torch.empty(self.n + self.inp.n_rows, groups + 1, dtype=torch.int32, device=self.dev)
+            seg[:self.n] = self.rec_seg
+            seg[self.n:] = ((self.inp_seg.long() & 0xFFFFFFFF) + nr).to(torch.int32)   # uint32 kept in int32
+            self.rec_seg, self.inp_seg = seg[:self.n], seg[self.n:]
+            self.res_unified = (packed, seg)
         self.res_span, self.res_groups = span, groups
 
     def check(self):
@@ -295,6 +310,8 @@ class Glif3Simulator:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
             s.res_spin_limit = int(self.spin_limit)
             s.rec_seg, s.inp_seg = _p(self.rec_seg), _p(self.inp_seg)
+            if self.res_unified is not None and s.inp_packed:
+                s.inp_packed = s.rec_packed      # the input offsets count from the start of the joint table
         if bits is not None:
             s.spike_bits, s.spike_bits_stride = _p(bits), bits.shape[1]
         if record is not None:
