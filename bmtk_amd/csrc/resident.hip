@@ -90,6 +90,15 @@ __device__ __forceinline__ unsigned load_agent(const unsigned *p)
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Wait until every vector memory operation this wavefront has issued is complete: its loads have returned and
+// its stores -- the write-through, device-coherent ballot store among them -- have been acknowledged.  A release
+// fence of workgroup scope does NOT do this: on this target it waits for LDS and scalar operations only, because
+// the wavefronts of a workgroup share one vector cache.
+__device__ __forceinline__ void wait_vector_memory()
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // add the weights of one row's synapses that target this workgroup's group,
 // positions [seg_row[g], seg_row[g+1]) of the packed table, to the LDS ring
 // slice.  Every lane of a wavefront reads a different cache line here, and the
@@ -156,12 +165,16 @@ constexpr unsigned kInputTag = 0x80000000u;
 // event (independent loads), a workgroup-wide prefix sum packs the rows that
 // fired into one LDS list, then one thread per listed row pulls this
 // workgroup's segment of it.  Must be called by all threads of the workgroup.
+// `arrival`, when not null, is the grid barrier counter this workgroup still has to bump for the step whose
+// ballots its wavefronts have just stored: the bump may only happen once every one of those stores has been
+// acknowledged, and the cheapest place to wait for that is where each wavefront waits for its scan loads anyway.
+// Returns true when the bump has been made.
 // kUnified: the input rows follow the recurrent rows in ONE table (inp_seg = rec_seg + n_neurons*(n_groups+1), both
 // sets of offsets index rec_packed), so a listed row needs no choice between two tables.
 template <bool kUnified>
-__device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int hist_row, int slot0,
-                                          float *ring_l, unsigned *act, unsigned *scan_l, int e0, int64_t words,
-                                          int64_t k0, int64_t k1)
+__device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int hist_row, int slot0,
+                                          float *ring_l, unsigned *act, unsigned *scan_l, int e0, int words,
+                                          int64_t k0, int64_t k1, unsigned *arrival = nullptr)
 {
     const int tid = threadIdx.x;
     const int L = s.ring_slots;
@@ -169,12 +182,13 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
     const bool has_rec = s.rec_seg != nullptr;
     const unsigned long long *bits =
         reinterpret_cast<const unsigned long long *>(s.work_bits) + (int64_t)hist_row * (words + 1);
-    const int64_t n_words = has_rec ? words : 0;
-    const int64_t word_rounds = (n_words + (int64_t)kScanWords * kResBlock - 1) / ((int64_t)kScanWords * kResBlock);
-    const int64_t event_rounds = (k1 - k0 + kResBlock - 1) / kResBlock;
-    const int64_t rounds = word_rounds > event_rounds ? word_rounds : event_rounds;
-    for (int64_t round = 0; round < rounds; ++round) {
-        const int64_t w0 = round * (int64_t)kScanWords * kResBlock;
+    // 32-bit counters wherever the sizes allow: the loop is short of scalar registers
+    const int n_words = has_rec ? words : 0;
+    const int word_rounds = (n_words + kScanWords * kResBlock - 1) / (kScanWords * kResBlock);
+    const int event_rounds = (int)((k1 - k0 + kResBlock - 1) / kResBlock);  // a step's events are below 2^31
+    const int rounds = word_rounds > event_rounds ? word_rounds : event_rounds;
+    for (int round = 0; round < rounds; ++round) {
+        const int w0 = round * kScanWords * kResBlock;
         PROF_T(p0);
         unsigned long long v[kScanWords];
         unsigned cnt = 0;
@@ -190,7 +204,7 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
 #pragma unroll
             for (int u = 0; u < kScanWords; ++u) v[u] = 0ull;
         }
-        const int64_t ke = k0 + round * kResBlock + tid;
+        const int64_t ke = k0 + (round * kResBlock + tid);
         const bool has_event = ke < k1;
         const unsigned event_row = has_event ? (unsigned)s.in_events[ke] : 0u;
 #pragma unroll
@@ -198,7 +212,10 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
         cnt += has_event ? 1u : 0u;
         const unsigned inc = wave_inclusive_scan(cnt);
         if (lane_id() == kWave - 1) scan_l[wave] = inc;
+        if (arrival && round == 0) wait_vector_memory();  // the loads are back already; this is for the ballot store
         __syncthreads();
+        if (arrival && round == 0 && tid == 0)
+            __hip_atomic_fetch_add(arrival, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         PROF_T(p1);
         // prefix over the 16 wavefront sums: one LDS read per lane and one more scan instead of 16 reads
         const unsigned part = wave_inclusive_scan(lane_id() < kResBlock / kWave ? scan_l[lane_id()] : 0u);
@@ -210,7 +227,7 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
 #pragma unroll
             for (int u = 0; u < kScanWords; ++u) {
                 unsigned long long x = v[u];
-                const unsigned j0 = (unsigned)((w0 + (int64_t)u * kResBlock + tid) << 6);
+                const unsigned j0 = (unsigned)(w0 + u * kResBlock + tid) << 6;
                 while (x) {
                     const int bit = __ffsll((long long)x) - 1;
                     x &= x - 1ull;
@@ -222,7 +239,7 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
             // more rows than the list holds: every thread pulls what it found itself, unbalanced but correct
             for (int u = 0; u < kScanWords; ++u) {
                 unsigned long long x = v[u];
-                const int64_t j0 = (w0 + (int64_t)u * kResBlock + tid) << 6;
+                const int64_t j0 = (int64_t)(w0 + u * kResBlock + tid) << 6;
                 while (x) {
                     const int bit = __ffsll((long long)x) - 1;
                     x &= x - 1ull;
@@ -265,6 +282,7 @@ __device__ __forceinline__ void pull_step(const bmtk_glif3_sim &s, const Residen
         PROF_ADD(6, p2, p3);
         PROF_BLK(3, p2, p3);
     }
+    return arrival != nullptr && rounds > 0;
 }
 
 // kLate: the run has slack (S > 0), see the loop body.  kLean: no membrane potential probes and no spike list are
@@ -290,14 +308,14 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     // contiguous and are fetched into that XCD's L2 once.
     const int per_xcd = (int)gridDim.x >> 3;
     const int g = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    const int64_t ne = s.n_neurons;  // batch 1
-    const int64_t words = (ne + 63) >> 6;
+    const int ne = (int)s.n_neurons;  // batch 1, at most 1024 elements per compute unit
+    const int words = (ne + 63) >> 6;
     const int L = s.ring_slots;
     const int span = r.span;
     const int e0 = g * span;
-    const int mine = (int)max((int64_t)0, min((int64_t)span, ne - e0));  // groups past the end own nothing
+    const int mine = max(0, min(span, ne - e0));  // groups past the end own nothing
     const bool own = tid < mine;
-    const int64_t e = e0 + tid;
+    const int e = e0 + tid;
     unsigned *act = reinterpret_cast<unsigned *>(ring_l + s.ring_slots * GLIF3_NREC * r.span);
     unsigned *abort_word = s.res_sync + 1;
     unsigned *arrivals = s.res_sync + kBarrierStride;  // [kBarrierWords] counters, kBarrierStride words apart
@@ -329,7 +347,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     int64_t probe_row = 0;
     const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
     bool aborted = false;
-    int64_t done = 0;  // steps whose update has run
+    int done = 0;  // steps whose update has run
     // the input events of the step pulled in step t, u = t-1-B, are in_events[ka, kb); the bound for the
     // next step is fetched a step ahead.  Steps before 0 have no events (in_ptr[0] = 0).
     const int B = r.offset;
@@ -344,8 +362,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     // false = the run was given up).  No acquire fence: it would invalidate this XCD's L2 every step, and
     // the only data other workgroups write during the run are the ballots, which are read with agent-scope
     // loads that bypass the non-coherent caches.
-    auto counter_of = [&](int64_t j) { return arrivals + ((j < 0 ? 0 : j) & (kBarrierWords - 1)) * kBarrierStride; };
-    auto poll = [&](int64_t j) -> int {  // one thread: 1 = everybody arrived at step j, 0 = given up
+    auto counter_of = [&](int j) { return arrivals + ((j < 0 ? 0 : j) & (kBarrierWords - 1)) * kBarrierStride; };
+    auto poll = [&](int j) -> int {  // one thread: 1 = everybody arrived at step j, 0 = given up
         const unsigned *word = counter_of(j);
         const unsigned target = j < 0 ? 0u : gridDim.x * (unsigned)(j / kBarrierWords + 1);
         unsigned spins = 0;
@@ -368,7 +386,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         }
         return 1;
     };
-    auto wait_for = [&](int64_t j) -> bool {
+    auto wait_for = [&](int j) -> bool {
         if (tid == 0) go_on = poll(j);
         __syncthreads();
         return go_on != 0;
@@ -388,7 +406,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     auto wrap = [](int64_t a, int m) { return (int)(((a % m) + m) % m); };
     int next_slot_prev = wrap(r.step0 - 1, L), next_row_t = wrap(r.step0, r.hist),
         next_row_p = wrap(r.step0 - 1 - B, r.hist);
-    for (int64_t k = 0; k < r.n_steps; ++k) {
+    const int n_steps = (int)r.n_steps;
+    for (int k = 0; k < n_steps; ++k) {
         const int64_t t = r.step0 + k;
         const int slot_prev = next_slot_prev, row_t = next_row_t, row_p = next_row_p;
         next_slot_prev = slot_prev + 1 == L ? 0 : slot_prev + 1;
@@ -429,7 +448,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         }
         const unsigned long long m = __ballot(spike);
         // only the wavefronts that cover this workgroup's span own a ballot word
-        if (lane == 0 && tid < span && (e & ~(int64_t)(kWave - 1)) < ne) {
+        if (lane == 0 && tid < span && (e & ~(kWave - 1)) < ne) {
             __hip_atomic_store(reinterpret_cast<unsigned long long *>(s.work_bits) + (int64_t)row_t * (words + 1) + (e >> 6),
                                m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (s.spike_bits) s.spike_bits[k * s.spike_bits_stride + (e >> 6)] = m;
@@ -447,24 +466,17 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
             }
         }
         done = k + 1;
-        // With no slack (S = 0) the arrival is signalled before the pull so that the barrier fills while
+        // With no slack (S = 0) the arrival is signalled early in the pull so that the barrier fills while
         // the pull runs.  With slack nobody is waiting for this step yet: the arrival moves behind the pull,
-        // which saves a workgroup barrier and the wait for the ballot store, and the counters are only
-        // looked at every `check` steps.
+        // which saves a workgroup barrier, and the counters are only looked at every `check` steps.
         constexpr bool late = kLate;
         const int check = late ? r.check : 1;
+        unsigned *const my_counter = counter_of(k) + (blockIdx.x & (kWays - 1)) * kWayStride;
         if (!late) {
-            // Every wavefront waits until its own ballot store (a write-through, device-coherent
-            // store) has been acknowledged, then the workgroup meets; only after that does the
-            // barrier count move.  No L2 write-back is needed: nothing else written inside the
-            // loop is read by another workgroup before the kernel ends.
+            // the workgroup meets, so that the looker's answer can be read
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __syncthreads();
             PROF_T(c1);
-            // 2. arrive at the barrier of step t (ballots of this workgroup are out)
-            if (tid == 0)
-                __hip_atomic_fetch_add(counter_of(k) + (blockIdx.x & (kWays - 1)) * kWayStride, 1u, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
             PROF_ADD(0, c0, c1);
             PROF_BLK(0, c0, c1);
 #ifdef BMTK_RES_PROFILE
@@ -479,29 +491,40 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
 #ifdef BMTK_RES_PROFILE
         if (!kLate) PROF_ADD(7, prof_c1, c2);
 #endif
-        // 3. pull the spikes and input events of step t-1-B while the barrier fills (the first step of a
-        //    call pulls nothing: the call before it closed with that pull)
+        // 2. + 3. pull the spikes and input events of step t-1-B (the first step of a call pulls nothing: the
+        //    call before it closed with that pull) and, without slack, arrive at the barrier of step t on the
+        //    way, so that the barrier fills while the pull runs.  The arrival tells the other workgroups that
+        //    this one's ballots of step t can be read: it must not move before every wavefront's ballot store
+        //    (a write-through, device-coherent store) has been acknowledged, which each wavefront waits for
+        //    together with the first loads of the pull.  No L2 write-back is needed: nothing else written
+        //    inside the loop is read by another workgroup before the kernel ends.
+        bool arrived = false;
         if (k > 0 && t - 1 - B >= 0 && mine > 0)
-            pull_step<kLean>(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb);
+            arrived = pull_step<kLean>(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb,
+                                       late ? nullptr : my_counter);
+        if (!late && !arrived) {
+            wait_vector_memory();
+            __syncthreads();
+            if (tid == 0) __hip_atomic_fetch_add(my_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         ka = kb;
         kb = ((int64_t)__builtin_amdgcn_readfirstlane((int)(kn_lanes >> 32)) << 32) |
              (int64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)kn_lanes);
         if (late) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            // every wavefront's ballot store has been acknowledged before the workgroup meets and arrives
+            wait_vector_memory();
             __syncthreads();
         }
         // (without slack no workgroup barrier is needed here: pull_step ends with one, and the word thread 0
         //  writes below was last read before the barrier that precedes the arrival)
         PROF_T(c3);
-        if (late && tid == 0)
-            __hip_atomic_fetch_add(counter_of(k) + (blockIdx.x & (kWays - 1)) * kWayStride, 1u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+        if (late && tid == 0) __hip_atomic_fetch_add(my_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // 4. every `check` steps (each step without slack) wait until every workgroup has published
         //    step k - S + (check - 1): enough for the steps up to the next look
-        if (late && k % check != check - 1 && k + 1 < r.n_steps) continue;
+        if (late && k % check != check - 1 && k + 1 < n_steps) continue;
         bool ok = true;
         if (!defer) {
-            int64_t j = late ? k - r.slack + (check - 1) : k;  // step of this call everybody must have published
+            int j = late ? k - r.slack + (check - 1) : k;  // step of this call everybody must have published
             ok = wait_for(j < k ? j : k);
         }
         PROF_T(c4);
@@ -589,6 +612,10 @@ __global__ __launch_bounds__(kBlock) void segment_offsets_kernel(int64_t n_rows,
 
 int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream)
 {
+    if (n_steps >= (1ll << 31)) {
+        set_error("glif3_simulate_fwd: a resident call covers fewer than 2^31 steps");
+        return BMTK_E_ARG;
+    }
     const int hist = s.hist_slots ? s.hist_slots : 3;
     int slack = s.delay_offset < hist - 3 - s.delay_offset ? s.delay_offset : hist - 3 - s.delay_offset;
     slack = slack < kMaxSlack ? slack : kMaxSlack;
