@@ -123,6 +123,27 @@ template <bool kLdsTable>
 __global__ __launch_bounds__(kBlock) void glif3_step_kernel(StepArgs a)
 {
     extern __shared__ float step_table[];  // [columns][GLIF3_NPROP] when kLdsTable
+    // with the table in LDS a workgroup takes kStepTiles tiles of 256 elements, so that staging the table is
+    // shared by 1024 elements.  The state of all tiles is asked for first, before the table is staged: the loads
+    // of the tiles travel together, and the staging runs while they are on their way.
+    constexpr int kTiles = kLdsTable ? kStepTiles : 1;
+    Glif3Elem s[kTiles];
+    float syn[kTiles][GLIF3_NREC], I[kTiles];
+    int64_t e[kTiles], col[kTiles];
+#pragma unroll
+    for (int t = 0; t < kTiles; ++t) {
+        e[t] = ((int64_t)blockIdx.x * kTiles + t) * kBlock + threadIdx.x;
+        col[t] = 0;
+        I[t] = 0.0f;
+        if (e[t] < a.ne) {
+            const int64_t n = (a.batch == 1) ? e[t] : (int64_t)((uint32_t)e[t] / (uint32_t)a.batch);
+            col[t] = a.class_id ? (int64_t)a.class_id[n] : n;
+            glif3_load(s[t], a.V, a.asc, a.y1, a.y2, a.ref, a.ne, e[t]);
+#pragma unroll
+            for (int k = 0; k < GLIF3_NREC; ++k) syn[t][k] = a.syn ? a.syn[k * a.ne + e[t]] : 0.0f;
+            I[t] = a.i_ext ? a.i_ext[e[t]] : 0.0f;
+        }
+    }
     if (kLdsTable) {
         const int n_cols = (int)a.stride;
         for (int i = threadIdx.x; i < n_cols * GLIF3_NPROP; i += kBlock) {
@@ -131,39 +152,29 @@ __global__ __launch_bounds__(kBlock) void glif3_step_kernel(StepArgs a)
         }
         __syncthreads();
     }
-    // with the table in LDS a workgroup takes kStepTiles tiles of 256 elements, so that staging the table is
-    // shared by 1024 elements
-    for (int tile = 0; tile < (kLdsTable ? kStepTiles : 1); ++tile) {
-    const int64_t e = ((int64_t)blockIdx.x * (kLdsTable ? kStepTiles : 1) + tile) * kBlock + threadIdx.x;
-    bool spike = false;
-    if (e < a.ne) {
-        const int64_t n = (a.batch == 1) ? e : (int64_t)((uint32_t)e / (uint32_t)a.batch);
-        const int64_t col = a.class_id ? (int64_t)a.class_id[n] : n;
-        Glif3Prop p;
-        if (kLdsTable)
-            p.load(step_table + col * GLIF3_NPROP, 1, 0);
-        else
-            p.load(a.prop, a.stride, col);
-        Glif3Elem s;
-        glif3_load(s, a.V, a.asc, a.y1, a.y2, a.ref, a.ne, e);
-        float syn[GLIF3_NREC];
 #pragma unroll
-        for (int k = 0; k < GLIF3_NREC; ++k) syn[k] = a.syn ? a.syn[k * a.ne + e] : 0.0f;
-        const float I = a.i_ext ? a.i_ext[e] : 0.0f;
-        float frac = 0.0f;
-        spike = glif3_update(s, p, a.h, syn, I, &frac);
-        glif3_store(s, a.V, a.asc, a.y1, a.y2, a.ref, a.ne, e);
-        if (a.syn && a.clear_syn) {
+    for (int t = 0; t < kTiles; ++t) {
+        bool spike = false;
+        if (e[t] < a.ne) {
+            Glif3Prop p;
+            if (kLdsTable)
+                p.load(step_table + col[t] * GLIF3_NPROP, 1, 0);
+            else
+                p.load(a.prop, a.stride, col[t]);
+            float frac = 0.0f;
+            spike = glif3_update(s[t], p, a.h, syn[t], I[t], &frac);
+            glif3_store(s[t], a.V, a.asc, a.y1, a.y2, a.ref, a.ne, e[t]);
+            if (a.syn && a.clear_syn) {
 #pragma unroll
-            for (int k = 0; k < GLIF3_NREC; ++k) a.syn[k * a.ne + e] = 0.0f;
+                for (int k = 0; k < GLIF3_NREC; ++k) a.syn[k * a.ne + e[t]] = 0.0f;
+            }
+            if (a.z) a.z[e[t]] = spike ? 1 : 0;
+            if (a.frac && spike) a.frac[e[t]] = frac;
         }
-        if (a.z) a.z[e] = spike ? 1 : 0;
-        if (a.frac && spike) a.frac[e] = frac;
-    }
-    if (a.zbits) {
-        const unsigned long long m = __ballot(spike);
-        if (lane_id() == 0 && (e & ~(int64_t)(kWave - 1)) < a.ne) a.zbits[e >> 6] = m;
-    }
+        if (a.zbits) {
+            const unsigned long long m = __ballot(spike);
+            if (lane_id() == 0 && (e[t] & ~(int64_t)(kWave - 1)) < a.ne) a.zbits[e[t] >> 6] = m;
+        }
     }
 }
 
