@@ -31,6 +31,7 @@ class Glif3Sim(C.Structure):
         ("pull_indptr", c_void_p), ("pull_packed", c_void_p), ("pull_syn", c_void_p), ("pull_work", c_void_p),
         ("pull_inp_indptr", c_void_p), ("pull_inp_packed", c_void_p), ("pull_inp_syn", c_void_p),
         ("pull_inp_work", c_void_p), ("in_hist", c_void_p), ("in_hist_stride", c_int64),
+        ("in_repeat_ptr", c_void_p), ("in_repeat_events", c_void_p),
         ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
         ("save_v", c_void_p), ("save_flags", c_void_p),
         ("probe_col", c_void_p), ("probe_v", c_void_p), ("probe_stride", c_int64), ("probe_every", c_int32),
@@ -57,7 +58,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 13  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 14  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {

@@ -42,6 +42,7 @@ struct SimLaunch {
     int lds_table;     // propagator table staged in LDS
     int pull;          // pull_syn holds the recurrent arrivals of step t-1, to be folded with slot t-1
     int pull_inp;      // pull_inp_syn holds the input arrivals of step t-1
+    int repeats;       // the input workgroups deliver the repeat lists (in_repeat_*) instead of the event lists
     int idx_bits;      // width of the index field of the packed tables (24 in the standard packing)
     int64_t probe_row; // row of probe_v this step's potentials go to, -1: not a sampled step
 };
@@ -91,11 +92,13 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
         // (not those of step t: with L = largest delay + 1 slots, a delay of L-1
         //  from step t would land in slot t-1, which this launch is clearing)
         const int slot0 = (int)((q.t - 1) % L);
-        const int64_t k0 = s.in_ptr[q.src], k1 = s.in_ptr[q.src + 1];
+        const int64_t *__restrict__ ptr = q.repeats ? s.in_repeat_ptr : s.in_ptr;
+        const int32_t *__restrict__ events = q.repeats ? s.in_repeat_events : s.in_events;
+        const int64_t k0 = ptr[q.src], k1 = ptr[q.src + 1];
         const int n_waves = q.n_input * kSimWaves;
         const int wave = bid * kSimWaves + threadIdx.x / kWave;
         for (int64_t k = k0 + wave; k < k1; k += n_waves) {
-            const int e = s.in_events[k];
+            const int e = events[k];
             const int j = batch == 1 ? e : (int)((uint32_t)e / (uint32_t)batch);
             deliver_row_packed(s.inp_indptr, s.inp_packed, j, e - j * batch, batch, s.ring, L, slot0, ne, q.idx_bits);
         }
@@ -367,7 +370,11 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     q.n_update = (int)((ne + kSimBlock - 1) / kSimBlock);
     const int64_t max_deliver = (words + kSimWaves - 1) / kSimWaves;  // at least one word per wavefront
     q.n_deliver = (has_rec && !pull) ? (int)(max_deliver < 128 ? max_deliver : 128) : 0;
-    const int n_input = (has_inp && !pull_inp) ? 64 : 0;
+    BMTK_REQUIRE((s.in_repeat_ptr == nullptr) == (s.in_repeat_events == nullptr),
+                 "glif3_simulate_fwd: in_repeat_ptr and in_repeat_events go together");
+    // with the pull form of the inputs only the few repeated ids of a step are still delivered as events
+    const bool repeats = pull_inp && s.in_repeat_ptr != nullptr;
+    const int n_input = has_inp ? (!pull_inp ? 64 : (repeats ? 4 : 0)) : 0;
     const size_t table_bytes = (size_t)s.prop_stride * GLIF3_NPROP * sizeof(float);
     q.lds_table = (s.class_id && table_bytes <= (size_t)kLdsTableBytes) ? 1 : 0;
     const size_t lds = q.lds_table ? table_bytes : 0;
@@ -413,6 +420,7 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
             }
         }
         q.n_input = (k > 0 && q.src >= 0) ? n_input : 0;
+        q.repeats = repeats ? 1 : 0;
         const unsigned grid = (unsigned)(q.n_update + q.n_deliver + q.n_input);
         hipLaunchKernelGGL(sim_step_kernel, dim3(grid), dim3(kSimBlock), lds, (hipStream_t)stream, s, q);
     }

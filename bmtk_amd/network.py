@@ -108,7 +108,7 @@ def check_input_events(in_ptr, in_events, n_ids):
     events, ids within 0..n_ids-1 and ascending within every step (the input-weight gradient kernel gives a
     source's run of events one writer and relies on the order).  Returns True when some id occurs more than
     once within a step -- two spikes of one generator inside one resolution step, which NEST delivers both;
-    such lists must stay on the event-list form of the delivery."""
+    the pull form of the inputs then needs the repeats listed apart (Glif3Simulator.set_input_events)."""
     in_ptr = np.asarray(in_ptr)
     in_events = np.asarray(in_events)
     if in_ptr.size < 1 or in_ptr[0] != 0 or np.any(np.diff(in_ptr) < 0) or in_ptr[-1] != in_events.size:

@@ -137,7 +137,7 @@ class Glif3Simulator:
         self.in_ptr = self.in_events = None
         self.in_steps = 0
         self.in_duplicates = False
-        self._inp_form = None  # "pull" or "list" once a run has delivered inputs with the pull tables present
+        self.in_repeat_ptr = self.in_repeat_events = None   # repeated ids of a step, for the pull form of the inputs
         self.step = 0
         self.words = n_words(self.ne)
         # history of spike bits: 2B+3 rows let resident workgroups drift B steps apart, one more lets them look
@@ -241,9 +241,10 @@ class Glif3Simulator:
         (source*batch+trial) must be ascending -- the input-weight gradient kernel
         gives every source's run of events one writer and relies on it.  The same id
         may occur more than once in a step (two spikes of one generator inside one
-        resolution step, which NEST delivers both): every occurrence is delivered;
-        such lists keep the inputs on the event-list form of the delivery, because
-        the bit rows of the pull form can hold an id only once per step."""
+        resolution step, which NEST delivers both): every occurrence is delivered.
+        The pull form of the inputs turns a step's events into bits, which hold an id
+        once; the second and later occurrences are then listed apart
+        (``in_repeat_ptr`` / ``in_repeat_events``) and delivered as events on top."""
         if self.inp is None:
             raise ValueError("no input synapse table")
         if torch.is_tensor(in_ptr):
@@ -252,27 +253,33 @@ class Glif3Simulator:
                 ok = ok and bool((in_events.min() >= 0) & (in_events.max() < self.n_inputs * self.batch))
             if not ok or in_ptr.dtype != torch.int64 or in_events.dtype != torch.int32:
                 raise ValueError("device input event lists are inconsistent")
-            dup = False
-            if in_events.numel() > 1:
-                step_start = torch.zeros(in_events.numel() + 1, dtype=torch.bool, device=in_events.device)
-                step_start[in_ptr] = True                      # an event that opens a step may be smaller than the last
-                d = in_events[1:] - in_events[:-1]
-                inside = ~step_start[1:-1]
-                if bool(((d < 0) & inside).any()):
-                    raise ValueError("input events must be ascending within every step")
-                dup = bool(((d == 0) & inside).any())
-            self.in_ptr = in_ptr.contiguous()
-            self.in_events = in_events.contiguous() if in_events.numel() else in_events.new_zeros(1)
-            self.in_steps = in_ptr.numel() - 1
-            self.in_duplicates = dup
-            return
-        in_ptr = np.ascontiguousarray(in_ptr, np.int64)
-        in_events = np.ascontiguousarray(in_events, np.int32)
-        dup = net.check_input_events(in_ptr, in_events, self.n_inputs * self.batch)
-        self.in_ptr = torch.as_tensor(in_ptr, device=self.dev)
-        self.in_events = torch.as_tensor(in_events if in_events.size else np.zeros(1, np.int32), device=self.dev)
-        self.in_steps = in_ptr.size - 1
-        self.in_duplicates = dup
+            in_ptr, in_events = in_ptr.contiguous(), in_events.contiguous()
+        else:
+            in_ptr = np.ascontiguousarray(in_ptr, np.int64)
+            in_events = np.ascontiguousarray(in_events, np.int32)
+            net.check_input_events(in_ptr, in_events, self.n_inputs * self.batch)
+            in_ptr = torch.as_tensor(in_ptr, device=self.dev)
+            in_events = torch.as_tensor(in_events, device=self.dev)
+        repeat = None
+        if in_events.numel() > 1:
+            step_start = torch.zeros(in_events.numel() + 1, dtype=torch.bool, device=in_events.device)
+            step_start[in_ptr] = True                      # an event that opens a step may be smaller than the last
+            d = in_events[1:] - in_events[:-1]
+            inside = ~step_start[1:-1]
+            if bool(((d < 0) & inside).any()):
+                raise ValueError("input events must be ascending within every step")
+            repeat = (d == 0) & inside                     # event k+1 repeats event k of the same step
+            if not bool(repeat.any()):
+                repeat = None
+        self.in_ptr = in_ptr
+        self.in_events = in_events if in_events.numel() else in_events.new_zeros(1)
+        self.in_steps = in_ptr.numel() - 1
+        self.in_duplicates = repeat is not None
+        self.in_repeat_ptr = self.in_repeat_events = None
+        if repeat is not None and self.pull_inp_table is not None:
+            where = repeat.nonzero().flatten() + 1         # positions of the second and later occurrences
+            self.in_repeat_events = in_events[where].contiguous()
+            self.in_repeat_ptr = torch.searchsorted(where, in_ptr).to(torch.int64).contiguous()
 
     def _struct(self, bits=None, record=None):
         s = _lib.Glif3Sim()
@@ -295,17 +302,12 @@ class Glif3Simulator:
         if self.pull_table is not None:
             s.pull_indptr, s.pull_packed = _p(self.pull_table.indptr), _p(self.pull_table.packed())
             s.pull_syn, s.pull_work = _p(self.pull_syn), _p(self.pull_work)
-            # the form the inputs take is fixed by the first run: arrivals still ahead live in the ring (event
-            # lists) or in the input-bit history (pull form), and a later run must find them where they are
-            if self.pull_inp_table is not None and self.in_ptr is not None and self._inp_form is None:
-                self._inp_form = "list" if self.in_duplicates else "pull"
-            if self._inp_form == "pull" and self.in_duplicates:
-                raise ValueError("input events repeat an id within a step, which the pull form of the inputs this "
-                                 "simulator has been running with cannot hold; build the simulator anew")
-            if self._inp_form == "pull":
+            if self.pull_inp_table is not None and self.in_ptr is not None:
                 s.pull_inp_indptr, s.pull_inp_packed = _p(self.pull_inp_table.indptr), _p(self.pull_inp_table.packed())
                 s.pull_inp_syn, s.pull_inp_work = _p(self.pull_inp_syn), _p(self.pull_inp_work)
                 s.in_hist, s.in_hist_stride = _p(self.in_hist), self.in_hist_stride
+                if self.in_repeat_ptr is not None:
+                    s.in_repeat_ptr, s.in_repeat_events = _p(self.in_repeat_ptr), _p(self.in_repeat_events)
         if self.res_span:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
             s.res_spin_limit = int(self.spin_limit)

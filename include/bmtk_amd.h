@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 13
+#define BMTK_AMD_ABI_VERSION 14
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -213,8 +213,9 @@ typedef struct bmtk_glif3_sim {
     const int32_t *in_events;    /* element ids source*batch+trial, emitted in that step; ascending within a step
                                   * (the input-weight gradient relies on it).  An id may repeat within a step (two
                                   * spikes of one source inside one resolution step): every occurrence is
-                                  * delivered, except by the pull form of the inputs (pull_inp_* below), whose
-                                  * bit rows hold an id once per step -- do not combine the two. */
+                                  * delivered.  The pull form of the inputs (pull_inp_* below) turns a step's
+                                  * events into bits, which hold an id once: with it, the second and later
+                                  * occurrences must also be listed in in_repeat_ptr / in_repeat_events. */
     const int32_t *inp_indptr, *inp_indices;
     const float *inp_weights;
     const uint8_t *inp_delays, *inp_receptors;
@@ -276,6 +277,12 @@ typedef struct bmtk_glif3_sim {
     void *pull_inp_work;                 /* bmtk_csr_propagate_pull_workspace_bytes(ring_slots, n_inputs) bytes */
     uint64_t *in_hist;                   /* [ring_slots][in_hist_stride], zeroed before the first run */
     int64_t in_hist_stride;              /* >= ceil(n_inputs*batch/64) + 1 */
+    /* With the pull form of the inputs only (ignored otherwise; both NULL when no id repeats within a step):
+     * per-step lists, laid out like in_ptr / in_events, of the second and later occurrences of an id within a
+     * step.  The bit rows deliver every id of a step once; these few are delivered on top as events, into the
+     * ring. */
+    const int64_t *in_repeat_ptr;        /* [total steps + 1] */
+    const int32_t *in_repeat_events;
     /* outputs */
     uint64_t *spike_bits;        /* [n_steps][words] spike bits per step, words = ceil(ne/64); or NULL.
                                   * Row k belongs to step step0+k of the call that wrote it. */

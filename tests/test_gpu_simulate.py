@@ -424,8 +424,9 @@ def _with_duplicate_events(cfg, rng, batch):
 @pytest.mark.parametrize("batch,resident", [(1, False), (1, True), (8, False)])
 def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     """Two spikes of one generator inside one resolution step are two deliveries.  Every driver must count them:
-    the launch-per-step driver, the resident one, and the batched driver whose pull form of the inputs (bit rows:
-    one bit per id and step) steps aside for such lists.  Exact weights: bit-identical to the fp32 oracle."""
+    the launch-per-step driver, the resident one, and the batched driver, whose pull form of the inputs (bit rows:
+    one bit per id and step) delivers the second and later occurrences as events on top.  Exact weights:
+    bit-identical to the fp32 oracle."""
     cfg = synthetic.small_glif3_network(n=700, n_in=300, steps=300, seed=14, in_w_scale=3.0, in_fanout=100,
                                         in_rate=30.0, p_conn=0.05, w_scale=1.5, batch=batch)
     cfg["rec_src"] = _integer_weights(cfg["rec_src"])
@@ -442,7 +443,9 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     a, b = sim.run(120), sim.run(180)
     sim.check()
     if batch >= 8:
-        assert sim.pull_table is not None and sim.pull_inp_table is not None and sim._inp_form == "list"
+        assert sim.pull_table is not None and sim.pull_inp_table is not None
+        n_rep = in_events.size - sum(np.unique(in_events[in_ptr[t]:in_ptr[t + 1]]).size for t in range(in_ptr.size - 1))
+        assert sim.in_repeat_events.numel() == n_rep > 0 and int(sim.in_repeat_ptr[-1]) == n_rep
     ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
     np.testing.assert_array_equal(ras, want["raster"])
     got = sim.state.to_numpy()
