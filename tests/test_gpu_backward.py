@@ -81,6 +81,34 @@ def test_weight_gradients_match_autograd(batch, seed, loss_kind, n_blocks):
     assert _rel(got_inp, want["d_inp_w"]) < 1e-4
 
 
+@pytest.mark.parametrize("batch", [1, 8, 32])
+def test_weight_gradients_with_input_ids_repeated_within_a_step(batch):
+    """Two or three spikes of one source inside one step: the forward run delivers every occurrence (batched runs
+    through the bit rows of the pull form plus the repeat lists), and the input-weight gradient counts every
+    occurrence too.  Same autograd reference and tolerance as above."""
+    from test_gpu_simulate import _with_duplicate_events
+    cfg = _net(batch, 21 + batch, n=60, n_in=40, steps=60)
+    n, T, h = cfg["n"], cfg["steps"], cfg["h"]
+    in_ptr, in_events = _with_duplicate_events(cfg, np.random.default_rng(5), batch)
+    assert in_events.size > 1.15 * cfg["in_events"].size
+    prop = orc.precompute(cfg["par"], h)
+    sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                         resident=False)
+    sim.set_input_events(in_ptr, in_events)
+    assert sim.in_duplicates and (batch < 8 or sim.in_repeat_ptr is not None)
+    fwd = sim.run(T, save_state=True)
+    ras = sim.raster(fwd["bits"]).cpu().numpy()
+    a = np.random.default_rng(6).normal(size=(T, n * batch))
+    bptt = training.Glif3Bptt(sim, dampening=0.3)
+    bptt.backward(fwd, dl_dz=torch.as_tensor(a.astype(np.float32), device="cuda"))
+    want = adj.simulate_with_grad(prop, h, T, n, batch, cfg["L"], cfg["rec_src"], cfg["inp_src"], in_ptr, in_events,
+                                  lambda z: (z * torch.as_tensor(a)).sum(), dampening=0.3)
+    np.testing.assert_array_equal(ras, want["raster"])
+    assert ras.sum() > 30 * batch
+    assert _rel(bptt.d_rec_w.cpu().numpy(), want["d_rec_w"]) < 1e-4
+    assert _rel(bptt.d_inp_w.cpu().numpy(), want["d_inp_w"]) < 1e-4
+
+
 def test_chunked_backward_equals_one_call():
     cfg = _net(2, 7)
     n, T, h = cfg["n"], cfg["steps"], cfg["h"]
