@@ -269,3 +269,39 @@ def test_v1_scale_forward_run_against_both_oracles():
         del want
     assert agree[np.float32] >= 0.99999, agree
     assert agree[np.float64] >= 0.999, agree
+
+
+def test_training_size_forward_run_is_bit_identical_to_the_oracle():
+    """The forward pass of the training configuration at its own size -- 51,978 neurons x batch 32, 52 M recurrent
+    and 8 M input synapses, 17,400 Poisson inputs at 5 Hz, per-step record on -- through the batched driver (pull
+    form for recurrent and input synapses, repeat lists for ids that occur twice in a step).  Quarter-pA weights:
+    raster, state and the recorded potentials must equal the fp32 oracle's bit for bit."""
+    n, n_in, batch, steps = N52K, 17400, 32, 120
+    rng = np.random.default_rng(4)
+    par = synthetic.random_cells(rng, n)
+    _, by_src, _ = synthetic.device_network(n, 1000, "poisson", seed=2, w_scale=0.2)
+    by_src = (by_src[0], by_src[1], _quarter(by_src[2]), by_src[3], by_src[4])
+    inp = synthetic.device_input_table(n_in, n, 8_000_000, seed=4, w_scale=2.0)
+    inp = (inp[0], inp[1], _quarter(inp[2]), inp[3], inp[4])
+    in_ptr, in_ev = ops.poisson_events(n_in, 5.0, 1.0, steps, batch=batch, seed=5)
+    sim = Glif3Simulator(n, par, 1.0, batch=batch, rec=by_src, inp=inp, resident=False)
+    assert sim.pull_table is not None and sim.pull_inp_table is not None
+    sim.set_input_events(in_ptr, in_ev)
+    assert sim.in_duplicates and sim.in_repeat_events.numel() > 0   # a few ids occur twice within a step
+    a = sim.run(50, save_state=True)
+    b = sim.run(steps - 50, save_state=True)
+    ras = torch.cat([sim.raster(a["bits"]), sim.raster(b["bits"])]).cpu().numpy()
+    rec_h = tuple(t.cpu().numpy() for t in by_src)
+    inp_h = tuple(t.cpu().numpy() for t in inp)
+    prop = orc.precompute(par, 1.0)
+    orc.set_threads(orc.max_threads())
+    st = orc.new_state(n, batch, np.float32)
+    ring = np.zeros((sim.L, 4, n * batch), np.float32)
+    want = orc.simulate(st, prop, 1.0, steps, batch=batch, ring=ring, rec=rec_h, inp=inp_h, in_ptr=in_ptr.cpu().numpy(),
+                        in_events=in_ev.cpu().numpy(), raster=True)
+    assert want["count"] > 100_000
+    np.testing.assert_array_equal(ras, want["raster"])
+    got = sim.state.to_numpy()
+    for k in ("V", "asc", "y1", "y2", "ref"):
+        np.testing.assert_array_equal(got[k], st[k], err_msg=k)
+    np.testing.assert_array_equal(b["saved"]["v"][-1].cpu().numpy(), st["V"])
