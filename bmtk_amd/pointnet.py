@@ -27,6 +27,7 @@ import torch
 
 from . import sonata
 from .simulator import Glif3Simulator
+from .sonata import add_weight_function, synaptic_weight  # noqa: F401  (bmtk.simulator.pointnet's registry calls)
 from .spike_trains import bin_spike_times
 
 

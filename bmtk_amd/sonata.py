@@ -120,6 +120,15 @@ class NodePopulation:
     def type_of(self, node_type_id):
         return self.types.loc[node_type_id]
 
+    def to_dataframe(self):
+        """One row per node, indexed by node id: ``node_type_id``, ``node_id``, the per-node group columns and the
+        type-table columns (what bmtk's ``get_nodes_df`` hands a weight function)."""
+        df = _frame(len(self), self.group_ids, self.group_index, self.groups, self.types, self.node_type_ids,
+                    "node_type_id")
+        df.insert(0, "node_id", self.node_ids)
+        df.insert(0, "node_type_id", self.node_type_ids)
+        return df.set_index(self.node_ids)
+
     def column(self, name):
         """A per-node attribute, from the groups where it is stored per node, else from the type table."""
         out = np.empty(len(self), object)
@@ -135,6 +144,29 @@ class NodePopulation:
         elif not have.all():
             raise KeyError(name)
         return out
+
+
+def _frame(n, group_ids, group_index, groups, types, type_ids, type_key):
+    """Per-item table of a population: the group datasets (a column of several components becomes ``name.0``,
+    ``name.1`` ...; items whose group lacks a column hold NaN / None) joined with the columns of the type table
+    that no group stores, the way bmtk/utils/sonata/group.py:209-243,339-372 builds its dataframes."""
+    cols = {}
+    for gid, datasets in groups.items():
+        sel = group_ids == gid
+        for name, values in datasets.items():
+            values = np.asarray(values)
+            parts = [(name, values)] if values.ndim == 1 else [("{}.{}".format(name, i), values[:, i])
+                                                               for i in range(values.shape[1])]
+            for cname, v in parts:
+                if cname not in cols:
+                    numeric = v.dtype.kind in "fiub"
+                    cols[cname] = np.full(n, np.nan) if numeric else np.full(n, None, object)
+                cols[cname][sel] = v[group_index[sel]]
+    df = pd.DataFrame(cols)
+    type_cols = [c for c in types.columns if c not in cols and c != type_key]
+    for c in type_cols:
+        df[c] = types[c].reindex(type_ids).to_numpy()
+    return df
 
 
 def read_nodes(nodes_file, node_types_file):
@@ -219,6 +251,34 @@ def node_parameter_classes(pop, models_dir, unsupported="raise"):
 # edges
 # ----------------------------------------------------------------------------------------------------------------
 
+def default_weight_fnc(edge_props, source_nodes, target_nodes):
+    """``syn_weight * nsyns`` (bmtk/simulator/pointnet/default_setters/synaptic_weights.py:6-7)."""
+    return np.array(edge_props["syn_weight"] * edge_props["nsyns"])
+
+
+# weight functions by the name an edge type's ``weight_function`` column gives; the three names bmtk registers at
+# import (synaptic_weights.py:10-12) all stand for the default rule
+_WEIGHT_FUNCTIONS = {"default_weight_fnc": default_weight_fnc, "set_syn_weight": default_weight_fnc,
+                     "wmax": default_weight_fnc}
+
+
+def add_weight_function(func, name=None, overwrite=True):
+    """Register ``func(edges_df, source_nodes_df, target_nodes_df) -> weights`` under ``name`` (default: the
+    function's own name), as bmtk's ``add_weight_function`` does (bmtk/simulator/core/pyfunction_cache.py)."""
+    name = name or func.__name__
+    if overwrite or name not in _WEIGHT_FUNCTIONS:
+        _WEIGHT_FUNCTIONS[name] = func
+    return func
+
+
+def synaptic_weight(*args, **kwargs):
+    """Decorator form: ``@synaptic_weight`` or ``@synaptic_weight(name='...')``."""
+    if len(args) == 1 and callable(args[0]) and not kwargs:
+        return add_weight_function(args[0])
+    name = kwargs.get("name", args[0] if args else None)
+    return lambda func: add_weight_function(func, name)
+
+
 class EdgePopulation:
     def __init__(self, name, source_population, target_population, source_node_id, target_node_id, edge_type_id,
                  group_ids, group_index, groups, indices, types):
@@ -236,6 +296,16 @@ class EdgePopulation:
 
     def __len__(self):
         return self.source_node_id.size
+
+    def to_dataframe(self):
+        """One row per edge in file order: ``edge_type_id``, ``source_node_id``, ``target_node_id``, the per-edge
+        group columns and the type-table columns no group stores (bmtk/utils/sonata/group.py:339-372)."""
+        df = _frame(len(self), self.group_ids, self.group_index, self.groups, self.types, self.edge_type_id,
+                    "edge_type_id")
+        df.insert(0, "target_node_id", self.target_node_id)
+        df.insert(0, "source_node_id", self.source_node_id)
+        df.insert(0, "edge_type_id", self.edge_type_id)
+        return df
 
     def per_edge(self, name):
         """Per-edge values of a group dataset (``nsyns``, ``syn_weight``, ``delay``) or None when no group has it;
@@ -272,17 +342,21 @@ class EdgePopulation:
                     raise ValueError("{}: index {} disagrees with the edge list at node {}".format(self.name, index,
                                                                                                    node))
 
-    def to_arrays(self, synaptic_models_dir, dt):
+    def to_arrays(self, synaptic_models_dir, dt, source_nodes=None, target_nodes=None):
         """-> (source ids, target ids, weights f32, delay steps, receptor_type), one entry per edge in file
         order, by the rules of sonata_adaptors.py:268-357: per-edge ``delay``/``syn_weight``/``nsyns`` win over
         the type table, ``nsyns`` defaults to 1, a missing ``syn_weight`` is an error, the synaptic-model file
         supplies ``receptor_type`` (NEST's 1-based port; 0 where the file names none, which ``glif_psc`` rejects),
-        the template must be a static synapse, and a delay below the resolution is a BadDelay."""
+        the template must be a static synapse, and a delay below the resolution is a BadDelay.  An edge type with
+        a ``weight_function`` gets its weights from the function registered under that name
+        (``add_weight_function``), called with the type's edges and their source and target nodes as dataframes
+        (``source_nodes`` / ``target_nodes``: the two ``NodePopulation``s), as sonata_adaptors.py:319-335 does."""
         n = len(self)
         w = np.empty(n, np.float64)
         delay = np.empty(n, np.float64)
         rec = np.empty(n, np.int64)
         nsyns_e, weight_e, delay_e = self.per_edge("nsyns"), self.per_edge("syn_weight"), self.per_edge("delay")
+        frames = None  # (edges, source nodes, target nodes) as dataframes, built when a weight function asks
         for et in np.unique(self.edge_type_id):
             row = self.types.loc[et]
             sel = self.edge_type_id == et
@@ -291,9 +365,9 @@ class EdgePopulation:
                 template = template[5:]
             if template != "static_synapse":
                 raise NotImplementedError("edge type {}: synapse model {!r} is not implemented".format(et, template))
-            if row.get("weight_function") is not None and not pd.isna(row.get("weight_function")):
-                raise NotImplementedError("edge type {}: weight_function {!r} (user Python code) is not "
-                                          "supported".format(et, row.get("weight_function")))
+            weight_function = row.get("weight_function")
+            if weight_function is not None and pd.isna(weight_function):
+                weight_function = None
             dyn = _load_dynamics(row.get("dynamics_params"), synaptic_models_dir)
             extra = set(dyn) - {"receptor_type", "weight", "delay"}
             if extra:
@@ -307,7 +381,27 @@ class EdgePopulation:
                 syn_weight = row["syn_weight"]
             else:
                 syn_weight = None
-            w[sel] = net.edge_weights(nsyns, syn_weight)
+            if weight_function is not None:
+                if weight_function not in _WEIGHT_FUNCTIONS:
+                    raise Exception('Unable to calculate synaptic weight for "{}" edges, missing "weight_function" '
+                                    'attribute value {} function.'.format(self.name, weight_function))
+                if source_nodes is None or target_nodes is None:
+                    raise ValueError("edge type {}: weight_function {!r} needs the source and target node "
+                                     "populations".format(et, weight_function))
+                if frames is None:
+                    frames = (self.to_dataframe(), source_nodes.to_dataframe(), target_nodes.to_dataframe())
+                    if "nsyns" not in frames[0].columns:
+                        frames[0]["nsyns"] = 1
+                edges = frames[0][sel]
+                got = np.asarray(_WEIGHT_FUNCTIONS[weight_function](
+                    edges, frames[1].loc[edges["source_node_id"].values], frames[2].loc[edges["target_node_id"].values]),
+                    np.float64)
+                if got.shape not in ((), (int(sel.sum()),)):
+                    raise ValueError("weight_function {!r} returned {} values for {} edges".format(
+                        weight_function, got.size, int(sel.sum())))
+                w[sel] = got
+            else:
+                w[sel] = net.edge_weights(nsyns, syn_weight)
             if delay_e is not None and not np.isnan(delay_e[sel]).any():
                 delay[sel] = delay_e[sel]
             elif "delay" in row.index and not pd.isna(row["delay"]):
@@ -615,7 +709,8 @@ def load_point_network(config, dt=None, unsupported="raise"):
         for ep in read_edges(entry["edges_file"], entry["edge_types_file"]).values():
             if ep.target_population != pop.name:
                 raise NotImplementedError("edges {} target population {}".format(ep.name, ep.target_population))
-            src, tgt, w, d, r = ep.to_arrays(comp.get("synaptic_models_dir", "."), dt)
+            src, tgt, w, d, r = ep.to_arrays(comp.get("synaptic_models_dir", "."), dt,
+                                             source_nodes=nodes.get(ep.source_population), target_nodes=pop)
             keep = ~silent[tgt]
             if ep.source_population == pop.name:
                 keep &= ~silent[src]

@@ -469,3 +469,63 @@ def test_current_segments_add_up_the_generators():
     segs = [(a, b, cur.tolist()) for a, b, cur in sim._segments()]
     assert segs == [(0, 11, [0, 0, 0, 0]), (11, 21, [10, 10, 0, 0]), (21, 31, [10, 6, -4, 0]),
                     (31, 81, [0, -4, -4, 0]), (81, 100, [0, 0, 0, 0])]
+
+
+def _edges_with_weight_functions(tmp_path):
+    """A copy of the example's recurrent edge types in which type 100 names a built-in weight function and type
+    101 a user-registered one."""
+    entry = _circuit()["networks"]["edges"][0]
+    with open(entry["edge_types_file"]) as fh:
+        head = fh.readline().split()
+        rows = [line.split() for line in fh if line.strip()]
+    fn = {"100": "wmax", "101": "by_distance"}
+    path = tmp_path / "edge_types.csv"
+    with open(path, "w") as fh:
+        fh.write(" ".join(head + ["weight_function"]) + "\n")
+        for r in rows:
+            fh.write(" ".join(r + [fn.get(r[0], "NONE")]) + "\n")
+    return entry, str(path)
+
+
+def test_weight_functions(tmp_path):
+    """`weight_function` of an edge type (sonata_adaptors.py:319-335): bmtk's built-in names give nsyns * syn_weight
+    (default_setters/synaptic_weights.py), a registered function is called with the type's edges and their source
+    and target nodes as dataframes, an unknown name is an error, and types without a function keep the rule."""
+    entry, types_file = _edges_with_weight_functions(tmp_path)
+    nodes_entry = _circuit()["networks"]["nodes"][0]
+    pop = sonata.read_nodes(nodes_entry["nodes_file"], nodes_entry["node_types_file"])["v1"]
+    plain = sonata.read_edges(entry["edges_file"], entry["edge_types_file"])["v1_to_v1"]
+    _, _, w_plain, d_plain, r_plain = plain.to_arrays(os.path.join(G, "synaptic_models"), dt=0.1)
+    ep = sonata.read_edges(entry["edges_file"], types_file)["v1_to_v1"]
+    with pytest.raises(Exception, match="by_distance"):
+        ep.to_arrays(os.path.join(G, "synaptic_models"), dt=0.1, source_nodes=pop, target_nodes=pop)
+    seen = {}
+
+    @sonata.synaptic_weight(name="by_distance")
+    def by_distance(edges, source_nodes, target_nodes):
+        seen["n"] = len(edges)
+        assert len(source_nodes) == len(target_nodes) == len(edges)
+        assert np.array_equal(source_nodes.index.values, edges["source_node_id"].values)
+        assert np.array_equal(target_nodes["node_id"].values, edges["target_node_id"].values)
+        assert set(edges["edge_type_id"]) == {101} and (target_nodes["ei"] == "i").all()
+        gap = np.abs(source_nodes["node_id"].values - target_nodes["node_id"].values)
+        return edges["syn_weight"].values * edges["nsyns"].values / (1.0 + gap)
+    try:
+        with pytest.raises(ValueError, match="node populations"):
+            ep.to_arrays(os.path.join(G, "synaptic_models"), dt=0.1)
+        src, tgt, w, d, r = ep.to_arrays(os.path.join(G, "synaptic_models"), dt=0.1, source_nodes=pop, target_nodes=pop)
+    finally:
+        sonata._WEIGHT_FUNCTIONS.pop("by_distance", None)
+    is101 = ep.edge_type_id == 101
+    assert seen["n"] == int(is101.sum()) > 0
+    assert np.array_equal(w[~is101], w_plain[~is101])            # wmax and the types without a function: the rule
+    want = w_plain[is101].astype(np.float64) / (1.0 + np.abs(src[is101] - tgt[is101]))
+    assert np.allclose(w[is101], want, rtol=1e-6) and not np.array_equal(w[is101], w_plain[is101])
+    assert np.array_equal(d, d_plain) and np.array_equal(r, r_plain)
+    # the dataframes themselves: one row per node / edge, type columns joined in
+    ndf = pop.to_dataframe()
+    assert len(ndf) == len(pop) and {"node_type_id", "node_id", "model_template", "ei"} <= set(ndf.columns)
+    edf = plain.to_dataframe()
+    assert len(edf) == len(plain) and {"edge_type_id", "source_node_id", "target_node_id", "nsyns", "syn_weight",
+                                       "delay"} <= set(edf.columns)
+    assert np.array_equal(edf["nsyns"].values * edf["syn_weight"].values, w_plain.astype(np.float64))
