@@ -317,6 +317,42 @@ class PoissonSpikeGenerator(SpikeTrains):
             self.add_spikes(nid, np.asarray(out), population)
 
 
+class GammaSpikeGenerator(PoissonSpikeGenerator):
+    """Spike trains of a gamma-distributed renewal process with a stationary rate
+    (bmtk/utils/reports/spike_trains/spike_trains.py:254-307): per node, ``round(1.5 * rate * duration)`` intervals
+    are drawn at once from Gamma(shape ``a``, scale 1/(a*rate)) with SciPy on NumPy's global stream, and spikes are
+    kept up to ``tstop``.  ``a`` = 1 gives Poisson statistics."""
+
+    def add(self, node_ids, firing_rate, a, population=None, times=(0.0, 1.0)):
+        from scipy.stats import gamma
+        if isinstance(node_ids, str):
+            from . import h5lite
+            with h5lite.File(node_ids) as h5:
+                node_ids = np.asarray(h5["/nodes/{}/node_id".format(population)][()], np.int64)
+        if np.isscalar(node_ids):
+            node_ids = [node_ids]
+        if not np.isscalar(firing_rate):
+            raise Exception("Firing rate must be stationary for GammaSpikeGenerator")
+        if np.isscalar(times) and times > 0.0:
+            tstart, tstop = 0.0, times
+        else:
+            tstart, tstop = times[0], times[-1]
+            if tstart >= tstop:
+                raise ValueError("Invalid start and stop times.")
+        if firing_rate < 0:
+            raise Exception("Firing rates must not be negative.")
+        if a < 0:
+            raise ValueError("Shape parameter `a` cannot be negative.")
+        for node_id in node_ids:
+            n_draws = int(round((tstop - tstart) * firing_rate * 1.5))
+            intervals = gamma.rvs(a, loc=0, scale=1 / (a * firing_rate), size=n_draws)
+            # the reference adds the intervals one by one starting from tstart: a running sum in that order
+            t = np.cumsum(np.concatenate([[tstart], intervals]))[1:]
+            t = t[:np.argmax(t > tstop)] if np.any(t > tstop) else t
+            if t.size:
+                self.add_spikes([node_id] * t.size, t * self.output_conversion, population=population)
+
+
 def check_spike_times(st):
     """The rule bmtk applies before ``nest.SetStatus(.., {'spike_times': ..})``
     (bmtk/simulator/pointnet/pointnetwork.py:39-61): empty/None trains are

@@ -134,3 +134,37 @@ def test_equals_and_subset_operators(tmp_path):
     assert SpikeTrains.from_sonata(str(tmp_path / "s.h5"), population="V2").populations == ["V2"]
     with pytest.raises(ValueError):
         SpikeTrains.load(str(tmp_path / "s.xyz"))
+
+
+def test_gamma_generator_draws_and_statistics():
+    """GammaSpikeGenerator (spike_trains.py:254-307; the reference holds no vector for it): the trains are exactly
+    the running sums of SciPy's gamma draws on the seeded global stream, node by node, cut at tstop; the interval
+    CV is 1/sqrt(a); a = 1 has Poisson statistics; bad arguments raise as in the reference."""
+    from scipy.stats import gamma
+    from bmtk_amd.spike_trains import GammaSpikeGenerator
+    g = GammaSpikeGenerator(population="p", seed=77)
+    g.add(node_ids=[3, 8], firing_rate=20.0, a=4.0, times=(0.5, 3.0))
+    np.random.seed(77)
+    for node in (3, 8):
+        draws = gamma.rvs(4.0, loc=0, scale=1 / (4.0 * 20.0), size=round(2.5 * 20.0 * 1.5))
+        t, want = 0.5, []
+        for d in draws:
+            t += d
+            if t > 3.0:
+                break
+            want.append(t * 1000.0)
+        np.testing.assert_allclose(g.get_times(node, "p"), want, rtol=0, atol=1e-9)
+    g = GammaSpikeGenerator(population="p", seed=5)
+    g.add(node_ids=range(200), firing_rate=10.0, a=9.0, times=(0.0, 5.0))
+    isi = np.concatenate([np.diff(g.get_times(n, "p")) for n in range(200)])
+    assert abs(isi.mean() - 100.0) < 2.0 and abs(isi.std() / isi.mean() - 1.0 / 3.0) < 0.02
+    g = GammaSpikeGenerator(population="p", seed=6, output_units="s")
+    g.add(node_ids=range(200), firing_rate=10.0, a=1.0, times=4.0)
+    isi = np.concatenate([np.diff(g.get_times(n, "p")) for n in range(200)])
+    assert abs(isi.std() / isi.mean() - 1.0) < 0.05 and g.time_range("p")[1] <= 4.0
+    with pytest.raises(Exception, match="stationary"):
+        g.add(node_ids=[0], firing_rate=[1.0, 2.0], a=2.0)
+    with pytest.raises(ValueError):
+        g.add(node_ids=[0], firing_rate=5.0, a=-1.0)
+    with pytest.raises(ValueError):
+        g.add(node_ids=[0], firing_rate=5.0, a=2.0, times=(2.0, 1.0))
