@@ -532,6 +532,10 @@ __global__ __launch_bounds__(kBlock) void bwd_rec_grad_kernel(bmtk_glif3_bwd a, 
 // Input weights.  The events of a step are ascending in source*batch+trial, so the trials in
 // which one source fired are adjacent: the wavefront that holds the first event of such a run
 // takes the whole run, which makes it the only writer of that source's row -- no atomics.
+#ifndef BWD_INP_GRID
+#define BWD_INP_GRID 1024
+#endif
+constexpr int kInpGradGrid = BWD_INP_GRID;
 __global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, BwdStep q)
 {
     const int batch = a.batch;
@@ -550,16 +554,34 @@ __global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, 
         while (k_end < k1 && (batch == 1 ? a.in_events[k_end] : (int)((uint32_t)a.in_events[k_end] / (uint32_t)batch)) == j)
             ++k_end;
         const int p0 = a.inp_indptr[j], p1 = a.inp_indptr[j + 1];
-        for (int p = p0 + lane_id(); p < p1; p += kWave) {
-            const uint2 sy = rows[p];
-            int slot = slot0 + (int)(sy.x >> 26);
-            slot = slot >= L ? slot - L : slot;
-            const int r = (sy.x >> 24) & 3;
-            const int64_t i = sy.x & 0xFFFFFFu;
-            const float *cell = a.lam_ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch;
-            float acc = 0.0f;
-            for (int64_t kk = k; kk < k_end; ++kk) acc += cell[a.in_events[kk] - j * batch];
-            a.d_inp_w[p] += acc;
+        // four synapses per lane at a time: their records, then their adjoint cells, travel together
+        constexpr int kUnroll = 4;
+        for (int base = p0 + lane_id(); base < p1; base += kUnroll * kWave) {
+            uint2 sy[kUnroll];
+            float old[kUnroll], acc[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int p = base + u * kWave;
+                if (p < p1) {
+                    sy[u] = rows[p];
+                    old[u] = a.d_inp_w[p];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                acc[u] = 0.0f;
+                if (base + u * kWave < p1) {
+                    int slot = slot0 + (int)(sy[u].x >> 26);
+                    slot = slot >= L ? slot - L : slot;
+                    const int r = (sy[u].x >> 24) & 3;
+                    const int64_t i = sy[u].x & 0xFFFFFFu;
+                    const float *cell = a.lam_ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch;
+                    for (int64_t kk = k; kk < k_end; ++kk) acc[u] += cell[a.in_events[kk] - j * batch];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+                if (base + u * kWave < p1) a.d_inp_w[base + u * kWave] = old[u] + acc[u];
         }
     }
 }
@@ -740,7 +762,7 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
         }
         hipLaunchKernelGGL(bwd_state_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q);
         if (a.d_rec_w && !fused) hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
-        if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(256), dim3(kBlock), 0, st, a, q);
+        if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(kInpGradGrid), dim3(kBlock), 0, st, a, q);
     }
     BMTK_CHECK_LAUNCH("glif3_simulate_bwd");
     return BMTK_OK;
