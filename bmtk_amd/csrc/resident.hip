@@ -5,14 +5,17 @@
 // to the last.  Per step a workgroup
 //   1. folds the arrivals of slot t-1 (LDS) into y1 and runs the GLIF3 update
 //      from registers, then publishes its wavefronts' spike ballots;
-//   2. signals the grid barrier of step t;
-//   3. while the barrier fills, pulls the spikes of step t-1: it scans the
-//      ballots every workgroup published before the previous barrier and, for
-//      each neuron that fired, reads ITS OWN segment of that neuron's synapse
-//      row (rows are sorted by target; a per-row offset table gives the
-//      segment bounds) and adds the weights into its LDS ring slice with LDS
-//      atomics; external input events of step t-1 are pulled the same way;
-//   4. waits for the barrier.
+//   2. pulls the spikes of step t-1: it scans the ballots every workgroup
+//      published before the previous barrier and, for each neuron that fired,
+//      reads ITS OWN segment of that neuron's synapse row (rows are sorted by
+//      target; a per-row offset table gives the segment bounds) and adds the
+//      weights into its LDS ring slice with LDS atomics; external input events
+//      of step t-1 are pulled the same way;
+//   3. on the way, once every wavefront's ballot store of step t has been
+//      acknowledged (an explicit wait on the vector memory counter, taken
+//      together with the pull's first loads), signals the grid barrier of
+//      step t, which then fills while the pull runs;
+//   4. waits for the barrier where the spikes behind it are needed.
 // Nothing but spike ballots, segment offsets and the synapses actually used
 // crosses the memory system: no global atomics, no state traffic.
 //
