@@ -37,7 +37,7 @@ class Glif3Sim(C.Structure):
         ("probe_col", c_void_p), ("probe_v", c_void_p), ("probe_stride", c_int64), ("probe_every", c_int32),
         ("_pad1", c_int32),
         ("spike_step", c_void_p), ("spike_elem", c_void_p), ("spike_frac", c_void_p),
-        ("spike_cap", c_int64), ("spike_count", c_void_p),
+        ("spike_cap", c_int64), ("spike_count", c_void_p), ("spike_ways", c_int32), ("_pad2", c_int32),
     ]
 
 
@@ -58,7 +58,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 14  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 15  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -103,6 +103,7 @@ SIGNATURES = {
 
 RES_SYNC_WORDS = (1 + 64 * 8) * 1088  # BMTK_RES_SYNC_WORDS
 COMPACT_NOALLOC_MAX_N = 1 << 24       # BMTK_COMPACT_NOALLOC_MAX_N
+RECORD_COUNT_STRIDE = 16              # BMTK_RECORD_COUNT_STRIDE
 
 
 class LibraryMissing(RuntimeError):

@@ -288,18 +288,24 @@ __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Residen
     return arrival != nullptr && rounds > 0;
 }
 
-// kLate: the run has slack (S > 0), see the loop body.  kLean: no membrane potential probes and no spike list are
-// asked for and the two tables are one (pull_step); their pointers and counters are then out of the loop, which is
-// short of scalar registers (98 spilled in the general form; every use in the loop is a lane read).
-template <bool kLate, bool kLean>
+// kLate: the run has slack (S > 0), see the loop body.  kForm: what the launch asks for beyond the simulation
+// itself.  The loop is short of scalar registers (98 spilled in the general form; every use in the loop is a lane
+// read), so the pointers and counters a launch does not use are taken out of it at compile time:
+//   kFormLean    spike bits only, and the two tables are one (pull_step);
+//   kFormRecord  the same with the spike record (what the PyNEST-shaped front end and the configuration runner
+//                ask for), no membrane potential probes;
+//   kFormAny     everything: probes, record, two tables.
+enum { kFormAny = 0, kFormRecord = 1, kFormLean = 2 };
+template <bool kLate, int kForm>
 __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim s, Resident r)
 {
-    if (kLean) {
+    constexpr bool kUnifiedTables = kForm != kFormAny;
+    if (kForm != kFormAny) {
         s.probe_col = nullptr;
-        s.spike_count = nullptr;
         s.inp_seg = nullptr;
         s.inp_packed = nullptr;
     }
+    if (kForm == kFormLean) s.spike_count = nullptr;
     extern __shared__ float ring_l[];  // [L*4][span], then the active-row list
     __shared__ int go_on;
     __shared__ unsigned scan_l[kResBlock / kWave];
@@ -351,6 +357,9 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
     bool aborted = false;
     int done = 0;  // steps whose update has run
+    // the spike record may be split into several lists, one per group of workgroups
+    const unsigned rec_ways = s.spike_ways > 1 ? (unsigned)s.spike_ways : 1u;
+    const unsigned long long rec_way = blockIdx.x & (rec_ways - 1u), rec_cap = (unsigned long long)s.spike_cap / rec_ways;
     // the input events of the step pulled in step t, u = t-1-B, are in_events[ka, kb); the bound for the
     // next step is fetched a step ahead.  Steps before 0 have no events (in_ptr[0] = 0).
     const int B = r.offset;
@@ -456,18 +465,13 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
                                m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (s.spike_bits) s.spike_bits[k * s.spike_bits_stride + (e >> 6)] = m;
         }
-        if (s.spike_count && m != 0ull) {
-            const int leader = __ffsll((long long)m) - 1;
-            unsigned long long base = 0ull;
-            if (lane == leader) base = atomicAdd(s.spike_count, (unsigned long long)__popcll(m));
-            base = bcast_u64(base, leader);
-            const unsigned long long idx = base + (unsigned long long)lane_prefix(m);
-            if (spike && idx < (unsigned long long)s.spike_cap) {
-                s.spike_step[idx] = (int32_t)t;
-                s.spike_elem[idx] = (int32_t)e;
-                if (s.spike_frac) s.spike_frac[idx] = frac;
-            }
-        }
+        // Spike record: a wavefront with spikes takes its places in the list with ONE atomic, whose answer is a
+        // memory round trip away.  It is only asked for here and looked at after the pull, so that no wavefront
+        // stops for it in the update (which every other wavefront of the workgroup would wait out at the next
+        // barrier).
+        unsigned long long rec_base = 0ull;
+        if (s.spike_count && m != 0ull && lane == __ffsll((long long)m) - 1)
+            rec_base = atomicAdd(s.spike_count + rec_way * BMTK_RECORD_COUNT_STRIDE, (unsigned long long)__popcll(m));
         done = k + 1;
         // With no slack (S = 0) the arrival is signalled early in the pull so that the barrier fills while
         // the pull runs.  With slack nobody is waiting for this step yet: the arrival moves behind the pull,
@@ -503,7 +507,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         //    inside the loop is read by another workgroup before the kernel ends.
         bool arrived = false;
         if (k > 0 && t - 1 - B >= 0 && mine > 0)
-            arrived = pull_step<kLean>(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb,
+            arrived = pull_step<kUnifiedTables>(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb,
                                        late ? nullptr : my_counter);
         if (!late && !arrived) {
             wait_vector_memory();
@@ -513,6 +517,15 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         ka = kb;
         kb = ((int64_t)__builtin_amdgcn_readfirstlane((int)(kn_lanes >> 32)) << 32) |
              (int64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)kn_lanes);
+        if (s.spike_count && m != 0ull) {  // the places asked for above: the answer has long arrived
+            unsigned long long idx = bcast_u64(rec_base, __ffsll((long long)m) - 1) + (unsigned long long)lane_prefix(m);
+            if (spike && idx < rec_cap) {
+                idx += rec_way * rec_cap;  // this workgroup's list
+                s.spike_step[idx] = (int32_t)t;
+                s.spike_elem[idx] = (int32_t)e;
+                if (s.spike_frac) s.spike_frac[idx] = frac;
+            }
+        }
         if (late) {
             // every wavefront's ballot store has been acknowledged before the workgroup meets and arrives
             wait_vector_memory();
@@ -550,7 +563,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         // closing: spikes and inputs of the last step (less the delay offset), then fold the last slot
         const int64_t tl = r.step0 + done - 1;
         if (tl - B >= 0 && mine > 0)
-            pull_step<kLean>(s, r, g, wrap(tl - B, r.hist), wrap(tl, L), ring_l, act, scan_l, e0, words, ka, kb);
+            pull_step<kUnifiedTables>(s, r, g, wrap(tl - B, r.hist), wrap(tl, L), ring_l, act, scan_l, e0, words, ka, kb);
         __syncthreads();
         if (own) {
             float *prev = ring_l + (int)(tl % L) * GLIF3_NREC * span + tid;
@@ -624,18 +637,21 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
     slack = slack < kMaxSlack ? slack : kMaxSlack;
     Resident r{step0, n_steps, s.res_span, s.res_groups, s.delay_offset, hist, slack, slack / 2 + 1};
     const size_t lds = (size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) + kActCap * sizeof(int);
-    // the lean form: nothing asked for beyond spike bits, and one table for recurrent and input rows
+    // one table for recurrent and input rows lets the kernel drop the second set of pointers
     const bool has_inputs = s.in_ptr != nullptr;
     const int64_t rows = s.n_neurons + (has_inputs ? s.n_inputs : 0);
     const bool unified = s.rec_seg != nullptr && rows < (1ll << 24) && rows * (s.res_groups + 1) < (1ll << 32) &&
                          (!has_inputs || (s.inp_packed == s.rec_packed &&
                                           s.inp_seg == s.rec_seg + s.n_neurons * (int64_t)(s.res_groups + 1)));
-    const bool lean = unified && s.probe_col == nullptr && s.spike_count == nullptr;
-    const void *kernel =
-        slack > 0 ? (lean ? reinterpret_cast<const void *>(sim_resident_kernel<true, true>)
-                          : reinterpret_cast<const void *>(sim_resident_kernel<true, false>))
-                  : (lean ? reinterpret_cast<const void *>(sim_resident_kernel<false, true>)
-                          : reinterpret_cast<const void *>(sim_resident_kernel<false, false>));
+    const int form = !unified || s.probe_col != nullptr ? kFormAny : (s.spike_count != nullptr ? kFormRecord : kFormLean);
+    const void *const kernels[2][3] = {
+        {reinterpret_cast<const void *>(sim_resident_kernel<false, kFormAny>),
+         reinterpret_cast<const void *>(sim_resident_kernel<false, kFormRecord>),
+         reinterpret_cast<const void *>(sim_resident_kernel<false, kFormLean>)},
+        {reinterpret_cast<const void *>(sim_resident_kernel<true, kFormAny>),
+         reinterpret_cast<const void *>(sim_resident_kernel<true, kFormRecord>),
+         reinterpret_cast<const void *>(sim_resident_kernel<true, kFormLean>)}};
+    const void *kernel = kernels[slack > 0 ? 1 : 0][form];
     hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) {
         set_error("glif3_simulate_fwd: resident mode needs %zu bytes of LDS: %s", lds, hipGetErrorString(err));

@@ -210,10 +210,15 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
         // one counter bump per wavefront, record slots handed out in lane order
         const int leader = __ffsll((long long)m) - 1;
         unsigned long long base = 0ull;
-        if (lane == leader) base = atomicAdd(s.spike_count, (unsigned long long)__popcll(m));
+        // the record may be split into several lists with a counter each (spike_ways)
+        const unsigned ways = s.spike_ways > 1 ? (unsigned)s.spike_ways : 1u;
+        const unsigned long long way = (unsigned)bid & (ways - 1u), way_cap = (unsigned long long)s.spike_cap / ways;
+        if (lane == leader)
+            base = atomicAdd(s.spike_count + way * BMTK_RECORD_COUNT_STRIDE, (unsigned long long)__popcll(m));
         base = bcast_u64(base, leader);
-        const unsigned long long idx = base + (unsigned long long)lane_prefix(m);
-        if (spike && idx < (unsigned long long)s.spike_cap) {
+        unsigned long long idx = base + (unsigned long long)lane_prefix(m);
+        if (spike && idx < way_cap) {
+            idx += way * way_cap;
             s.spike_step[idx] = (int32_t)q.t;
             s.spike_elem[idx] = (int32_t)e;
             if (s.spike_frac) s.spike_frac[idx] = frac;
@@ -325,6 +330,9 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
                  "glif3_simulate_fwd: spike_bits_stride smaller than ceil(ne/64)");
     BMTK_REQUIRE(!s.spike_count || (s.spike_step && s.spike_elem && s.spike_cap > 0),
                  "glif3_simulate_fwd: spike record needs spike_step, spike_elem and a positive spike_cap");
+    BMTK_REQUIRE(s.spike_ways >= 0 && s.spike_ways <= 256 && (s.spike_ways & (s.spike_ways - 1)) == 0 &&
+                     (s.spike_ways <= 1 || !s.spike_count || s.spike_cap % s.spike_ways == 0),
+                 "glif3_simulate_fwd: spike_ways must be 0 or a power of two up to 256 that divides spike_cap");
     BMTK_REQUIRE(step0 >= 0 && n_steps >= 0, "glif3_simulate_fwd: step0 and n_steps must be non-negative");
     const int hist = s.hist_slots ? s.hist_slots : 3;
     BMTK_REQUIRE(s.delay_offset >= 0 && (hist >= s.delay_offset + 3 || (s.pull_packed && s.res_span == 0)),

@@ -491,14 +491,12 @@ def Simulate(t_ms):
                 mm_rows[m][1].append(np.repeat(stamps[keep] * dt, ids.size))
                 mm_rows[m][2].append(v.reshape(-1))
         if want_record:
-            rec = out["record"]
-            sim.check()
-            c = int(rec["count"].item())
-            if c > cap:
+            rec = sim.collect_record(out["record"])
+            if rec["overflow"]:
                 raise NESTError("more than {} spikes in one Simulate call; simulate in shorter pieces".format(cap))
-            st = rec["step"][:c].cpu().numpy().astype(np.float64)
-            fr = rec["frac"][:c].cpu().numpy().astype(np.float64)
-            el = rec["elem"][:c].cpu().numpy()
+            st = rec["step"].cpu().numpy().astype(np.float64)
+            fr = rec["frac"].cpu().numpy().astype(np.float64)
+            el = rec["elem"].cpu().numpy()
             order = np.lexsort((el, st + fr))
             # NEST stamps a spike at the end of its step and records stamp - offset, i.e. the
             # interpolated threshold crossing (step + fraction) * resolution

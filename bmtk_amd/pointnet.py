@@ -294,13 +294,12 @@ class PointSimulator:
                         cols = np.searchsorted(probed, rep["node_ids"])
                         rep["rows"].append((stamps[keep] * self.dt,
                                             sampled[keep][:, cols] + e_l[rep["node_ids"]][None, :]))
-            r = out["record"]
-            c = int(r["count"].item())
-            if c > cap:
-                raise RuntimeError("spike record overflow: {} spikes, room for {}".format(c, cap))
-            steps.append(r["step"][:c].cpu().numpy().astype(np.int64))
-            elems.append(r["elem"][:c].cpu().numpy().astype(np.int64))
-            fracs.append(r["frac"][:c].cpu().numpy().astype(np.float64))
+            r = sim.collect_record(out["record"])
+            if r["overflow"]:
+                raise RuntimeError("spike record overflow: {} spikes, room for {}".format(r["count"], cap))
+            steps.append(r["step"].cpu().numpy().astype(np.int64))
+            elems.append(r["elem"].cpu().numpy().astype(np.int64))
+            fracs.append(r["frac"].cpu().numpy().astype(np.float64))
         self.simulator = sim
         st, el, fr = (np.concatenate(x) for x in (steps, elems, fracs))
         times = (st + fr) * self.dt  # threshold crossing interpolated inside the step, as glif_psc stamps it

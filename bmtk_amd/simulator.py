@@ -19,6 +19,7 @@ PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what 
 RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
 RES_ACT_ENTRIES = 8192          # active-row list of the resident kernel (kActCap of csrc/resident.hip), 4 B each
 RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static LDS (rounded up)
+RECORD_WAYS = 64                # lists a large spike record is split into (bmtk_glif3_sim.spike_ways)
 
 
 def resident_span(ne, batch, ring_slots, n_cu):
@@ -319,6 +320,7 @@ class Glif3Simulator:
         if record is not None:
             s.spike_step, s.spike_elem, s.spike_frac = _p(record["step"]), _p(record["elem"]), _p(record["frac"])
             s.spike_cap, s.spike_count = record["step"].numel(), _p(record["count"])
+            s.spike_ways = record.get("ways", 1)
         return s
 
     def set_probes(self, element_ids, every=1):
@@ -338,10 +340,11 @@ class Glif3Simulator:
         self.probe_ids, self.probe_every = ids, int(every)
         self.probe_col = torch.as_tensor(col, device=self.dev)
 
-    def run(self, n_steps, spike_bits=True, record_cap=0, save_state=False):
+    def run(self, n_steps, spike_bits=True, record_cap=0, save_state=False, record_ways=None):
         """Advance ``n_steps`` steps.  Returns a dict with ``bits`` (int64
         [n_steps, words], spike bits per step) and, when ``record_cap`` > 0,
-        the atomic spike record with crossing fractions; ``save_state`` adds the
+        the atomic spike record with crossing fractions (read it with ``collect_record``: a large record is
+        kept as several lists); ``save_state`` adds the
         per-step record (potentials and flags) the backward pass reads; ``probe``
         holds the potentials asked for with ``set_probes``.  Does not
         synchronise."""
@@ -351,10 +354,25 @@ class Glif3Simulator:
         bits = torch.zeros(n_steps, self.words, dtype=torch.int64, device=self.dev) if spike_bits else None
         record = None
         if record_cap:
+            # A large record is kept as RECORD_WAYS lists with a counter each (``collect_record`` joins them): the
+            # wavefronts of a whole network bumping ONE counter cost the resident kernel 1.5 of 5.5 us per step.
+            # No more lists than workgroups (a list nobody appends to is room lost), each of at least 1024 entries.
+            # Workgroups are dealt out to the lists in turn, so a list may serve one workgroup more than another:
+            # callers size the record with room to spare, as they had to for one list.
+            n_wg = self.res_groups if self.res_span else -(-self.ne // 512)
+            ways = 1
+            while ways * 2 <= min(RECORD_WAYS, n_wg) and record_cap >= ways * 2 * 1024:
+                ways *= 2
+            if record_ways is not None:      # the caller's choice: a power of two up to 256
+                ways = int(record_ways)
+                if ways < 1 or ways > 256 or ways & (ways - 1):
+                    raise ValueError("record_ways must be a power of two in 1..256")
+            record_cap = -(-int(record_cap) // ways) * ways
             record = dict(step=torch.zeros(record_cap, dtype=torch.int32, device=self.dev),
                           elem=torch.zeros(record_cap, dtype=torch.int32, device=self.dev),
                           frac=torch.zeros(record_cap, dtype=torch.float32, device=self.dev),
-                          count=torch.zeros(1, dtype=torch.int64, device=self.dev))
+                          count=torch.zeros(1 if ways == 1 else ways * _lib.RECORD_COUNT_STRIDE, dtype=torch.int64,
+                                            device=self.dev), ways=ways)
         s = self._struct(bits, record)
         saved = None
         if save_state:
@@ -376,6 +394,25 @@ class Glif3Simulator:
         self.step += n_steps
         self._pending_check = bool(self.res_span)
         return dict(bits=bits, record=record, saved=saved, probe=probe)
+
+    def collect_record(self, record):
+        """The spike record of a ``run(..., record_cap=...)`` as one list: dict(step int32[], elem int32[], frac
+        float32[], count int, overflow bool), unordered within a step.  ``count`` is the number of spikes the run
+        produced; ``overflow`` says that some of them found no room (then the lists are incomplete).
+        Synchronises."""
+        self.check()
+        ways = record.get("ways", 1)
+        cap = record["step"].numel()
+        way_cap = cap // ways
+        counts = record["count"][::_lib.RECORD_COUNT_STRIDE][:ways] if ways > 1 else record["count"][:1]
+        stored = torch.clamp(counts, max=way_cap)
+        if ways == 1:
+            keep = slice(0, int(stored[0].item()))
+        else:
+            pos = torch.arange(cap, device=counts.device)
+            keep = (pos % way_cap) < stored[pos // way_cap]
+        return dict(step=record["step"][keep], elem=record["elem"][keep], frac=record["frac"][keep],
+                    count=int(counts.sum().item()), overflow=bool((counts > way_cap).any().item()))
 
     def spikes_from_bits(self, bits, step0=0):
         """Spike bits -> (step int64[], element int64[]) ascending, via the

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 14
+#define BMTK_AMD_ABI_VERSION 15
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -307,7 +307,18 @@ typedef struct bmtk_glif3_sim {
     float *spike_frac;
     int64_t spike_cap;
     unsigned long long *spike_count; /* device counter, keeps counting past spike_cap */
+    /* The record in several lists.  Every wavefront with a spike takes its places in the list with one atomic
+     * on the counter; at V1 scale that is 600 atomics on ONE address per step, which the memory side works off
+     * one after the other (1.5 us of a 5.5 us step).  With spike_ways = W > 1 (a power of two up to 256;
+     * spike_cap a multiple of W) the record is W lists of spike_cap / W entries each, list w in entries
+     * [w * spike_cap / W, (w + 1) * spike_cap / W) of spike_step / spike_elem / spike_frac with its counter in
+     * spike_count[w * BMTK_RECORD_COUNT_STRIDE]; a workgroup appends to list (its number mod W).  A counter keeps
+     * counting past its list's end.  0 or 1: one list, as above. */
+    int32_t spike_ways;
+    int32_t _pad2;
 } bmtk_glif3_sim;
+
+#define BMTK_RECORD_COUNT_STRIDE 16 /* 64-bit words between two counters of a record in several lists */
 
 #define BMTK_F_SPIKE 1       /* the element spiked in this step */
 #define BMTK_F_INTEGRATING 2 /* it was not refractory when the step began */

@@ -86,6 +86,9 @@ def test_argument_validation_needs_no_gpu():
     limit = int(re.search(r"#define BMTK_COMPACT_NOALLOC_MAX_N \(1ll << (\d+)\)",
                           open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()).group(1))
     assert _lib.COMPACT_NOALLOC_MAX_N == 1 << limit
+    stride = int(re.search(r"#define BMTK_RECORD_COUNT_STRIDE (\d+)",
+                           open(os.path.join(ROOT, "include", "bmtk_amd.h")).read()).group(1))
+    assert _lib.RECORD_COUNT_STRIDE == stride
 
 
 def test_ops_refuse_to_run_without_a_gpu():

@@ -465,3 +465,46 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     for form in (lambda x: x, lambda x: torch.as_tensor(x, device="cuda")):
         with pytest.raises(ValueError, match="ascending"):
             dev.set_input_events(form(in_ptr), form(bad))
+
+
+@pytest.mark.parametrize("resident", [False, True])
+def test_spike_record_in_several_lists(resident):
+    """A record large enough to be kept as several lists (one counter per group of workgroups instead of one for
+    the whole network): joined by collect_record it holds exactly the spikes of the raster, with the fractions of
+    the single-list record; a list that runs full is reported."""
+    import torch
+    from bmtk_amd.simulator import RECORD_WAYS
+    cfg = synthetic.small_glif3_network(n=20000, n_in=2000, steps=120, seed=21, in_w_scale=6.0, in_fanout=200,
+                                        in_rate=40.0, p_conn=0.002, w_scale=2.0)
+    cfg["rec_src"] = _integer_weights(cfg["rec_src"])       # exact sums: the runs below are the same run
+    cfg["inp_src"] = _integer_weights(cfg["inp_src"])
+    def run(cap, ways=None):
+        sim = _gpu_sim(cfg, resident=resident)
+        out = sim.run(cfg["steps"], record_cap=cap, record_ways=ways)
+        return sim, out
+    sim, out = run(RECORD_WAYS * 4096)
+    # as many lists as the power of two below the number of workgroups (40 per-step, 312 resident), at most 64
+    assert out["record"]["ways"] == (RECORD_WAYS if resident else 32) and bool(sim.res_span) == resident
+    rec = sim.collect_record(out["record"])
+    ras = sim.raster(out["bits"]).cpu().numpy()
+    assert rec["count"] == int(ras.sum()) > 20000 and not rec["overflow"]
+    got = np.zeros_like(ras)
+    np.add.at(got, (rec["step"].cpu().numpy(), rec["elem"].cpu().numpy()), 1)
+    np.testing.assert_array_equal(got, ras)                       # every spike once, none invented
+    sim1, out1 = run(60000, ways=1)                               # one list: the same spikes and fractions
+    assert out1["record"]["ways"] == 1
+    rec1 = sim1.collect_record(out1["record"])
+    def keyed(r):
+        key = r["step"].cpu().numpy().astype(np.int64) * cfg["n"] + r["elem"].cpu().numpy()
+        order = np.argsort(key)
+        return key[order], r["frac"].cpu().numpy()[order]
+    k, f = keyed(rec)
+    k1, f1 = keyed(rec1)
+    np.testing.assert_array_equal(k, k1)
+    np.testing.assert_array_equal(f, f1)
+    frac = f
+    assert frac.min() >= 0.0 and frac.max() <= 1.0
+    # a record too small for the run: counted in full, reported as incomplete
+    sim2 = _gpu_sim(cfg, resident=resident)
+    small = sim2.collect_record(sim2.run(cfg["steps"], record_cap=2000)["record"])
+    assert small["overflow"] and small["count"] == rec["count"] and small["step"].numel() <= 2000
