@@ -491,17 +491,13 @@ def Simulate(t_ms):
                 mm_rows[m][1].append(np.repeat(stamps[keep] * dt, ids.size))
                 mm_rows[m][2].append(v.reshape(-1))
         if want_record:
-            rec = sim.collect_record(out["record"])
+            # NEST stamps a spike at the end of its step and records stamp - offset, i.e. the
+            # interpolated threshold crossing (step + fraction) * resolution; ordered by time on the device
+            rec = sim.collect_record(out["record"], sort_scale=dt)
             if rec["overflow"]:
                 raise NESTError("more than {} spikes in one Simulate call; simulate in shorter pieces".format(cap))
-            st = rec["step"].cpu().numpy().astype(np.float64)
-            fr = rec["frac"].cpu().numpy().astype(np.float64)
-            el = rec["elem"].cpu().numpy()
-            order = np.lexsort((el, st + fr))
-            # NEST stamps a spike at the end of its step and records stamp - offset, i.e. the
-            # interpolated threshold crossing (step + fraction) * resolution
-            times.append(((st + fr) * dt)[order])
-            senders.append(s["neuron_ids"][el[order]])
+            times.append(rec["time"].cpu().numpy())
+            senders.append(s["neuron_ids"][rec["elem"].cpu().numpy()])
     sim.check()  # also without a recorder: Simulate returns only after the run is known to be valid
     s["steps_done"] = step0 + n_steps
     _S.status["biological_time"] = s["steps_done"] * dt

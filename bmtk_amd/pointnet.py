@@ -270,7 +270,7 @@ class PointSimulator:
             sim.set_probes(probed, every=every)
         if inp is not None:
             sim.set_input_events(*bin_spike_times(self._trains, self.dt, self.n_steps))
-        steps, elems, fracs = [], [], []
+        elems, times = [], []
         from .layout import PAR
         e_l = nw.par[PAR["E_L"]][nw.class_id]
         pieces = []
@@ -294,17 +294,15 @@ class PointSimulator:
                         cols = np.searchsorted(probed, rep["node_ids"])
                         rep["rows"].append((stamps[keep] * self.dt,
                                             sampled[keep][:, cols] + e_l[rep["node_ids"]][None, :]))
-            r = sim.collect_record(out["record"])
+            # threshold crossing interpolated inside the step, as glif_psc stamps it; ordered by time (ties by
+            # node) on the device.  The pieces follow one another in time, so their order is the run's.
+            r = sim.collect_record(out["record"], sort_scale=self.dt)
             if r["overflow"]:
                 raise RuntimeError("spike record overflow: {} spikes, room for {}".format(r["count"], cap))
-            steps.append(r["step"].cpu().numpy().astype(np.int64))
             elems.append(r["elem"].cpu().numpy().astype(np.int64))
-            fracs.append(r["frac"].cpu().numpy().astype(np.float64))
+            times.append(r["time"].cpu().numpy())
         self.simulator = sim
-        st, el, fr = (np.concatenate(x) for x in (steps, elems, fracs))
-        times = (st + fr) * self.dt  # threshold crossing interpolated inside the step, as glif_psc stamps it
-        order = np.lexsort((el, times))
-        self.spikes = {nw.population: (el[order], times[order])}
+        self.spikes = {nw.population: (np.concatenate(elems), np.concatenate(times))}
         self._write_outputs()
         return self.spikes
 

@@ -395,10 +395,13 @@ class Glif3Simulator:
         self._pending_check = bool(self.res_span)
         return dict(bits=bits, record=record, saved=saved, probe=probe)
 
-    def collect_record(self, record):
+    def collect_record(self, record, sort_scale=None):
         """The spike record of a ``run(..., record_cap=...)`` as one list: dict(step int32[], elem int32[], frac
         float32[], count int, overflow bool), unordered within a step.  ``count`` is the number of spikes the run
         produced; ``overflow`` says that some of them found no room (then the lists are incomplete).
+        With ``sort_scale`` (the resolution in ms) the list comes back ordered by spike time
+        (step + frac) * sort_scale, ties by element -- sorted on the device, where two million spikes take
+        milliseconds instead of the second a host sort takes -- and ``time`` (float64, ms) is added.
         Synchronises."""
         self.check()
         ways = record.get("ways", 1)
@@ -411,8 +414,14 @@ class Glif3Simulator:
         else:
             pos = torch.arange(cap, device=counts.device)
             keep = (pos % way_cap) < stored[pos // way_cap]
-        return dict(step=record["step"][keep], elem=record["elem"][keep], frac=record["frac"][keep],
-                    count=int(counts.sum().item()), overflow=bool((counts > way_cap).any().item()))
+        out = dict(step=record["step"][keep], elem=record["elem"][keep], frac=record["frac"][keep],
+                   count=int(counts.sum().item()), overflow=bool((counts > way_cap).any().item()))
+        if sort_scale is not None:
+            t = (out["step"].to(torch.float64) + out["frac"].to(torch.float64)) * float(sort_scale)
+            by_elem = torch.argsort(out["elem"], stable=True)
+            order = by_elem[torch.argsort(t[by_elem], stable=True)]
+            out.update(step=out["step"][order], elem=out["elem"][order], frac=out["frac"][order], time=t[order])
+        return out
 
     def spikes_from_bits(self, bits, step0=0):
         """Spike bits -> (step int64[], element int64[]) ascending, via the

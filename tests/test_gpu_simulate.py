@@ -491,6 +491,13 @@ def test_spike_record_in_several_lists(resident):
     got = np.zeros_like(ras)
     np.add.at(got, (rec["step"].cpu().numpy(), rec["elem"].cpu().numpy()), 1)
     np.testing.assert_array_equal(got, ras)                       # every spike once, none invented
+    # ordered on the device: by time (step + fraction) * resolution, ties by element, as numpy's lexsort orders them
+    srt = sim.collect_record(out["record"], sort_scale=0.1)
+    st, fr, el = (rec[k].cpu().numpy() for k in ("step", "frac", "elem"))
+    t = (st.astype(np.float64) + fr.astype(np.float64)) * 0.1
+    order = np.lexsort((el, t))
+    np.testing.assert_array_equal(srt["time"].cpu().numpy(), t[order])
+    np.testing.assert_array_equal(srt["elem"].cpu().numpy(), el[order])
     sim1, out1 = run(60000, ways=1)                               # one list: the same spikes and fractions
     assert out1["record"]["ways"] == 1
     rec1 = sim1.collect_record(out1["record"])
