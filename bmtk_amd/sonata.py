@@ -465,6 +465,12 @@ def read_edges(edges_file, edge_types_file):
 def _sorted(node_ids, timestamps, sort_order):
     node_ids, timestamps = np.asarray(node_ids), np.asarray(timestamps, np.float64)
     if sort_order == "by_time":
+        # a simulation hands its spikes over in this order already; seeing that takes a hundredth of the sort
+        if timestamps.size < 2:
+            return node_ids, timestamps
+        dt = np.diff(timestamps)
+        if not (dt < 0).any() and not ((dt == 0) & (np.diff(node_ids) < 0)).any():
+            return node_ids, timestamps
         order = np.lexsort((node_ids, timestamps))  # time first, node id breaks ties (spike_trains_api to_dataframe)
     elif sort_order == "by_id":
         order = np.lexsort((timestamps, node_ids))
