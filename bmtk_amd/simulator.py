@@ -408,14 +408,15 @@ class Glif3Simulator:
         cap = record["step"].numel()
         way_cap = cap // ways
         counts = record["count"][::_lib.RECORD_COUNT_STRIDE][:ways] if ways > 1 else record["count"][:1]
-        stored = torch.clamp(counts, max=way_cap)
+        counts = counts.cpu()                                  # the one synchronisation
+        stored = torch.clamp(counts, max=way_cap).tolist()
         if ways == 1:
-            keep = slice(0, int(stored[0].item()))
-        else:
-            pos = torch.arange(cap, device=counts.device)
-            keep = (pos % way_cap) < stored[pos // way_cap]
+            keep = slice(0, stored[0])
+        else:                                                  # the filled part of every list, one after the other
+            dev = record["step"].device
+            keep = torch.cat([torch.arange(w * way_cap, w * way_cap + c, device=dev) for w, c in enumerate(stored)])
         out = dict(step=record["step"][keep], elem=record["elem"][keep], frac=record["frac"][keep],
-                   count=int(counts.sum().item()), overflow=bool((counts > way_cap).any().item()))
+                   count=int(counts.sum()), overflow=bool((counts > way_cap).any()))
         if sort_scale is not None:
             t = (out["step"].to(torch.float64) + out["frac"].to(torch.float64)) * float(sort_scale)
             by_elem = torch.argsort(out["elem"], stable=True)
