@@ -628,6 +628,7 @@ __global__ __launch_bounds__(kBlock) void segment_offsets_kernel(int64_t n_rows,
 
 int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream)
 {
+    if (s.res_groups == 1) return simulate_resident_solo(s, step0, n_steps, stream);  // the whole network in one workgroup
     if (n_steps >= (1ll << 31)) {
         set_error("glif3_simulate_fwd: a resident call covers fewer than 2^31 steps");
         return BMTK_E_ARG;

@@ -8,9 +8,14 @@ namespace bmtk {
 constexpr int kActCap = 8192;                                   // active-row list of the resident kernel (entries)
 constexpr size_t kResLdsBytes = 160u * 1024u;                   // LDS of one gfx950 compute unit
 constexpr size_t kResLdsExtra = kActCap * sizeof(int) + 256u;   // the list plus the kernel's static LDS (rounded up)
+constexpr size_t kSoloLdsExtra = 1024u * sizeof(int) + 512u;    // the same for the single-workgroup form
 
 // Whole run as one cooperative launch with state in registers and the ring in
 // LDS (resident.hip).  Arguments have been validated by the caller.
 int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream);
+
+// The same for a network that fits ONE workgroup (res_groups == 1): no grid barrier, ballots handed over in LDS,
+// whole synapse rows walked by a wavefront (resident_solo.hip).
+int simulate_resident_solo(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream);
 
 }  // namespace bmtk

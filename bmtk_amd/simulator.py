@@ -19,17 +19,24 @@ PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what 
 RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
 RES_ACT_ENTRIES = 8192          # active-row list of the resident kernel (kActCap of csrc/resident.hip), 4 B each
 RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static LDS (rounded up)
+SOLO_LDS_EXTRA = 1024 * 4 + 512 # the single-workgroup form: a list of 1024 fired neurons plus its static LDS
 RECORD_WAYS = 64                # lists a large spike record is split into (bmtk_glif3_sim.spike_ways)
 
 
-def resident_span(ne, batch, ring_slots, n_cu):
+def resident_span(ne, batch, ring_slots, n_cu, single=True):
     """Elements per workgroup of the resident kernel for a network of ``ne`` elements on ``n_cu`` compute
     units, or 0 when the network does not fit: batch 1, one workgroup per compute unit (rounded down to a
     multiple of 8), at most 1024 elements each, and ring slice + active-row list + static LDS within the
-    compute unit's LDS.  ``bmtk_glif3_simulate_fwd`` applies the same bound."""
+    compute unit's LDS.  ``bmtk_glif3_simulate_fwd`` applies the same bound.  A network of up to 1024 elements
+    goes to ONE workgroup when its whole ring fits (``single``): the library then runs the form without a grid
+    barrier."""
     cus = n_cu - n_cu % 8
     if batch != 1 or cus <= 0 or ne <= 0:
         return 0
+    if single and ne <= 1024:
+        whole = -(-ne // 64) * 64
+        if ring_slots * NREC * whole * 4 + SOLO_LDS_EXTRA <= RES_LDS_BYTES:
+            return whole
     span = -(-(-(-ne // cus)) // 64) * 64
     if span > 1024 or ring_slots * NREC * span * 4 + RES_LDS_EXTRA > RES_LDS_BYTES:
         return 0
@@ -48,6 +55,9 @@ class Glif3Simulator:
                 LDS (the resident kernel) whenever the network fits it -- batch 1, at most 1024 elements per
                 compute unit, ring slice within LDS; True: insist on it (ValueError otherwise); False: one launch
                 per step, which takes any batch and size
+    single_workgroup  resident mode: a network of up to 1024 elements whose whole ring fits LDS runs in ONE
+                workgroup, without a grid barrier (about 1 us per step instead of 3); False keeps such a network
+                on the many-workgroup form
     pull        launch-per-step mode only: sum the recurrent arrivals of a step in one pass over a target-major
                 copy of the table from the spike-bit history, instead of pushing them into the ring with global
                 atomics as spikes occur -- the faster form for batched runs.  "auto": batch >= 8 (and delay_offset
@@ -63,7 +73,7 @@ class Glif3Simulator:
 
     def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
                  asc_init=None, u_init=None, i_ext=None, device=None, resident="auto", delay_offset="auto",
-                 pull="auto"):
+                 pull="auto", single_workgroup=True):
         self.lib = _lib.load()
         self.dev = device or _dev()
         self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
@@ -156,6 +166,7 @@ class Glif3Simulator:
         self.probe_ids = self.probe_col = None
         self.probe_every = 1
         self.spin_limit = 0  # resident mode: polls of the grid barrier before giving up (0 = built-in limit)
+        self.single_workgroup = bool(single_workgroup)
         if resident:
             self._setup_resident(required=(resident is True))
         self.pull_table = self.pull_syn = self.pull_work = None
@@ -186,7 +197,7 @@ class Glif3Simulator:
         run; it needs batch 1, at most 1024 elements per compute unit and a ring
         slice that fits in LDS beside the kernel's active-row list."""
         n_cu = torch.cuda.get_device_properties(self.dev).multi_processor_count
-        span = resident_span(self.ne, self.batch, self.L, n_cu)
+        span = resident_span(self.ne, self.batch, self.L, n_cu, single=self.single_workgroup)
         if not span:
             if required:
                 raise ValueError("network does not fit resident mode (batch 1, <= 1024 elements per compute unit, "
@@ -313,7 +324,7 @@ class Glif3Simulator:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
             s.res_spin_limit = int(self.spin_limit)
             s.rec_seg, s.inp_seg = _p(self.rec_seg), _p(self.inp_seg)
-            if self.res_unified is not None and s.inp_packed:
+            if self.res_unified is not None and s.inp_packed and self.res_groups > 1:
                 s.inp_packed = s.rec_packed      # the input offsets count from the start of the joint table
         if bits is not None:
             s.spike_bits, s.spike_bits_stride = _p(bits), bits.shape[1]
@@ -385,10 +396,10 @@ class Glif3Simulator:
         if self.probe_col is not None:
             every = self.probe_every
             first = -(-(self.step + 1) // every) * every - 1  # first step t >= self.step with (t + 1) % every == 0
-            steps = torch.arange(first, self.step + n_steps, every, dtype=torch.int64)
-            probe = dict(v=torch.empty(max(1, steps.numel()), self.probe_ids.size, device=self.dev)[:steps.numel()],
-                         steps=steps)
-            s.probe_col, s.probe_v = _p(self.probe_col), probe["v"].data_ptr()
+            steps = torch.arange(first, max(first, self.step + n_steps), every, dtype=torch.int64)  # may be none
+            room = torch.empty(max(1, steps.numel()), self.probe_ids.size, device=self.dev)  # a call may sample nothing
+            probe = dict(v=room[:steps.numel()], steps=steps)
+            s.probe_col, s.probe_v = _p(self.probe_col), room.data_ptr()
             s.probe_stride, s.probe_every = self.probe_ids.size, every
         _lib.check(self.lib.bmtk_glif3_simulate_fwd(C.byref(s), self.step, n_steps, _stream()))
         self.step += n_steps

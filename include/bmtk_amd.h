@@ -247,6 +247,10 @@ typedef struct bmtk_glif3_sim {
      * the whole run.  rec_seg / inp_seg are bmtk_csr_segment_offsets tables
      * built with the same span over tables whose rows are sorted by target;
      * rec_packed / inp_packed are those same tables packed. */
+    /* A network of up to 1024 elements may be given to ONE workgroup (res_span = n rounded up to a multiple of 64,
+     * res_groups = 1, the whole ring within LDS): the library then runs a form without grid barrier that hands the
+     * spikes of a step over in LDS and walks whole rows of rec_packed / inp_packed through rec_indptr /
+     * inp_indptr (rec_seg / inp_seg are not read); a step costs about a third. */
     int32_t res_span;            /* elements per workgroup: multiple of 64, at most 1024 */
     int32_t res_groups;
     const uint32_t *rec_seg;     /* [neurons][res_groups+1] */

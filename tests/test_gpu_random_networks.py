@@ -58,11 +58,14 @@ def test_every_driver_equals_the_oracle(seed):
     if has_rec and cfg["extra"] == 0:
         drivers.append(dict(resident=False, pull=True))
     if batch == 1:
-        drivers.append(dict(resident=True))
+        drivers.append(dict(resident=True))                           # up to 1024 neurons: the single-workgroup form
+        drivers.append(dict(resident=True, single_workgroup=False))   # the many-workgroup form at the same odd sizes
     for kw in drivers:
         sim = Glif3Simulator(n, cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=rec, inp=inp,
                              i_ext=cfg["i_ext"], **kw)
         assert sim.delay_offset == (cfg["extra"] if (has_rec or has_inp) and cfg["extra"] else 0)
+        if kw.get("resident"):
+            assert (sim.res_groups == 1) == (kw.get("single_workgroup", True) or n <= 64)
         if has_inp:
             sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
         a = sim.run(60)

@@ -27,16 +27,18 @@ def _oracle_run(cfg, dtype, steps=None, batch=1, in_ptr=None, in_events=None):
     return out, st, ring
 
 
-def _gpu_sim(cfg, batch=1, in_ptr=None, in_events=None, resident=False):
+def _gpu_sim(cfg, batch=1, in_ptr=None, in_events=None, resident=False, single_workgroup=True):
+    if resident == "many":       # the many-workgroup form of the resident kernel also where one workgroup would do
+        resident, single_workgroup = True, False
     sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
-                         inp=cfg["inp_src"], ring_slots=cfg["L"], resident=resident)
+                         inp=cfg["inp_src"], ring_slots=cfg["L"], resident=resident, single_workgroup=single_workgroup)
     assert bool(sim.res_span) == bool(resident)
     sim.set_input_events(cfg["in_ptr"] if in_ptr is None else in_ptr,
                          cfg["in_events"] if in_events is None else in_events)
     return sim
 
 
-@pytest.mark.parametrize("resident", [False, True])
+@pytest.mark.parametrize("resident", [False, True, "many"])
 @pytest.mark.parametrize("classes", [None, 11])
 def test_450_neuron_network_raster_and_state(classes, resident):
     """The 450-GLIF3 shape (Erdos-Renyi p=0.1, 1000 Poisson inputs at 10 Hz x 50
@@ -421,7 +423,7 @@ def _with_duplicate_events(cfg, rng, batch):
     return np.asarray(new_ptr, np.int64), np.concatenate(chunks).astype(np.int32)
 
 
-@pytest.mark.parametrize("batch,resident", [(1, False), (1, True), (8, False)])
+@pytest.mark.parametrize("batch,resident", [(1, False), (1, True), (1, "many"), (8, False)])
 def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     """Two spikes of one generator inside one resolution step are two deliveries.  Every driver must count them:
     the launch-per-step driver, the resident one, and the batched driver, whose pull form of the inputs (bit rows:
@@ -436,8 +438,13 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     want, st, _ = _oracle_run(cfg, np.float32, batch=batch, in_ptr=in_ptr, in_events=in_events)
     plain, _, _ = _oracle_run(cfg, np.float32, batch=batch)
     assert want["count"] > 1.05 * plain["count"] > 500 * batch      # the repeats matter
+    if resident == "many":       # 700 neurons on a dozen workgroups instead of one
+        kw = dict(resident=True, single_workgroup=False)
+    else:
+        kw = dict(resident=resident)
     sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
-                         inp=cfg["inp_src"], ring_slots=cfg["L"], resident=resident)
+                         inp=cfg["inp_src"], ring_slots=cfg["L"], **kw)
+    assert sim.res_groups == (0 if not resident else 1 if resident is True else 11)
     sim.set_input_events(in_ptr, in_events)
     assert sim.in_duplicates
     a, b = sim.run(120), sim.run(180)
@@ -453,7 +460,7 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
         np.testing.assert_array_equal(got[k], st[k], err_msg=k)
     # device tensors take the same checks
     dev = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
-                         inp=cfg["inp_src"], ring_slots=cfg["L"], resident=resident)
+                         inp=cfg["inp_src"], ring_slots=cfg["L"], **kw)
     dev.set_input_events(torch.as_tensor(in_ptr, device="cuda"), torch.as_tensor(in_events, device="cuda"))
     assert dev.in_duplicates
     dev.set_input_events(torch.as_tensor(cfg["in_ptr"], device="cuda"), torch.as_tensor(cfg["in_events"], device="cuda"))
@@ -515,3 +522,45 @@ def test_spike_record_in_several_lists(resident):
     sim2 = _gpu_sim(cfg, resident=resident)
     small = sim2.collect_record(sim2.run(cfg["steps"], record_cap=2000)["record"])
     assert small["overflow"] and small["count"] == rec["count"] and small["step"].numel() <= 2000
+
+
+@pytest.mark.parametrize("n,max_delay,extra", [(1000, 4, 0), (333, 6, 0), (1024, 3, 40), (70, 2, 1)])
+def test_single_workgroup_form_equals_the_other_drivers(n, max_delay, extra):
+    """A network of up to 1024 neurons runs in ONE workgroup (no grid barrier, ballots handed over in LDS or, with
+    a delay offset, through the history).  Exact weights: raster, state, ring, membrane probes and spike record
+    equal those of the launch-per-step driver and of the many-workgroup form bit for bit, over three calls."""
+    import torch
+    cfg = synthetic.small_glif3_network(n=n, n_in=200, steps=400, seed=31 + n, in_w_scale=8.0, in_fanout=min(n, 60),
+                                        in_rate=40.0, p_conn=min(0.3, 40.0 / n), w_scale=2.0, max_delay=max_delay)
+    for key in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = _integer_weights(cfg[key])
+        cfg[key] = (indptr, indices, w, d.astype(np.int32) + extra, r)
+    ids = np.unique(np.array([0, n // 2, n - 1]))
+    outs = {}
+    for name, kw in (("step", dict(resident=False)), ("one", dict(resident=True)),
+                     ("many", dict(resident=True, single_workgroup=False))):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], delay_offset=extra, **kw)
+        assert sim.delay_offset == extra and sim.res_groups == {"step": 0, "one": 1}.get(name, sim.res_groups)
+        if name == "many":
+            assert sim.res_groups > 1
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        sim.set_probes(ids, every=3)
+        bits, probes, recs = [], [], []
+        for steps in (1, 149, 250):
+            out = sim.run(steps, record_cap=1 << 17)
+            bits.append(out["bits"])
+            probes.append(out["probe"]["v"])
+            rec = sim.collect_record(out["record"], sort_scale=1.0)
+            assert not rec["overflow"]
+            recs.append(torch.stack([rec["time"], rec["elem"].double()]))
+        sim.check()
+        outs[name] = dict(bits=torch.cat(bits).cpu().numpy(), probe=torch.cat(probes).cpu().numpy(),
+                          rec=torch.cat(recs, dim=1).cpu().numpy(), state=sim.state.to_numpy(),
+                          ring=sim.ring.cpu().numpy())
+    assert int(ops_popcount(torch.as_tensor(outs["step"]["bits"]))) > 2 * n
+    for name in ("one", "many"):
+        for k in ("bits", "probe", "rec", "ring"):
+            np.testing.assert_array_equal(outs[name][k], outs["step"][k], err_msg="%s %s" % (name, k))
+        for k in outs["step"]["state"]:
+            np.testing.assert_array_equal(outs[name]["state"][k], outs["step"]["state"][k], err_msg="%s %s" % (name, k))
