@@ -336,6 +336,49 @@ def bench_bptt(torch, steps=600):
     return entries
 
 
+def bench_front_end(torch, sim, steps):
+    """What a run through the front ends costs (bmtk_amd.nest.Simulate, bmtk_amd.pointnet.PointSimulator.run): the same
+    V1-scale simulation with the spike record on (spike times need the crossing fraction), then the record joined,
+    ordered by spike time on the device and copied to the host.  And the size of the reference's own examples: 450
+    neurons, which one workgroup holds."""
+    import numpy as np
+    from bmtk_amd import synthetic
+    from bmtk_amd.simulator import Glif3Simulator
+    res = {}
+
+    def run():
+        res["out"] = sim.run(steps, spike_bits=False, record_cap=steps * N_V1 // 8)
+
+    run()
+    wall, dev = time_region(torch, run)
+    t0 = time.perf_counter()
+    rec = sim.collect_record(res["out"]["record"], sort_scale=1.0)
+    senders, times = rec["elem"].cpu().numpy(), rec["time"].cpu().numpy()
+    collect = time.perf_counter() - t0
+    alg_step = N_V1 * B_PER_UPDATE_CLASS   # the state update alone; the events ride on top as in the headline
+    out = [{"kernel": "sim_resident_kernel (spike record on) + collect_record",
+            "workload": "V1-scale forward simulation as the front ends run it, %d steps" % steps,
+            "us_per_sim_step": dev / steps * 1e6, "neuron_updates_per_s": N_V1 * steps / wall,
+            "spikes": int(times.size), "record_overflow": bool(rec["overflow"]),
+            "collect_sort_copy_ms": collect * 1e3,
+            "roofline": {"bound": "hbm", "achieved": alg_step * steps / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": alg_step * steps / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                         "what": "state update bytes only (103 B per neuron and step)"}}]
+    cfg = synthetic.small_glif3_network(n=450, n_in=1000, steps=21000, seed=0, in_w_scale=2.0)
+    small = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"])
+    small.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    small.run(1000)
+    wall, dev = time_region(torch, lambda: small.run(20000, spike_bits=False, record_cap=1 << 20))
+    small.check()
+    out.append({"kernel": "sim_solo_kernel (one workgroup, spike record on)",
+                "workload": "450 GLIF3 neurons (configuration 0's network), 20000 steps", "groups": small.res_groups,
+                "us_per_sim_step": dev / 20000 * 1e6, "neuron_updates_per_s": 450 * 20000 / wall,
+                "roofline": {"bound": "hbm", "achieved": 450 * B_PER_UPDATE_PLAIN * 20000 / dev / 1e9, "peak": HBM_PEAK_GBS,
+                             "unit": "GB/s", "frac": 450 * B_PER_UPDATE_PLAIN * 20000 / dev / 1e9 / HBM_PEAK_GBS,
+                             "traffic": None, "what": "latency-bound: a step is a chain of dependent phases"}})
+    return out
+
+
 def cpu_baseline(torch, sim, par, class_id, settled, sample_steps):
     """The NEST-algorithm CPU restatement (fp64, event-driven source-major delivery into per-neuron ring
     buffers, OpenMP) on `sample_steps` steps of the same network, started from the settled state the GPU's
@@ -467,7 +510,7 @@ def main():
         sys.exit("bench.py: --steps and --sim-steps must be positive, --warmup non-negative")
     if K * S * ((N_V1 + 63) // 64) * 8 > 100e9:
         sys.exit("bench.py: --steps x --sim-steps spike bits would exceed 100 GB; use fewer passes")
-    overhead_steps = 3 * (100 + 1100)
+    overhead_steps = 3 * (100 + 1100) + 2 * S      # launch-overhead runs and the front-end entry
     sim, par, class_id = build_v1(torch, SETTLE_MAX_STEPS + (W + K) * S + overhead_steps,
                                   resident=False if args.per_step else "auto")
     # untimed: leave the transient from rest behind, whatever --warmup says
@@ -530,7 +573,8 @@ def main():
     }
     if not args.no_kernels:
         del passes
-        line["kernels"] = sum((groups[g](torch) for g in groups if g in want), [])
+        line["kernels"] = (bench_front_end(torch, sim, S) if resident else []) + \
+            sum((groups[g](torch) for g in groups if g in want), [])
     if args.cpu_steps > 0:
         line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, settled, max(CPU_MIN_STEPS, args.cpu_steps))
     print(json.dumps(line))

@@ -233,7 +233,7 @@ int simulate_resident_solo(const bmtk_glif3_sim &s, int64_t step0, int64_t n_ste
         set_error("glif3_simulate_fwd: the single-workgroup form needs %zu bytes of LDS: %s", lds, hipGetErrorString(err));
         return BMTK_E_LAUNCH;
     }
-    const int threads = s.res_span > 256 ? s.res_span : 256;
+    const int threads = kSoloBlock;  // wavefronts without elements still walk rows: a step's spikes and events in one round
     hipLaunchKernelGGL(sim_solo_kernel, dim3(1), dim3(threads), lds, stream, s, r);
     err = hipGetLastError();
     if (err != hipSuccess) {
