@@ -349,7 +349,7 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
         BMTK_REQUIRE(!has_rec || s.rec_seg, "glif3_simulate_fwd: resident mode needs rec_seg");
         BMTK_REQUIRE(!has_inp || s.inp_seg, "glif3_simulate_fwd: resident mode needs inp_seg");
         BMTK_REQUIRE((size_t)s.ring_slots * GLIF3_NREC * s.res_span * sizeof(float) +
-                             (s.res_groups == 1 ? kSoloLdsExtra : kResLdsExtra) <= kResLdsBytes,
+                             (s.res_groups == 1 ? solo_lds_extra(s.res_span) : kResLdsExtra) <= kResLdsBytes,
                      "glif3_simulate_fwd: ring slice does not fit in LDS beside the active-row list");
         bmtk_glif3_sim r = s;
         if (!has_rec) r.rec_seg = nullptr;

@@ -19,7 +19,10 @@ PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what 
 RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
 RES_ACT_ENTRIES = 8192          # active-row list of the resident kernel (kActCap of csrc/resident.hip), 4 B each
 RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static LDS (rounded up)
-SOLO_LDS_EXTRA = 1024 * 4 + 512 # the single-workgroup form: a list of 1024 fired neurons plus its static LDS
+# the single-workgroup form: per element the spike offsets and probed potentials of two steps (SOLO_LDS_PER_ELEMENT);
+# the row bounds of up to 1024 neurons, two steps' input events and its static LDS (SOLO_LDS_EXTRA)
+SOLO_LDS_PER_ELEMENT = 4 * 4
+SOLO_LDS_EXTRA = 1026 * 4 + 256 * 4 + 1024
 RECORD_WAYS = 64                # lists a large spike record is split into (bmtk_glif3_sim.spike_ways)
 
 
@@ -35,7 +38,7 @@ def resident_span(ne, batch, ring_slots, n_cu, single=True):
         return 0
     if single and ne <= 1024:
         whole = -(-ne // 64) * 64
-        if ring_slots * NREC * whole * 4 + SOLO_LDS_EXTRA <= RES_LDS_BYTES:
+        if (ring_slots * NREC * 4 + SOLO_LDS_PER_ELEMENT) * whole + SOLO_LDS_EXTRA <= RES_LDS_BYTES:
             return whole
     span = -(-(-(-ne // cus)) // 64) * 64
     if span > 1024 or ring_slots * NREC * span * 4 + RES_LDS_EXTRA > RES_LDS_BYTES:

@@ -105,6 +105,6 @@ def test_resident_fit_bound_counts_the_active_row_list():
                 assert L * 4 * span * 4 + RES_LDS_EXTRA <= RES_LDS_BYTES
     assert resident_span(1000, 1, 6, 250, single=False) == 64      # 248 usable compute units
     assert resident_span(1000, 1, 6, 250) == 1024                  # a small network: one workgroup holds all of it
-    assert resident_span(300, 1, 6, 256) == 320 and resident_span(1024, 1, 9, 256) == 1024
-    assert resident_span(1024, 1, 10, 256) == 64                   # its whole ring does not fit: many workgroups
+    assert resident_span(300, 1, 6, 256) == 320 and resident_span(1024, 1, 8, 256) == 1024
+    assert resident_span(1024, 1, 9, 256) == 64                    # its whole ring does not fit: many workgroups
     assert resident_span(1025, 1, 6, 256) == 64
