@@ -8,12 +8,9 @@ namespace bmtk {
 constexpr int kActCap = 8192;                                   // active-row list of the resident kernel (entries)
 constexpr size_t kResLdsBytes = 160u * 1024u;                   // LDS of one gfx950 compute unit
 constexpr size_t kResLdsExtra = kActCap * sizeof(int) + 256u;   // the list plus the kernel's static LDS (rounded up)
-// the single-workgroup form, with span elements: spike offsets and probed potentials of two steps, the row bounds of up
-// to 1024 neurons, two steps' input events, its static LDS (rounded up)
-constexpr size_t solo_lds_extra(int span)
-{
-    return (size_t)span * 4u * sizeof(float) + 1026u * sizeof(int) + 256u * sizeof(int) + 1024u;
-}
+// the single-workgroup form, with span elements: spike offsets and probed potentials of two steps, the items (rows to
+// walk) of two steps, its static LDS (rounded up)
+constexpr size_t solo_lds_extra(int span) { return (size_t)span * 4u * sizeof(float) + 4096u + 1024u; }
 
 // Whole run as one cooperative launch with state in registers and the ring in
 // LDS (resident.hip).  Arguments have been validated by the caller.

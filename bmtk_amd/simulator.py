@@ -20,9 +20,9 @@ RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
 RES_ACT_ENTRIES = 8192          # active-row list of the resident kernel (kActCap of csrc/resident.hip), 4 B each
 RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static LDS (rounded up)
 # the single-workgroup form: per element the spike offsets and probed potentials of two steps (SOLO_LDS_PER_ELEMENT);
-# the row bounds of up to 1024 neurons, two steps' input events and its static LDS (SOLO_LDS_EXTRA)
+# the items (rows to walk) of two steps and its static LDS (SOLO_LDS_EXTRA)
 SOLO_LDS_PER_ELEMENT = 4 * 4
-SOLO_LDS_EXTRA = 1026 * 4 + 256 * 4 + 1024
+SOLO_LDS_EXTRA = 4096 + 1024
 RECORD_WAYS = 64                # lists a large spike record is split into (bmtk_glif3_sim.spike_ways)
 
 
