@@ -374,12 +374,9 @@ __global__ __launch_bounds__(kSoloBlock) void sim_solo_kernel(bmtk_glif3_sim s, 
                     near_l[near_row][wave] = m;
                 }
                 if (spike && s.spike_frac) frac_l[buf * span + tid] = frac;
-                if (sample && probe_col >= 0) {
-                    if (probe_col < span)
-                        probe_l[buf * span + probe_col] = st.V;
-                    else
-                        probe_out[probe_col] = st.V;
-                }
+                if (sample && probe_col >= 0 && probe_col < span) probe_l[buf * span + probe_col] = st.V;
+                asm volatile("" ::: "memory");  // two stores, not one generic store to either place
+                if (sample && probe_col >= span) probe_out[probe_col] = st.V;
             }
             if (kRole == kStoreRole && !kZeroB && B >= kNearSteps) {
                 if (wait_in == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
