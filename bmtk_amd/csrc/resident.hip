@@ -117,20 +117,27 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
                                              int L, int slot0)
 {
     const SegBounds sb = *reinterpret_cast<const SegBounds *>(seg_row + g);
-    const uint32_t lo = sb.lo, hi = sb.hi;
-    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(tab);
+    const uint32_t len = sb.hi - sb.lo;  // the offsets never decrease
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(tab) + sb.lo;
     // An LDS float atomic costs about three clocks per LANE on gfx950 (its lanes are worked off one after the
     // other), an integer compare-and-swap a few clocks per INSTRUCTION.  Where most lanes of a wavefront take
     // part -- the first two synapses of the segments -- the addition is therefore a compare-and-swap loop (a
     // lane repeats only if another thread changed its cell in between, which is rare among 23,000 cells); the
     // thinly populated later ones keep the float atomic.  The sum is the same either way.
     // ring cell of a synapse: the record's upper byte is delay*4 + receptor, so (slot0 + delay) % L * 4 + receptor
-    // = min(u, u - 4L) with u = slot0*4 + that byte (unsigned), times the span, plus the target's place in it
+    // = min(u, u - 4L) with u = slot0*4 + that byte (unsigned), times the span, plus the target's place in it.
+    // Instruction issue is what the pull is short of (every lane walks its own segment, so each addition is a
+    // wavefront instruction for a handful of lanes): the cell's address takes six instructions -- two byte adds, min,
+    // mask, one 24-bit multiply-add, one shift-add onto the slice's origin less e0 -- and a synapse's load a compare
+    // against the segment's length and an immediate offset.
     const unsigned q_lo = (unsigned)slot0 * 4u, q_wrap = q_lo - 4u * (unsigned)L;
+    float *origin = ring_l - e0;
+    unsigned span_v;  // in a vector register once, not before every multiply
+    asm("v_mov_b32 %0, %1" : "=v"(span_v) : "s"(span));
     auto add = [&](const uint2 sy, bool crowded) {
         const unsigned dq = sy.x >> 24;
         const unsigned plane = min(dq + q_lo, dq + q_wrap);
-        float *cell = ring_l + (mul_u24(plane, (unsigned)span) + (sy.x & 0xFFFFFFu) - (unsigned)e0);
+        float *cell = origin + mad_u24(plane, span_v, sy.x & 0xFFFFFFu);
         const float w = __uint_as_float(sy.y);
         if (!crowded) {
             atomicAdd(cell, w);
@@ -150,11 +157,11 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
     uint2 first[kTogether];
 #pragma unroll
     for (int u = 0; u < kTogether; ++u)
-        if (lo + (uint32_t)u < hi) first[u] = rows[lo + (uint32_t)u];
+        if ((uint32_t)u < len) first[u] = rows[u];
 #pragma unroll
     for (int u = 0; u < kTogether; ++u)
-        if (lo + (uint32_t)u < hi) add(first[u], u < 2);
-    for (uint32_t p = lo + (uint32_t)kTogether; p < hi; ++p) add(rows[p], false);
+        if ((uint32_t)u < len) add(first[u], u < 2);
+    for (uint32_t q = (uint32_t)kTogether; q < len; ++q) add(rows[q], false);
 }
 
 constexpr int kScanWords = 4;   // ballot words per thread and round
