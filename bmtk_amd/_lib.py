@@ -27,7 +27,7 @@ class Glif3Sim(C.Structure):
         ("work_bits", c_void_p), ("delay_offset", c_int32), ("hist_slots", c_int32),
         ("delay_bits", c_int32), ("res_spin_limit", C.c_uint32),
         ("res_span", c_int32), ("res_groups", c_int32), ("rec_seg", c_void_p), ("inp_seg", c_void_p),
-        ("res_sync", c_void_p),
+        ("res_sync", c_void_p), ("res_fired", c_void_p),
         ("pull_indptr", c_void_p), ("pull_packed", c_void_p), ("pull_syn", c_void_p), ("pull_work", c_void_p),
         ("pull_inp_indptr", c_void_p), ("pull_inp_packed", c_void_p), ("pull_inp_syn", c_void_p),
         ("pull_inp_work", c_void_p), ("in_hist", c_void_p), ("in_hist_stride", c_int64),
@@ -58,7 +58,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 15  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 16  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -103,7 +103,8 @@ SIGNATURES = {
 
 RES_SYNC_WORDS = (1 + 64 * 8) * 1088  # BMTK_RES_SYNC_WORDS
 COMPACT_NOALLOC_MAX_N = 1 << 24       # BMTK_COMPACT_NOALLOC_MAX_N
-RECORD_COUNT_STRIDE = 16              # BMTK_RECORD_COUNT_STRIDE
+RECORD_COUNT_STRIDE = 16
+RES_FIRED_SLOTS = 16              # BMTK_RES_FIRED_SLOTS
 
 
 class LibraryMissing(RuntimeError):

@@ -121,7 +121,7 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
     const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(tab) + sb.lo;
     // An LDS float atomic costs about three clocks per LANE on gfx950 (its lanes are worked off one after the
     // other), an integer compare-and-swap a few clocks per INSTRUCTION.  Where most lanes of a wavefront take
-    // part -- the first two synapses of the segments -- the addition is therefore a compare-and-swap loop (a
+    // part -- the first synapse of the segments -- the addition is therefore a compare-and-swap loop (a
     // lane repeats only if another thread changed its cell in between, which is rare among 23,000 cells); the
     // thinly populated later ones keep the float atomic.  The sum is the same either way.
     // ring cell of a synapse: the record's upper byte is delay*4 + receptor, so (slot0 + delay) % L * 4 + receptor
@@ -152,15 +152,16 @@ __device__ __forceinline__ void pull_segment(const uint32_t *__restrict__ seg_ro
         }
     };
     // all of a segment's loads go out together: a loop of dependent loads for the few long segments would
-    // hold up the whole wavefront (1 in 25 segments has more than 3 synapses, 1 in 5000 more than 6)
-    constexpr int kTogether = 6;
+    // hold up the whole wavefront (1 in 25 segments has more than 3 synapses, 1 in 5000 more than 6); measured at V1
+    // scale: four together and the compare-and-swap for the first only, 5.35 us per step; six and two, 5.43
+    constexpr int kTogether = 4;
     uint2 first[kTogether];
 #pragma unroll
     for (int u = 0; u < kTogether; ++u)
         if ((uint32_t)u < len) first[u] = rows[u];
 #pragma unroll
     for (int u = 0; u < kTogether; ++u)
-        if ((uint32_t)u < len) add(first[u], u < 2);
+        if ((uint32_t)u < len) add(first[u], u < 1);
     for (uint32_t q = (uint32_t)kTogether; q < len; ++q) add(rows[q], false);
 }
 
@@ -181,7 +182,11 @@ constexpr unsigned kInputTag = 0x80000000u;
 // Returns true when the bump has been made.
 // kUnified: the input rows follow the recurrent rows in ONE table (inp_seg = rec_seg + n_neurons*(n_groups+1), both
 // sets of offsets index rec_packed), so a listed row needs no choice between two tables.
-template <bool kUnified>
+// kLists: the workgroups publish the neurons that fired as short lists (res_fired) and a step is read from those
+// when every list sufficed: two 8-byte loads per thread bring four places of the lists, the occupied ones go
+// straight to the row list -- no ballot words to take apart bit by bit, which is the larger part of the
+// instructions a quiet step costs.
+template <bool kUnified, bool kLists>
 __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Resident &r, int g, int hist_row, int slot0,
                                           float *ring_l, unsigned *act, unsigned *scan_l, int e0, int words,
                                           int64_t k0, int64_t k1, unsigned *arrival = nullptr)
@@ -190,6 +195,67 @@ __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Residen
     const int L = s.ring_slots;
     const int wave = tid / kWave;
     const bool has_rec = s.rec_seg != nullptr;
+    // one thread per listed row pulls this workgroup's segment of it
+    auto pull_listed = [&](unsigned total) {
+        for (unsigned a = tid; a < total; a += kResBlock) {
+            // one code path for both kinds of rows: a wavefront nearly always holds some of each, and a
+            // branch would make it walk the two chains of dependent loads one after the other
+            const unsigned entry = act[a];
+            if (kUnified) {  // rows * (n_groups + 1) stays below 2^32 (checked before the launch)
+                pull_segment(s.rec_seg + mul_u24(entry, (unsigned)(r.n_groups + 1)), g, s.rec_packed, ring_l, r.span,
+                             e0, L, slot0);
+            } else {
+                const int64_t row = entry & ~kInputTag;
+                const bool is_input = (entry & kInputTag) != 0u;
+                const uint32_t *seg = is_input ? s.inp_seg : s.rec_seg;
+                const bmtk_synapse *tab = is_input ? s.inp_packed : s.rec_packed;
+                pull_segment(seg + row * (r.n_groups + 1), g, tab, ring_l, r.span, e0, L, slot0);
+            }
+        }
+    };
+    bool arrived_above = false;
+    if (kLists && s.res_fired && k1 - k0 <= kResBlock) {
+        constexpr unsigned kManyFlag = 1u << 20;  // in a count: some list did not suffice (1024 of them still fit 32 bits)
+        static_assert(kManyFlag > (unsigned)kActCap && 5 * kResBlock <= kActCap, "a step read from the lists always fits the row list");
+        const unsigned long long *lists = reinterpret_cast<const unsigned long long *>(
+            s.res_fired + (int64_t)hist_row * r.n_groups * BMTK_RES_FIRED_SLOTS);
+        unsigned long long w0 = 0ull, w1 = 0ull;  // four places: kResBlock threads cover 256 workgroups' lists
+        if (has_rec && tid < r.n_groups * (BMTK_RES_FIRED_SLOTS / 4)) {
+            w0 = __hip_atomic_load(lists + 2 * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            w1 = __hip_atomic_load(lists + 2 * tid + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        const int64_t ke = k0 + tid;
+        const bool has_event = ke < k1;
+        const unsigned event_row = has_event ? (unsigned)s.in_events[ke] : 0u;
+        const unsigned id[4] = {(unsigned)w0, (unsigned)(w0 >> 32), (unsigned)w1, (unsigned)(w1 >> 32)};
+        unsigned cnt = has_event ? 1u : 0u;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) cnt += id[u] != 0u ? 1u : 0u;
+        if (id[0] == BMTK_RES_FIRED_MANY) cnt = kManyFlag;  // such a list is marked in every place
+        const unsigned inc = wave_inclusive_scan(cnt);
+        if (lane_id() == kWave - 1) scan_l[wave] = inc;
+        if (arrival) wait_vector_memory();  // the loads are back already; this is for the stores of the update
+        __syncthreads();
+        if (arrival && tid == 0) __hip_atomic_fetch_add(arrival, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned part = wave_inclusive_scan(lane_id() < kResBlock / kWave ? scan_l[lane_id()] : 0u);
+        const unsigned total = (unsigned)bcast_i((int)part, kResBlock / kWave - 1);
+        const unsigned base = wave > 0 ? (unsigned)__shfl((int)part, wave - 1, kWave) : 0u;
+        if (total <= (unsigned)kActCap) {  // workgroup-uniform: every list sufficed, and the row list holds them
+            unsigned pos = base + inc - cnt;
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (id[u] != 0u) act[pos++] = id[u] - 1u;
+            if (has_event) act[pos] = kUnified ? event_row + (unsigned)s.n_neurons : event_row | kInputTag;
+            __syncthreads();
+            pull_listed(total);
+            __syncthreads();
+            return arrival != nullptr;
+        }
+        // this step from the ballots (the arrival has been made)
+        __syncthreads();  // scan_l is written again below
+        arrived_above = arrival != nullptr;
+        arrival = nullptr;
+    }
     const unsigned long long *bits =
         reinterpret_cast<const unsigned long long *>(s.work_bits) + (int64_t)hist_row * (words + 1);
     // 32-bit counters wherever the sizes allow: the loop is short of scalar registers
@@ -268,23 +334,7 @@ __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Residen
         }
         __syncthreads();
         PROF_T(p2);
-        if (listed) {
-            for (unsigned a = tid; a < total; a += kResBlock) {
-                // one code path for both kinds of rows: a wavefront nearly always holds some of each, and a
-                // branch would make it walk the two chains of dependent loads one after the other
-                const unsigned entry = act[a];
-                if (kUnified) {  // rows * (n_groups + 1) stays below 2^32 (checked before the launch)
-                    pull_segment(s.rec_seg + mul_u24(entry, (unsigned)(r.n_groups + 1)), g, s.rec_packed, ring_l, r.span,
-                                 e0, L, slot0);
-                } else {
-                    const int64_t row = entry & ~kInputTag;
-                    const bool is_input = (entry & kInputTag) != 0u;
-                    const uint32_t *seg = is_input ? s.inp_seg : s.rec_seg;
-                    const bmtk_synapse *tab = is_input ? s.inp_packed : s.rec_packed;
-                    pull_segment(seg + row * (r.n_groups + 1), g, tab, ring_l, r.span, e0, L, slot0);
-                }
-            }
-        }
+        if (listed) pull_listed(total);
         __syncthreads();
         PROF_T(p3);
         PROF_ADD(4, p0, p1);
@@ -292,7 +342,7 @@ __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Residen
         PROF_ADD(6, p2, p3);
         PROF_BLK(3, p2, p3);
     }
-    return arrival != nullptr && rounds > 0;
+    return arrived_above || (arrival != nullptr && rounds > 0);
 }
 
 // kLate: the run has slack (S > 0), see the loop body.  kForm: what the launch asks for beyond the simulation
@@ -307,6 +357,7 @@ template <bool kLate, int kForm>
 __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim s, Resident r)
 {
     constexpr bool kUnifiedTables = kForm != kFormAny;
+    constexpr bool kLists = !kLate;  // lists of fired neurons beside the ballots (res_fired), see pull_step
     if (kForm != kFormAny) {
         s.probe_col = nullptr;
         s.inp_seg = nullptr;
@@ -316,6 +367,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     extern __shared__ float ring_l[];  // [L*4][span], then the active-row list
     __shared__ int go_on;
     __shared__ unsigned scan_l[kResBlock / kWave];
+    __shared__ unsigned fired_l[BMTK_RES_FIRED_SLOTS];  // this workgroup's list of the step: neuron + 1
+    __shared__ unsigned fired_n;
     const int tid = threadIdx.x;
     const int lane = lane_id();
     // Workgroups are dispatched round-robin over the 8 XCDs (block b runs on XCD
@@ -337,7 +390,10 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     unsigned *arrivals = s.res_sync + kBarrierStride;  // [kBarrierWords] counters, kBarrierStride words apart
     // a run before this one gave up and nobody has looked yet: do nothing, so that the failure is still there to see
     // (one thread looks for the whole workgroup, so that all of its threads take the same way)
-    if (tid == 0) go_on = load_agent(abort_word) == 0u;
+    if (tid == 0) {
+        go_on = load_agent(abort_word) == 0u;
+        fired_n = 0u;
+    }
     __syncthreads();
     if (!go_on) return;
     __syncthreads();  // go_on is written again in the loop
@@ -476,6 +532,10 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         // memory round trip away.  It is only asked for here and looked at after the pull, so that no wavefront
         // stops for it in the update (which every other wavefront of the workgroup would wait out at the next
         // barrier).
+        if (kLists && s.res_fired && m != 0ull && spike) {
+            const unsigned at = atomicAdd(&fired_n, 1u);
+            if (at < BMTK_RES_FIRED_SLOTS) fired_l[at] = (unsigned)e + 1u;
+        }
         unsigned long long rec_base = 0ull;
         if (s.spike_count && m != 0ull && lane == __ffsll((long long)m) - 1)
             rec_base = atomicAdd(s.spike_count + rec_way * BMTK_RECORD_COUNT_STRIDE, (unsigned long long)__popcll(m));
@@ -500,6 +560,15 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
                 aborted = true;
                 break;
             }
+            // the list of this step, complete since the workgroup met: out with it, like the ballots (the arrival
+            // waits for the store), and the count back to zero (it is added to again after the barriers of the pull)
+            if (kLists && s.res_fired && tid < BMTK_RES_FIRED_SLOTS && g < r.n_groups) {  // (the grid is rounded up)
+                const unsigned n = fired_n;
+                const unsigned word = n > BMTK_RES_FIRED_SLOTS ? BMTK_RES_FIRED_MANY : ((unsigned)tid < n ? fired_l[tid] : 0u);
+                __hip_atomic_store(s.res_fired + ((int64_t)row_t * r.n_groups + g) * BMTK_RES_FIRED_SLOTS + tid, word,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (tid == 0) fired_n = 0u;
+            }
         }
         PROF_T(c2);
 #ifdef BMTK_RES_PROFILE
@@ -514,8 +583,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         //    inside the loop is read by another workgroup before the kernel ends.
         bool arrived = false;
         if (k > 0 && t - 1 - B >= 0 && mine > 0)
-            arrived = pull_step<kUnifiedTables>(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb,
-                                       late ? nullptr : my_counter);
+            arrived = pull_step<kUnifiedTables, kLists>(s, r, g, row_p, slot_prev, ring_l, act, scan_l, e0, words, ka, kb,
+                                               late ? nullptr : my_counter);
         if (!late && !arrived) {
             wait_vector_memory();
             __syncthreads();
@@ -570,7 +639,8 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         // closing: spikes and inputs of the last step (less the delay offset), then fold the last slot
         const int64_t tl = r.step0 + done - 1;
         if (tl - B >= 0 && mine > 0)
-            pull_step<kUnifiedTables>(s, r, g, wrap(tl - B, r.hist), wrap(tl, L), ring_l, act, scan_l, e0, words, ka, kb);
+            pull_step<kUnifiedTables, kLists>(s, r, g, wrap(tl - B, r.hist), wrap(tl, L), ring_l, act, scan_l, e0, words, ka,
+                                              kb);
         __syncthreads();
         if (own) {
             float *prev = ring_l + (int)(tl % L) * GLIF3_NREC * span + tid;

@@ -61,6 +61,10 @@ class Glif3Simulator:
     single_workgroup  resident mode: a network of up to 1024 elements whose whole ring fits LDS runs in ONE
                 workgroup, without a grid barrier (about 1 us per step instead of 3); False keeps such a network
                 on the many-workgroup form
+    fired_lists  resident mode with several workgroups: every workgroup publishes the neurons that fired in a step
+                as a short list beside its ballots, and the others read the lists instead of expanding the whole
+                network's ballots (steps in which a list does not suffice are read from the ballots); False: always
+                from the ballots.  Same results either way.
     pull        launch-per-step mode only: sum the recurrent arrivals of a step in one pass over a target-major
                 copy of the table from the spike-bit history, instead of pushing them into the ring with global
                 atomics as spikes occur -- the faster form for batched runs.  "auto": batch >= 8 (and delay_offset
@@ -76,7 +80,7 @@ class Glif3Simulator:
 
     def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
                  asc_init=None, u_init=None, i_ext=None, device=None, resident="auto", delay_offset="auto",
-                 pull="auto", single_workgroup=True):
+                 pull="auto", single_workgroup=True, fired_lists=True):
         self.lib = _lib.load()
         self.dev = device or _dev()
         self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
@@ -164,12 +168,13 @@ class Glif3Simulator:
             raise ValueError("the packed synapse tables index at most 2^24 neurons")
         self.res_sync = torch.zeros(_lib.RES_SYNC_WORDS, dtype=torch.int32, device=self.dev)
         self.res_span = self.res_groups = 0
-        self.rec_seg = self.inp_seg = self.res_unified = None
+        self.rec_seg = self.inp_seg = self.res_unified = self.res_fired = None
         self._pending_check = False
         self.probe_ids = self.probe_col = None
         self.probe_every = 1
         self.spin_limit = 0  # resident mode: polls of the grid barrier before giving up (0 = built-in limit)
         self.single_workgroup = bool(single_workgroup)
+        self.fired_lists = bool(fired_lists)
         if resident:
             self._setup_resident(required=(resident is True))
         self.pull_table = self.pull_syn = self.pull_work = None
@@ -230,6 +235,9 @@ class Glif3Simulator:
             self.rec_seg, self.inp_seg = seg[:self.n], seg[self.n:]
             self.res_unified = (packed, seg)
         self.res_span, self.res_groups = span, groups
+        # the lists of fired neurons the workgroups publish beside their ballots (bmtk_glif3_sim.res_fired)
+        self.res_fired = (torch.zeros(self.hist_slots * groups * _lib.RES_FIRED_SLOTS, dtype=torch.int32, device=self.dev)
+                          if groups > 1 and self.fired_lists else None)
 
     def check(self):
         """Raise if a resident run since the last check gave up on its grid barrier (synchronises).  The abort
@@ -327,6 +335,7 @@ class Glif3Simulator:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
             s.res_spin_limit = int(self.spin_limit)
             s.rec_seg, s.inp_seg = _p(self.rec_seg), _p(self.inp_seg)
+            s.res_fired = _p(self.res_fired)
             if self.res_unified is not None and s.inp_packed and self.res_groups > 1:
                 s.inp_packed = s.rec_packed      # the input offsets count from the start of the joint table
         if bits is not None:

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 15
+#define BMTK_AMD_ABI_VERSION 16
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -187,6 +187,8 @@ int bmtk_csr_segment_offsets(int64_t n_rows, const int32_t *indptr, const int32_
 
 #define BMTK_RES_SYNC_STRIDE 1088                          /* words: 4 KiB + 256 B */
 #define BMTK_RES_SYNC_WAYS 8                               /* counters a step's arrivals are spread over */
+#define BMTK_RES_FIRED_SLOTS 16       /* places of a workgroup's list in bmtk_glif3_sim.res_fired */
+#define BMTK_RES_FIRED_MANY 0xFFFFFFFFu /* ... more neurons fired than the list holds */
 #define BMTK_RES_SYNC_WORDS ((1 + 64 * BMTK_RES_SYNC_WAYS) * BMTK_RES_SYNC_STRIDE) /* size of bmtk_glif3_sim.res_sync */
 
 /* Everything nest.Simulate needs for a forward run (bmtk/simulator/pointnet/pointsimulator.py:159-166). */
@@ -262,6 +264,15 @@ typedef struct bmtk_glif3_sim {
                                   * flag is sticky: no call clears it, and a call that finds it set does nothing,
                                   * so a failure cannot be overwritten before the host has seen it; the host
                                   * clears it after reading. */
+    uint32_t *res_fired;         /* optional, several workgroups only: [hist_slots][res_groups][BMTK_RES_FIRED_SLOTS]
+                                  * words, zeroed by the caller once and then left to the library.  Beside its
+                                  * ballots a workgroup publishes the neurons that fired in a step as a short list
+                                  * (number + 1; 0 = free place; all places BMTK_RES_FIRED_MANY when the list does not
+                                  * hold them), and the other workgroups read the lists instead of expanding the
+                                  * ballots of the whole network, each for itself; steps in which some list did not
+                                  * suffice are read from the ballots.  NULL: always from the ballots (a simulation passes it in
+                                  * every call or in none: the lists of a call's last steps are read by the next).  Used by runs
+                                  * without slack only (largest delay offset: the others do not wait per step). */
     /* Pull form of the recurrent delivery for batched runs (optional; launch-per-step mode with delay_offset 0
      * and hist_slots == ring_slots): a TARGET-major packed copy of the recurrent table.  The recurrent arrivals
      * of step t-1 are then summed in one pass over that table from the spike-bit history

@@ -60,6 +60,7 @@ def test_every_driver_equals_the_oracle(seed):
     if batch == 1:
         drivers.append(dict(resident=True))                           # up to 1024 neurons: the single-workgroup form
         drivers.append(dict(resident=True, single_workgroup=False))   # the many-workgroup form at the same odd sizes
+        drivers.append(dict(resident=True, single_workgroup=False, fired_lists=False))   # ... read from the ballots only
     for kw in drivers:
         sim = Glif3Simulator(n, cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=rec, inp=inp,
                              i_ext=cfg["i_ext"], **kw)

@@ -564,3 +564,39 @@ def test_single_workgroup_form_equals_the_other_drivers(n, max_delay, extra):
             np.testing.assert_array_equal(outs[name][k], outs["step"][k], err_msg="%s %s" % (name, k))
         for k in outs["step"]["state"]:
             np.testing.assert_array_equal(outs[name]["state"][k], outs["step"]["state"][k], err_msg="%s %s" % (name, k))
+
+
+def test_lists_of_fired_neurons_equal_the_ballots():
+    """Beside its ballots a workgroup of the many-workgroup form publishes the neurons that fired as a list of 16
+    places, which the other workgroups read instead of expanding the ballots; a step in which some workgroup had more
+    spikes than places is read from the ballots.  A network driven into volleys (steps with 40 spikes in one
+    workgroup) between quiet stretches (steps with a few) takes both ways: raster, state and ring equal those of a run
+    that never uses the lists and those of the launch-per-step driver, bit for bit, over three calls."""
+    import torch
+    n = 300
+    cfg = synthetic.small_glif3_network(n=n, n_in=100, steps=600, seed=77, in_w_scale=8.0, in_fanout=60, in_rate=30.0,
+                                        p_conn=0.1, w_scale=2.0, max_delay=4, n_classes=1)
+    for key in ("rec_src", "inp_src"):
+        cfg[key] = _integer_weights(cfg[key])
+    rng = np.random.default_rng(5)
+    i_ext = np.where(np.arange(n) % 64 < 40, 3000.0, rng.uniform(0.0, 300.0, n)).astype(np.float32)  # 40 of 64 in step
+    outs = {}
+    for name, kw in (("step", dict(resident=False)), ("lists", dict(resident=True, single_workgroup=False)),
+                     ("ballots", dict(resident=True, single_workgroup=False, fired_lists=False))):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], i_ext=i_ext, **kw)
+        if name != "step":
+            assert sim.res_groups == 5 and (sim.res_fired is not None) == (name == "lists")
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        bits = [sim.run(steps)["bits"] for steps in (1, 249, 350)]
+        sim.check()
+        outs[name] = dict(raster=sim.raster(torch.cat(bits)).cpu().numpy(), state=sim.state.to_numpy(),
+                          ring=sim.ring.cpu().numpy())
+    per_group = np.add.reduceat(outs["step"]["raster"].astype(np.int64), np.arange(0, n, 64), axis=1)  # [steps][5]
+    busiest = per_group.max(axis=1)
+    assert (busiest > 16).sum() >= 50 and ((busiest >= 1) & (busiest <= 16)).sum() >= 50   # both ways are taken
+    for name in ("lists", "ballots"):
+        for k in ("raster", "ring"):
+            np.testing.assert_array_equal(outs[name][k], outs["step"][k], err_msg="%s %s" % (name, k))
+        for k in outs["step"]["state"]:
+            np.testing.assert_array_equal(outs[name]["state"][k], outs["step"]["state"][k], err_msg="%s %s" % (name, k))
