@@ -215,6 +215,7 @@ __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Residen
     };
     bool arrived_above = false;
     if (kLists && s.res_fired && k1 - k0 <= kResBlock) {
+        PROF_T(p0);
         constexpr unsigned kManyFlag = 1u << 20;  // in a count: some list did not suffice (1024 of them still fit 32 bits)
         static_assert(kManyFlag > (unsigned)kActCap && 5 * kResBlock <= kActCap, "a step read from the lists always fits the row list");
         const unsigned long long *lists = reinterpret_cast<const unsigned long long *>(
@@ -237,6 +238,7 @@ __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Residen
         if (arrival) wait_vector_memory();  // the loads are back already; this is for the stores of the update
         __syncthreads();
         if (arrival && tid == 0) __hip_atomic_fetch_add(arrival, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        PROF_T(p1);
         const unsigned part = wave_inclusive_scan(lane_id() < kResBlock / kWave ? scan_l[lane_id()] : 0u);
         const unsigned total = (unsigned)bcast_i((int)part, kResBlock / kWave - 1);
         const unsigned base = wave > 0 ? (unsigned)__shfl((int)part, wave - 1, kWave) : 0u;
@@ -247,8 +249,14 @@ __device__ __forceinline__ bool pull_step(const bmtk_glif3_sim &s, const Residen
                 if (id[u] != 0u) act[pos++] = id[u] - 1u;
             if (has_event) act[pos] = kUnified ? event_row + (unsigned)s.n_neurons : event_row | kInputTag;
             __syncthreads();
+            PROF_T(p2);
             pull_listed(total);
             __syncthreads();
+            PROF_T(p3);
+            PROF_ADD(4, p0, p1);
+            PROF_ADD(5, p1, p2);
+            PROF_ADD(6, p2, p3);
+            PROF_BLK(3, p2, p3);
             return arrival != nullptr;
         }
         // this step from the ballots (the arrival has been made)
