@@ -376,7 +376,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     __shared__ int go_on;
     __shared__ unsigned scan_l[kResBlock / kWave];
     __shared__ unsigned fired_l[BMTK_RES_FIRED_SLOTS];  // this workgroup's list of the step: neuron + 1
-    __shared__ unsigned fired_n;
+    __shared__ unsigned fired_n[2];  // how many fired in this step and the one before
     const int tid = threadIdx.x;
     const int lane = lane_id();
     // Workgroups are dispatched round-robin over the 8 XCDs (block b runs on XCD
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     // (one thread looks for the whole workgroup, so that all of its threads take the same way)
     if (tid == 0) {
         go_on = load_agent(abort_word) == 0u;
-        fired_n = 0u;
+        fired_n[0] = fired_n[1] = 0u;
     }
     __syncthreads();
     if (!go_on) return;
@@ -431,6 +431,13 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
     // the spike record may be split into several lists, one per group of workgroups
     const unsigned rec_ways = s.spike_ways > 1 ? (unsigned)s.spike_ways : 1u;
     const unsigned long long rec_way = blockIdx.x & (rec_ways - 1u), rec_cap = (unsigned long long)s.spike_cap / rec_ways;
+    // With as many lists as workgroups this one appends to its list alone: its count lives in a register of every
+    // thread (first loaded, written back at the end), a spike's place is that count plus the spike's rank among the
+    // workgroup's spikes of the step (the LDS atomic that also builds the list of fired neurons), and no wavefront
+    // waits for an atomic on device memory, which the arrivals of a step would queue up behind.
+    const bool own_record = !kLate && s.spike_count != nullptr && rec_ways >= gridDim.x;
+    unsigned long long rec_count = own_record ? s.spike_count[rec_way * BMTK_RECORD_COUNT_STRIDE] : 0ull;
+    const bool count_fired = own_record || (kLists && s.res_fired != nullptr);
     // the input events of the step pulled in step t, u = t-1-B, are in_events[ka, kb); the bound for the
     // next step is fetched a step ahead.  Steps before 0 have no events (in_ptr[0] = 0).
     const int B = r.offset;
@@ -540,12 +547,18 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         // memory round trip away.  It is only asked for here and looked at after the pull, so that no wavefront
         // stops for it in the update (which every other wavefront of the workgroup would wait out at the next
         // barrier).
-        if (kLists && s.res_fired && m != 0ull && spike) {
-            const unsigned at = atomicAdd(&fired_n, 1u);
-            if (at < BMTK_RES_FIRED_SLOTS) fired_l[at] = (unsigned)e + 1u;
+        if (count_fired && m != 0ull && spike) {
+            const unsigned at = atomicAdd(&fired_n[k & 1], 1u);
+            if (kLists && s.res_fired && at < BMTK_RES_FIRED_SLOTS) fired_l[at] = (unsigned)e + 1u;
+            if (own_record && rec_count + at < rec_cap) {
+                const unsigned long long idx = rec_way * rec_cap + rec_count + at;
+                s.spike_step[idx] = (int32_t)t;
+                s.spike_elem[idx] = (int32_t)e;
+                if (s.spike_frac) s.spike_frac[idx] = frac;
+            }
         }
         unsigned long long rec_base = 0ull;
-        if (s.spike_count && m != 0ull && lane == __ffsll((long long)m) - 1)
+        if (s.spike_count && !own_record && m != 0ull && lane == __ffsll((long long)m) - 1)
             rec_base = atomicAdd(s.spike_count + rec_way * BMTK_RECORD_COUNT_STRIDE, (unsigned long long)__popcll(m));
         done = k + 1;
         // With no slack (S = 0) the arrival is signalled early in the pull so that the barrier fills while
@@ -570,13 +583,15 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
             }
             // the list of this step, complete since the workgroup met: out with it, like the ballots (the arrival
             // waits for the store), and the count back to zero (it is added to again after the barriers of the pull)
+            if (own_record) rec_count += fired_n[k & 1];
             if (kLists && s.res_fired && tid < BMTK_RES_FIRED_SLOTS && g < r.n_groups) {  // (the grid is rounded up)
-                const unsigned n = fired_n;
+                const unsigned n = fired_n[k & 1];
                 const unsigned word = n > BMTK_RES_FIRED_SLOTS ? BMTK_RES_FIRED_MANY : ((unsigned)tid < n ? fired_l[tid] : 0u);
                 __hip_atomic_store(s.res_fired + ((int64_t)row_t * r.n_groups + g) * BMTK_RES_FIRED_SLOTS + tid, word,
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (tid == 0) fired_n = 0u;
             }
+            // the other count, last read a barrier ago and next added to a barrier on, back to zero
+            if (count_fired && tid == 0) fired_n[(k + 1) & 1] = 0u;
         }
         PROF_T(c2);
 #ifdef BMTK_RES_PROFILE
@@ -601,7 +616,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         ka = kb;
         kb = ((int64_t)__builtin_amdgcn_readfirstlane((int)(kn_lanes >> 32)) << 32) |
              (int64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)kn_lanes);
-        if (s.spike_count && m != 0ull) {  // the places asked for above: the answer has long arrived
+        if (s.spike_count && !own_record && m != 0ull) {  // the places asked for above: the answer has long arrived
             unsigned long long idx = bcast_u64(rec_base, __ffsll((long long)m) - 1) + (unsigned long long)lane_prefix(m);
             if (spike && idx < rec_cap) {
                 idx += rec_way * rec_cap;  // this workgroup's list
@@ -662,6 +677,7 @@ __global__ __launch_bounds__(kResBlock) void sim_resident_kernel(bmtk_glif3_sim 
         __syncthreads();
     }
     if (own) glif3_store(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
+    if (own_record && tid == 0) s.spike_count[rec_way * BMTK_RECORD_COUNT_STRIDE] = rec_count;
     for (int c = tid; c < L * GLIF3_NREC * span; c += kResBlock) {
         const int dr = c / span, i = c - dr * span;
         if (i < mine) s.ring[(int64_t)dr * ne + e0 + i] = ring_l[c];

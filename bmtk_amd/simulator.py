@@ -386,14 +386,19 @@ class Glif3Simulator:
             ways = 1
             while ways * 2 <= min(RECORD_WAYS, n_wg) and record_cap >= ways * 2 * 1024:
                 ways *= 2
+            if self.res_groups > RECORD_WAYS and self.delay_offset == 0 and record_cap >= 256 * 1024:
+                # the resident kernel without slack: with a list per workgroup (at most 256 are launched) a
+                # workgroup keeps its count in a register and no wavefront waits for an atomic on device memory
+                ways = 256
             if record_ways is not None:      # the caller's choice: a power of two up to 256
                 ways = int(record_ways)
                 if ways < 1 or ways > 256 or ways & (ways - 1):
                     raise ValueError("record_ways must be a power of two in 1..256")
             record_cap = -(-int(record_cap) // ways) * ways
-            record = dict(step=torch.zeros(record_cap, dtype=torch.int32, device=self.dev),
-                          elem=torch.zeros(record_cap, dtype=torch.int32, device=self.dev),
-                          frac=torch.zeros(record_cap, dtype=torch.float32, device=self.dev),
+            # (only the counted entries are ever read: no need to clear a gigabyte of room first)
+            record = dict(step=torch.empty(record_cap, dtype=torch.int32, device=self.dev),
+                          elem=torch.empty(record_cap, dtype=torch.int32, device=self.dev),
+                          frac=torch.empty(record_cap, dtype=torch.float32, device=self.dev),
                           count=torch.zeros(1 if ways == 1 else ways * _lib.RECORD_COUNT_STRIDE, dtype=torch.int64,
                                             device=self.dev), ways=ways)
         s = self._struct(bits, record)
@@ -437,7 +442,9 @@ class Glif3Simulator:
             keep = slice(0, stored[0])
         else:                                                  # the filled part of every list, one after the other
             dev = record["step"].device
-            keep = torch.cat([torch.arange(w * way_cap, w * way_cap + c, device=dev) for w, c in enumerate(stored)])
+            filled = torch.tensor(stored, dtype=torch.int64, device=dev)
+            first = torch.arange(ways, dtype=torch.int64, device=dev) * way_cap - (torch.cumsum(filled, 0) - filled)
+            keep = torch.arange(sum(stored), dtype=torch.int64, device=dev) + torch.repeat_interleave(first, filled)
         out = dict(step=record["step"][keep], elem=record["elem"][keep], frac=record["frac"][keep],
                    count=int(counts.sum()), overflow=bool((counts > way_cap).any()))
         if sort_scale is not None:

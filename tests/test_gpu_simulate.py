@@ -490,8 +490,10 @@ def test_spike_record_in_several_lists(resident):
         out = sim.run(cfg["steps"], record_cap=cap, record_ways=ways)
         return sim, out
     sim, out = run(RECORD_WAYS * 4096)
-    # as many lists as the power of two below the number of workgroups (40 per-step, 312 resident), at most 64
-    assert out["record"]["ways"] == (RECORD_WAYS if resident else 32) and bool(sim.res_span) == resident
+    # as many lists as the power of two below the number of workgroups (40 per-step), at most 64; the resident kernel
+    # without slack gets 256, a list per workgroup, which appends to it with its count in a register
+    assert out["record"]["ways"] == (256 if resident else 32) and bool(sim.res_span) == resident
+    assert not resident or sim.res_groups > RECORD_WAYS
     rec = sim.collect_record(out["record"])
     ras = sim.raster(out["bits"]).cpu().numpy()
     assert rec["count"] == int(ras.sum()) > 20000 and not rec["overflow"]
@@ -516,6 +518,11 @@ def test_spike_record_in_several_lists(resident):
     k1, f1 = keyed(rec1)
     np.testing.assert_array_equal(k, k1)
     np.testing.assert_array_equal(f, f1)
+    sim64, out64 = run(RECORD_WAYS * 4096, ways=RECORD_WAYS)      # lists shared by workgroups: a counter in memory each
+    assert out64["record"]["ways"] == RECORD_WAYS
+    k64, f64 = keyed(sim64.collect_record(out64["record"]))
+    np.testing.assert_array_equal(k, k64)
+    np.testing.assert_array_equal(f, f64)
     frac = f
     assert frac.min() >= 0.0 and frac.max() <= 1.0
     # a record too small for the run: counted in full, reported as incomplete
