@@ -265,7 +265,8 @@ typedef struct bmtk_glif3_sim {
                                   * so a failure cannot be overwritten before the host has seen it; the host
                                   * clears it after reading. */
     uint32_t *res_fired;         /* optional, several workgroups only: [hist_slots][res_groups][BMTK_RES_FIRED_SLOTS]
-                                  * words, zeroed by the caller once and then left to the library.  Beside its
+                                  * words (3 rows when hist_slots is 0), zeroed by the caller once and then left to
+                                  * the library.  Beside its
                                   * ballots a workgroup publishes the neurons that fired in a step as a short list
                                   * (number + 1; 0 = free place; all places BMTK_RES_FIRED_MANY when the list does not
                                   * hold them), and the other workgroups read the lists instead of expanding the
@@ -328,7 +329,9 @@ typedef struct bmtk_glif3_sim {
      * spike_cap a multiple of W) the record is W lists of spike_cap / W entries each, list w in entries
      * [w * spike_cap / W, (w + 1) * spike_cap / W) of spike_step / spike_elem / spike_frac with its counter in
      * spike_count[w * BMTK_RECORD_COUNT_STRIDE]; a workgroup appends to list (its number mod W).  A counter keeps
-     * counting past its list's end.  0 or 1: one list, as above. */
+     * counting past its list's end.  0 or 1: one list, as above.  With at least as many lists as workgroups (the
+     * resident mode launches at most 256) and no delay offset, a workgroup has a list of its own and keeps the count
+     * in a register for the length of a call: no atomics on device memory at all. */
     int32_t spike_ways;
     int32_t _pad2;
 } bmtk_glif3_sim;
