@@ -36,7 +36,7 @@
 //     up, fired neurons from the last walker down, so that a walker seldom has
 //     two;
 //   * running counters instead of 64-bit divisions and multiplications.
-// Items beyond the 128 + 128 a step's lists hold, and all fired neurons when
+// Items beyond the 128 events and 512 neurons a step's lists hold, and all fired neurons when
 // the delay offset B > 0 (their spikes are B steps old: from the ballots of the
 // last steps kept in LDS when B < 4, else from the history row written B steps
 // ago), take a slower way at delivery time: prefix sums over the ballots'
@@ -63,7 +63,7 @@ constexpr int kSoloWaves = kSoloBlock / kWave;
 constexpr int kStoreWave = kSoloWaves - 1, kFetchWave = kSoloWaves - 2, kWalkers = kSoloWaves - 2;
 constexpr int kWalkRole = 0, kFetchRole = 1, kStoreRole = 2;  // what a wavefront does beside updating its neurons
 constexpr int kEvCap = 128;                  // input events of a step that become items; further ones are read in place
-constexpr int kFiredCap = 128;               // fired neurons of a step that become items; further ones: overflow ballot
+constexpr int kFiredCap = 512;               // fired neurons of a step that become items; further ones: overflow ballot
 constexpr int kNearSteps = 4;                // the ballots of so many steps stay in LDS (delay offsets below that)
 constexpr size_t kSoloStaticLds = 1024;      // the kernel's static LDS, rounded up
 constexpr unsigned kNoSample = 0xFFFFFFFFu;  // a probe cell nobody writes (a NaN no update produces)
@@ -177,7 +177,19 @@ __global__ __launch_bounds__(kSoloBlock) void sim_solo_kernel(bmtk_glif3_sim s, 
         // = min(x, x - 4L) with x = slot0*4 + that byte (unsigned)
         const unsigned dq = sy.x >> 24;
         const unsigned plane = min(dq + q_lo, dq + q_wrap);
-        atomicAdd(ring_l + (plane * (unsigned)span + (sy.x & 0xFFFFFFu)), __uint_as_float(sy.y));
+        // An LDS float atomic is worked off lane by lane (about three clocks each: 135 for a row of 45 synapses), a
+        // compare-and-swap in some 40 clocks per instruction whatever the number of lanes: the addition is a
+        // compare-and-swap loop (a lane goes round again only if its cell changed in between: two synapses of
+        // the row on one target and receptor, or another wavefront's row).  The one LDS unit is what a busy step of
+        // this form is short of: 150 rows a step are 6,700 lanes.
+        unsigned *cell = reinterpret_cast<unsigned *>(ring_l + (plane * (unsigned)span + (sy.x & 0xFFFFFFu)));
+        const float w = __uint_as_float(sy.y);
+        unsigned old = *cell;  // only seeds the loop: a stale value costs one more round
+        while (true) {
+            const unsigned seen = atomicCAS(cell, old, __float_as_uint(__uint_as_float(old) + w));
+            if (seen == old) break;
+            old = seen;
+        }
     };
     auto walk = [&](const uint2 *__restrict__ tab, int p0, int p1) {
         for (int q = p0 + lane; q < p1; q += kWave) add(tab[q]);
@@ -216,26 +228,43 @@ __global__ __launch_bounds__(kSoloBlock) void sim_solo_kernel(bmtk_glif3_sim s, 
     uint2 ev_first = make_uint2(0u, 0u), fi_first = make_uint2(0u, 0u);
     // The additions go to slots t .. t+L-2, never to slot t-1, which other wavefronts may still be folding: no
     // barrier is needed before them.
-    auto deliver = [&]() {
+    // Items j, j + kWalkers, ... of a list (below n): a busy step has many more items than walkers, and a row taken
+    // alone costs a whole trip to memory, so four rows' first synapses are asked for before any is added.
+    auto rounds = [&](const int2 *__restrict__ items, const uint2 *__restrict__ tab, int j, int n)
+                      __attribute__((always_inline)) {
+        constexpr int kAhead = 4;
+        for (; j < n; j += kAhead * kWalkers) {
+            int p0[kAhead], len[kAhead];
+            uint2 head[kAhead];
+#pragma unroll
+            for (int q = 0; q < kAhead; ++q) {
+                const int2 it = j + q * kWalkers < n ? items[j + q * kWalkers] : make_int2(0, 0);
+                p0[q] = __builtin_amdgcn_readfirstlane(it.x);
+                len[q] = __builtin_amdgcn_readfirstlane(it.y);
+            }
+#pragma unroll
+            for (int q = 0; q < kAhead; ++q)
+                if (lane < len[q]) head[q] = tab[p0[q] + lane];
+#pragma unroll
+            for (int q = 0; q < kAhead; ++q) {
+                if (lane < len[q]) add(head[q]);
+                walk(tab, p0[q] + kWave, p0[q] + len[q]);
+            }
+        }
+    };
+    // (inlined by force: called out of line, everything it captures would live in memory)
+    auto deliver = [&]() __attribute__((always_inline)) {
         if (wave >= kWalkers) return;
         const int n_evf = min(c_n_ev, kEvCap);
         if (wave < n_evf) {
             if (lane < ev_len) add(ev_first);
             walk(inp_tab, ev_p0 + kWave, ev_p0 + ev_len);
-            for (int j = wave + kWalkers; j < n_evf; j += kWalkers) {
-                const int2 it = ev_items[c_buf * kEvCap + j];
-                const int p0 = __builtin_amdgcn_readfirstlane(it.x);
-                walk(inp_tab, p0, p0 + __builtin_amdgcn_readfirstlane(it.y));
-            }
+            rounds(ev_items + c_buf * kEvCap, inp_tab, wave + kWalkers, n_evf);
         }
         if (kWalkers - 1 - wave < c_n_fi) {
             if (lane < fi_len) add(fi_first);
             walk(rec_tab, fi_p0 + kWave, fi_p0 + fi_len);
-            for (int j = 2 * kWalkers - 1 - wave; j < c_n_fi; j += kWalkers) {
-                const int2 it = fi_items[c_buf * kFiredCap + j];
-                const int p0 = __builtin_amdgcn_readfirstlane(it.x);
-                walk(rec_tab, p0, p0 + __builtin_amdgcn_readfirstlane(it.y));
-            }
+            rounds(fi_items + c_buf * kFiredCap, rec_tab, 2 * kWalkers - 1 - wave, c_n_fi);
         }
         // the slower ways
         for (int i = kEvCap + wave; i < c_n_ev; i += kWalkers) {

@@ -22,7 +22,7 @@ RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static 
 # the single-workgroup form: per element the spike offsets and probed potentials of two steps (SOLO_LDS_PER_ELEMENT);
 # the items (rows to walk) of two steps and its static LDS (SOLO_LDS_EXTRA)
 SOLO_LDS_PER_ELEMENT = 4 * 4
-SOLO_LDS_EXTRA = 4096 + 1024
+SOLO_LDS_EXTRA = 10240 + 1024
 RECORD_WAYS = 64                # lists a large spike record is split into (bmtk_glif3_sim.spike_ways)
 
 
