@@ -336,6 +336,27 @@ def bench_bptt(torch, steps=600):
     return entries
 
 
+def bench_small_network(torch):
+    """The size of the reference's own examples: configuration 0's 450 neurons, which ONE workgroup holds (the
+    single-workgroup form of the resident kernel), with the spike record on as the front ends run it."""
+    from bmtk_amd import synthetic
+    from bmtk_amd.simulator import Glif3Simulator
+    out = []
+    cfg = synthetic.small_glif3_network(n=450, n_in=1000, steps=21000, seed=0, in_w_scale=2.0)
+    small = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"])
+    small.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    small.run(1000)
+    wall, dev = time_region(torch, lambda: small.run(20000, spike_bits=False, record_cap=1 << 20))
+    small.check()
+    out.append({"kernel": "sim_solo_kernel (one workgroup, spike record on)",
+                "workload": "450 GLIF3 neurons (configuration 0's network), 20000 steps", "groups": small.res_groups,
+                "us_per_sim_step": dev / 20000 * 1e6, "neuron_updates_per_s": 450 * 20000 / wall,
+                "roofline": {"bound": "hbm", "achieved": 450 * B_PER_UPDATE_PLAIN * 20000 / dev / 1e9, "peak": HBM_PEAK_GBS,
+                             "unit": "GB/s", "frac": 450 * B_PER_UPDATE_PLAIN * 20000 / dev / 1e9 / HBM_PEAK_GBS,
+                             "traffic": None, "what": "one workgroup on one compute unit: bound by instruction issue (about 2,200 instructions per step over its 16 wavefronts), not by memory"}})
+    return out
+
+
 def bench_front_end(torch, sim, steps):
     """What a run through the front ends costs (bmtk_amd.nest.Simulate, bmtk_amd.pointnet.PointSimulator.run): the same
     V1-scale simulation with the spike record on (spike times need the crossing fraction), then the record joined,
@@ -364,18 +385,7 @@ def bench_front_end(torch, sim, steps):
             "roofline": {"bound": "hbm", "achieved": alg_step * steps / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": alg_step * steps / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
                          "what": "state update bytes only (103 B per neuron and step)"}}]
-    cfg = synthetic.small_glif3_network(n=450, n_in=1000, steps=21000, seed=0, in_w_scale=2.0)
-    small = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"])
-    small.set_input_events(cfg["in_ptr"], cfg["in_events"])
-    small.run(1000)
-    wall, dev = time_region(torch, lambda: small.run(20000, spike_bits=False, record_cap=1 << 20))
-    small.check()
-    out.append({"kernel": "sim_solo_kernel (one workgroup, spike record on)",
-                "workload": "450 GLIF3 neurons (configuration 0's network), 20000 steps", "groups": small.res_groups,
-                "us_per_sim_step": dev / 20000 * 1e6, "neuron_updates_per_s": 450 * 20000 / wall,
-                "roofline": {"bound": "hbm", "achieved": 450 * B_PER_UPDATE_PLAIN * 20000 / dev / 1e9, "peak": HBM_PEAK_GBS,
-                             "unit": "GB/s", "frac": 450 * B_PER_UPDATE_PLAIN * 20000 / dev / 1e9 / HBM_PEAK_GBS,
-                             "traffic": None, "what": "one workgroup on one compute unit: bound by instruction issue (about 2,200 instructions per step over its 16 wavefronts), not by memory"}})
+    out += bench_small_network(torch)
     return out
 
 
@@ -496,7 +506,8 @@ def main():
     if set(modes) - set(PROPAGATION_MODES):
         sys.exit("bench.py: --propagation-modes takes %s" % ", ".join(PROPAGATION_MODES))
     groups = {"state": bench_state_update, "compaction": bench_compaction,
-              "propagation": lambda t: bench_propagation(t, modes=modes), "bptt": bench_bptt}
+              "propagation": lambda t: bench_propagation(t, modes=modes), "bptt": bench_bptt,
+              "small": bench_small_network}   # (the headline run reports "small" with its front-end entries)
     want = [g for g in args.kernels.split(",") if g]
     unknown = set(want) - set(groups)
     if unknown:
