@@ -11,12 +11,15 @@
 // microsecond, i.e. millions of steps) are this case: a step costs about a
 // microsecond instead of the three the grid barrier sets as a floor.
 //
-// What sets the pace of such a step is the chain of things that must follow
-// one another -- LDS round trips, waits for memory, serial sections -- not the
-// amount of work.  On this hardware a wavefront's vector memory operations
-// complete in the order issued: a wavefront that waits for a load also waits
-// for every store it issued before it, and a store is acknowledged only after
-// a trip to the far side of L2, about as long as the whole step.  Hence:
+// One compute unit runs it all, so what sets the pace of a step is how many
+// instructions its sixteen wavefronts issue (a SIMD issues for one of its four
+// wavefronts every four cycles; scalar bookkeeping counts like arithmetic), the
+// chain of things that must follow one another -- LDS round trips, waits for
+// memory, serial sections -- and, in a busy step, the one LDS unit.  On this
+// hardware a wavefront's vector memory operations complete in the order
+// issued: a wavefront that waits for a load also waits for every store it
+// issued before it, and a store is acknowledged only after a trip to the far
+// side of L2, about as long as the whole step.  Hence:
 //   * a neuron that fires appends ITS OWN row (first synapse, length: two
 //     registers of its thread) to the step's list of items in LDS; the input
 //     events of the step arrive there the same way.  After the barrier a
@@ -35,9 +38,13 @@
 //     other fourteen WALK rows: input events are dealt from the first walker
 //     up, fired neurons from the last walker down, so that a walker seldom has
 //     two;
-//   * running counters instead of 64-bit divisions and multiplications.
-// Items beyond the 128 events and 512 neurons a step's lists hold, and all fired neurons when
-// the delay offset B > 0 (their spikes are B steps old: from the ballots of the
+//   * the loop over the steps is compiled once per role of a wavefront, so
+//     that none steps through the branches and counters of the others, with
+//     running counters instead of 64-bit divisions and multiplications;
+//   * additions into the LDS ring are compare-and-swap loops: the LDS unit
+//     works a float atomic off lane by lane.
+// Items beyond the 128 events and 512 neurons a step's lists hold, and all
+// fired neurons when the delay offset B > 0 (their spikes are B steps old: from the ballots of the
 // last steps kept in LDS when B < 4, else from the history row written B steps
 // ago), take a slower way at delivery time: prefix sums over the ballots'
 // popcounts, row bounds from device memory.
