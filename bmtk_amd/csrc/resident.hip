@@ -19,6 +19,15 @@
 // Nothing but spike ballots, segment offsets and the synapses actually used
 // crosses the memory system: no global atomics, no state traffic.
 //
+// Without slack (see below) a workgroup publishes, beside its ballots, the
+// neurons that fired as a list of 16 places (res_fired: filled in LDS with one
+// LDS atomic per spiking lane, written out by one wavefront once the workgroup
+// has met after the update), and step 2 reads the lists -- four places per
+// thread -- instead of taking the ballots of the whole network apart bit by
+// bit, which every workgroup would do for itself; a step in which some list
+// did not suffice is read from the ballots.  The same count gives a spike its
+// place in the spike record when the workgroup has a record list of its own.
+//
 // Ballots live in a history of D rows, row t%D for step t.  With D = 3 a
 // workgroup waits for the barrier of step t at the end of step t: row t%3 is
 // read in step t+1 and next overwritten in step t+3, which a workgroup can only
