@@ -374,7 +374,7 @@ def bench_front_end(torch, sim, steps):
     wall, dev = time_region(torch, run)
     t0 = time.perf_counter()
     rec = sim.collect_record(res["out"]["record"], sort_scale=1.0)
-    senders, times = rec["elem"].cpu().numpy(), rec["time"].cpu().numpy()
+    times, senders = sim.to_host(rec["time"], rec["elem"])
     collect = time.perf_counter() - t0
     alg_step = N_V1 * B_PER_UPDATE_CLASS   # the state update alone; the events ride on top as in the headline
     out = [{"kernel": "sim_resident_kernel (spike record on) + collect_record",

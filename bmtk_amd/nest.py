@@ -496,8 +496,9 @@ def Simulate(t_ms):
             rec = sim.collect_record(out["record"], sort_scale=dt)
             if rec["overflow"]:
                 raise NESTError("more than {} spikes in one Simulate call; simulate in shorter pieces".format(cap))
-            times.append(rec["time"].cpu().numpy())
-            senders.append(s["neuron_ids"][rec["elem"].cpu().numpy()])
+            rec_time, rec_elem = sim.to_host(rec["time"], rec["elem"])
+            times.append(rec_time)
+            senders.append(s["neuron_ids"][rec_elem])
     sim.check()  # also without a recorder: Simulate returns only after the run is known to be valid
     s["steps_done"] = step0 + n_steps
     _S.status["biological_time"] = s["steps_done"] * dt

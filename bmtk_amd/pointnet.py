@@ -299,8 +299,9 @@ class PointSimulator:
             r = sim.collect_record(out["record"], sort_scale=self.dt)
             if r["overflow"]:
                 raise RuntimeError("spike record overflow: {} spikes, room for {}".format(r["count"], cap))
-            elems.append(r["elem"].cpu().numpy().astype(np.int64))
-            times.append(r["time"].cpu().numpy())
+            r_time, r_elem = sim.to_host(r["time"], r["elem"])
+            elems.append(r_elem.astype(np.int64))
+            times.append(r_time)
         self.simulator = sim
         self.spikes = {nw.population: (np.concatenate(elems), np.concatenate(times))}
         self._write_outputs()
