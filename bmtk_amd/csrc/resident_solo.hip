@@ -361,7 +361,7 @@ __global__ __launch_bounds__(kSoloBlock) void sim_solo_kernel(bmtk_glif3_sim s, 
                 }
                 int n_slow = 0;
                 if constexpr (!kZeroB) {
-                    // the neurons that fired in step u: all of them go the slower way
+                    // the neurons that fired in step u
                     unsigned long long v = 0ull;
                     if (u >= 0 && lane < words && has_rec) {
                         if (B < kNearSteps)
@@ -369,15 +369,38 @@ __global__ __launch_bounds__(kSoloBlock) void sim_solo_kernel(bmtk_glif3_sim s, 
                         else
                             v = __hip_atomic_load(hist + far_row * (words + 1) + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
+                    const unsigned cnt = (unsigned)__popcll(v);
+                    const bool any = __ballot(v != 0ull) != 0ull;  // (most steps of a fine resolution have none)
+                    const unsigned upto = any ? wave_inclusive_scan(cnt) : 0u;
+                    const int n_fired = any ? __builtin_amdgcn_readlane((int)upto, kWave - 1) : 0;
+                    unsigned n_items = 0u;
+                    if (!any) {
+                    } else if (n_fired <= kFiredCap) {
+                        // they become items here, a step's worth of time before the walkers want them: the neurons'
+                        // numbers first (into the places of the items), then, 64 at a time, their rows' bounds
+                        int2 *items = fi_items + buf * kFiredCap;
+                        unsigned at = upto - cnt;
+                        for (unsigned long long x = v; x; x &= x - 1ull)
+                            items[at++].x = lane * kWave + (__ffsll((long long)x) - 1);
+                        for (int i = lane; i < n_fired; i += kWave) {
+                            const int id = items[i].x;
+                            const int p0 = s.rec_indptr[id];
+                            items[i] = make_int2(p0, s.rec_indptr[id + 1] - p0);
+                        }
+                        n_items = (unsigned)n_fired;
+                        v = 0ull;
+                    } else {
+                        n_slow = n_fired;  // a volley beyond the list: all of them the slower way
+                    }
+                    if (lane == 0) count_l[cnt_row] = n_items;
                     if (lane < kSoloWaves) pair_l[buf][lane].y = v;
-                    n_slow = __builtin_amdgcn_readlane((int)wave_inclusive_scan((unsigned)__popcll(v)), kWave - 1);
                     far_row = far_row + 1 == r.hist ? 0 : far_row + 1;
                 }
                 if (lane == 0) {
                     meta_l[buf] = make_int4(n_ev, n_slow, (int)(unsigned)f_lo, (int)(f_lo >> 32));
                     // B = 0: the neurons count themselves as they fire; the entry of the NEXT step is cleared here: it
                     // was last read before the barrier behind us and is added to after the barrier ahead
-                    count_l[cnt_row == 2 ? 0 : cnt_row + 1] = 0u;
+                    if (kZeroB) count_l[cnt_row == 2 ? 0 : cnt_row + 1] = 0u;
                 }
                 // a step on: the events of step u+1, the bound after those of step u+2
                 if (s.in_ptr && k + 1 < r.n_steps) {

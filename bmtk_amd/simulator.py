@@ -75,6 +75,8 @@ class Glif3Simulator:
                 arrivals with a ring B slots shorter.  "auto": 0 while the largest delay is at most 63
                 steps (what the ring and the packed tables hold), else the smallest delay minus one --
                 the case of NEST networks run at a fine resolution (1-2 ms delays at 0.001-0.1 ms steps).
+                Also the smallest delay minus one when that is what lets a network of up to 1024 neurons keep its
+                whole ring in ONE workgroup's LDS (the resident form without a grid barrier).
                 The delay columns may then be any integer type; residual delays must stay within 63.
     """
 
@@ -108,6 +110,17 @@ class Glif3Simulator:
             raise ValueError("delays must be at least one step")
         if delay_offset == "auto":
             delay_offset = 0 if max_delay <= 63 else min_delay - 1
+            if (delay_offset == 0 and min_delay > 1 and resident and single_workgroup and self.batch == 1
+                    and self.n <= 1024 and not ring_slots):
+                # a small network whose whole ring only fits ONE workgroup's LDS (the form without a grid barrier)
+                # once the part all delays have in common is taken off: bmtk's example networks at dt = 0.1 ms
+                # (every delay 2 ms: 21 ring slots for 450 cells are 172 KB, 2 slots 16 KB)
+                whole = -(-self.n // 64) * 64
+
+                def fits(slots):
+                    return (slots * NREC * 4 + SOLO_LDS_PER_ELEMENT) * whole + SOLO_LDS_EXTRA <= RES_LDS_BYTES
+                if not fits(max_delay + 1) and fits(max_delay - min_delay + 2):
+                    delay_offset = min_delay - 1
         self.delay_offset = int(delay_offset)
         if not 0 <= self.delay_offset < min_delay:
             raise ValueError("delay_offset must lie in 0..smallest delay - 1")

@@ -607,3 +607,38 @@ def test_lists_of_fired_neurons_equal_the_ballots():
             np.testing.assert_array_equal(outs[name][k], outs["step"][k], err_msg="%s %s" % (name, k))
         for k in outs["step"]["state"]:
             np.testing.assert_array_equal(outs[name]["state"][k], outs["step"]["state"][k], err_msg="%s %s" % (name, k))
+
+
+def test_delay_offset_chosen_so_that_a_small_network_fits_one_workgroup():
+    """450 cells whose delays are all 20 steps (bmtk's example networks at dt = 0.1 ms: 2 ms everywhere) need 21 ring
+    slots, more than one workgroup's LDS holds for them; with the 19 steps all delays have in common taken off, two.
+    The automatic choice takes them off and runs the single-workgroup form: same raster, state and spike record as
+    the many-workgroup form with the full ring, bit for bit."""
+    import torch
+    n = 450
+    cfg = synthetic.small_glif3_network(n=n, n_in=100, steps=900, seed=5, in_w_scale=8.0, in_fanout=60, in_rate=30.0,
+                                        p_conn=0.08, w_scale=2.0, max_delay=1)
+    for key in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = _integer_weights(cfg[key])
+        cfg[key] = (indptr, indices, w, np.full_like(d, 20), r)
+    outs = {}
+    for name, kw in (("auto", dict()), ("full ring", dict(delay_offset=0))):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], **kw)
+        assert (sim.delay_offset, sim.L, sim.res_groups) == ((19, 2, 1) if name == "auto" else (0, 21, 8))
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        bits, recs = [], []
+        for steps in (1, 399, 500):
+            out = sim.run(steps, record_cap=1 << 17)
+            bits.append(out["bits"])
+            rec = sim.collect_record(out["record"], sort_scale=1.0)
+            assert not rec["overflow"]
+            recs.append(torch.stack([rec["time"], rec["elem"].double()]))
+        sim.check()
+        outs[name] = dict(raster=sim.raster(torch.cat(bits)).cpu().numpy(), rec=torch.cat(recs, dim=1).cpu().numpy(),
+                          state=sim.state.to_numpy())
+    assert outs["auto"]["raster"].sum() > 2 * n
+    np.testing.assert_array_equal(outs["auto"]["raster"], outs["full ring"]["raster"])
+    np.testing.assert_array_equal(outs["auto"]["rec"], outs["full ring"]["rec"])
+    for k in ("V", "asc", "y1", "y2", "ref"):
+        np.testing.assert_array_equal(outs["auto"]["state"][k], outs["full ring"]["state"][k], err_msg=k)
