@@ -43,11 +43,13 @@
 //     running counters instead of 64-bit divisions and multiplications;
 //   * additions into the LDS ring are compare-and-swap loops: the LDS unit
 //     works a float atomic off lane by lane.
-// Items beyond the 128 events and 512 neurons a step's lists hold, and all
-// fired neurons when the delay offset B > 0 (their spikes are B steps old: from the ballots of the
-// last steps kept in LDS when B < 4, else from the history row written B steps
-// ago), take a slower way at delivery time: prefix sums over the ballots'
-// popcounts, row bounds from device memory.
+// With a delay offset B > 0 the spikes handed over are B steps old: the fetch
+// wavefront takes their ballots (from the last steps' ballots kept in LDS when
+// B < 4, else from the history row written B steps ago) and turns them into
+// items itself, a step's worth of time before the walkers want them.  Items
+// beyond the 128 events and 512 neurons a step's lists hold take a slower way
+// at delivery time: prefix sums over ballots' popcounts, row bounds from device
+// memory.
 //
 // Per step t:
 //   1. fetch wavefront: the events of step t-B become items; the others: fold
