@@ -9,7 +9,7 @@
 // synapse row of a neuron that fired (every target is its own workgroup's).
 // bmtk's example networks (a few hundred cells, often at resolutions of a
 // microsecond, i.e. millions of steps) are this case: a step costs about a
-// microsecond instead of the three the grid barrier sets as a floor.
+// microsecond instead of the two and a half the grid barrier sets as a floor.
 //
 // One compute unit runs it all, so what sets the pace of a step is how many
 // instructions its sixteen wavefronts issue (a SIMD issues for one of its four

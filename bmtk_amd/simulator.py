@@ -59,7 +59,7 @@ class Glif3Simulator:
                 compute unit, ring slice within LDS; True: insist on it (ValueError otherwise); False: one launch
                 per step, which takes any batch and size
     single_workgroup  resident mode: a network of up to 1024 elements whose whole ring fits LDS runs in ONE
-                workgroup, without a grid barrier (about 1 us per step instead of 3); False keeps such a network
+                workgroup, without a grid barrier (about 1 us per step instead of 2.5); False keeps such a network
                 on the many-workgroup form
     fired_lists  resident mode with several workgroups: every workgroup publishes the neurons that fired in a step
                 as a short list beside its ballots, and the others read the lists instead of expanding the whole
