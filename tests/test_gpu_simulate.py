@@ -609,6 +609,49 @@ def test_lists_of_fired_neurons_equal_the_ballots():
             np.testing.assert_array_equal(outs[name]["state"][k], outs["step"]["state"][k], err_msg="%s %s" % (name, k))
 
 
+@pytest.mark.parametrize("extra", [0, 2, 6])
+def test_single_workgroup_form_with_more_spikes_and_events_than_its_lists_hold(extra):
+    """The single-workgroup form hands the rows to walk from step to step as items in LDS: up to 512 fired neurons
+    and up to 128 input events; what exceeds them is taken from the ballots and from the event list in place.  800 of
+    1024 neurons driven in step (volleys of more than 512 between steps with a few spikes) and 93-148 input events
+    per step take every way, without a delay offset (ballots in LDS), with one shorter than the kernel's near rows
+    and with a longer one (ballots through the history): raster, state, ring and spike record equal those of the
+    launch-per-step driver bit for bit, over three calls."""
+    import torch
+    n = 1024
+    cfg = synthetic.small_glif3_network(n=n, n_in=600, steps=500, seed=91, in_w_scale=4.0, in_fanout=30, in_rate=200.0,
+                                        p_conn=0.03, w_scale=1.0, max_delay=3, n_classes=1)
+    for key in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = _integer_weights(cfg[key])
+        cfg[key] = (indptr, indices, w, d.astype(np.int32) + extra, r)
+    rng = np.random.default_rng(5)
+    i_ext = np.where(np.arange(n) < 800, 3000.0, rng.uniform(0.0, 300.0, n)).astype(np.float32)
+    events = np.diff(cfg["in_ptr"])[:500]
+    assert (events > 128).sum() >= 50 and (events <= 128).sum() >= 50
+    outs = {}
+    for name, kw in (("step", dict(resident=False)), ("one", dict(resident=True))):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], i_ext=i_ext, delay_offset=extra, **kw)
+        assert sim.delay_offset == extra and sim.res_groups == (1 if name == "one" else 0)
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        bits, recs = [], []
+        for steps in (1, 199, 300):
+            out = sim.run(steps, record_cap=1 << 19)
+            bits.append(out["bits"])
+            rec = sim.collect_record(out["record"], sort_scale=1.0)
+            assert not rec["overflow"]
+            recs.append(torch.stack([rec["time"], rec["elem"].double()]))
+        sim.check()
+        outs[name] = dict(raster=sim.raster(torch.cat(bits)).cpu().numpy(), rec=torch.cat(recs, dim=1).cpu().numpy(),
+                          state=sim.state.to_numpy(), ring=sim.ring.cpu().numpy())
+    per_step = outs["step"]["raster"].sum(axis=1)
+    assert (per_step > 512).sum() >= 20 and ((per_step >= 1) & (per_step <= 512)).sum() >= 100
+    for k in ("raster", "rec", "ring"):
+        np.testing.assert_array_equal(outs["one"][k], outs["step"][k], err_msg=k)
+    for k in outs["step"]["state"]:
+        np.testing.assert_array_equal(outs["one"]["state"][k], outs["step"]["state"][k], err_msg=k)
+
+
 def test_delay_offset_chosen_so_that_a_small_network_fits_one_workgroup():
     """450 cells whose delays are all 20 steps (bmtk's example networks at dt = 0.1 ms: 2 ms everywhere) need 21 ring
     slots, more than one workgroup's LDS holds for them; with the 19 steps all delays have in common taken off, two.
