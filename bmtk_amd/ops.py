@@ -474,4 +474,4 @@ def unpack_bits(bits, ne):
     """int64 spike-bit words ``[..., words]`` -> uint8 flags ``[..., ne]`` (host or device)."""
     shifts = torch.arange(64, device=bits.device, dtype=torch.int64)
     flags = ((bits.unsqueeze(-1) >> shifts) & 1).to(torch.uint8)
-    return flags.reshape(*bits.shape[:-1], -1)[..., :ne]
+    return flags.reshape(*bits.shape[:-1], bits.shape[-1] * 64)[..., :ne]

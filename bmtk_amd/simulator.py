@@ -160,6 +160,13 @@ class Glif3Simulator:
             if t is not None:
                 t.delay_bits = self.delay_bits
         self.n_inputs = self.inp.n_rows if self.inp is not None else 0
+        # A table without a synapse delivers nothing and its arrays have no address to hand over: the kernels are
+        # not given it.  Events of input sources that project nowhere are still accepted (and checked).
+        if self.rec is not None and self.rec.nnz == 0:
+            self.rec = None
+        self.inp_without_synapses = self.inp is not None and self.inp.nnz == 0
+        if self.inp_without_synapses:
+            self.inp = None
         self.state = Glif3State.zeros(self.n, self.batch, asc_init=asc_init, u_init=u_init, device=self.dev)
         self.ring = torch.zeros(self.L, NREC, self.ne, device=self.dev)
         self.i_ext = None if i_ext is None else torch.as_tensor(np.asarray(i_ext, np.float32), device=self.dev)
@@ -281,7 +288,7 @@ class Glif3Simulator:
         The pull form of the inputs turns a step's events into bits, which hold an id
         once; the second and later occurrences are then listed apart
         (``in_repeat_ptr`` / ``in_repeat_events``) and delivered as events on top."""
-        if self.inp is None:
+        if self.inp is None and not self.inp_without_synapses:
             raise ValueError("no input synapse table")
         if torch.is_tensor(in_ptr):
             ok = bool((in_ptr[0] == 0) & (in_ptr[1:] >= in_ptr[:-1]).all() & (in_ptr[-1] == in_events.numel()))

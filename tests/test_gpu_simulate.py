@@ -652,6 +652,44 @@ def test_single_workgroup_form_with_more_spikes_and_events_than_its_lists_hold(e
         np.testing.assert_array_equal(outs["one"]["state"][k], outs["step"]["state"][k], err_msg=k)
 
 
+@pytest.mark.parametrize("n,empty", [(1, ""), (2, ""), (65, "rec"), (65, "inp"), (2049, "rec"), (2049, "rec inp")])
+def test_tiny_networks_and_tables_without_a_synapse(n, empty):
+    """One neuron (which has nobody to connect to), two, and networks whose recurrent or input table has rows but no
+    synapse at all (a population that projects nowhere): every driver runs them, calls of 0 steps included, with
+    the raster, state and ring of the launch-per-step driver, bit for bit (exact weights)."""
+    import torch
+    cfg = synthetic.small_glif3_network(n=n, n_in=20, steps=200, seed=3, in_w_scale=30.0, in_fanout=min(n, 5),
+                                        in_rate=100.0, p_conn=min(1.0, 8.0 / max(n, 2)), w_scale=5.0, max_delay=3)
+    for key in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = _integer_weights(cfg[key])
+        if key[:3] in empty.split():
+            indptr, indices, w, d, r = np.zeros_like(indptr), indices[:0], w[:0], d[:0], r[:0]
+        cfg[key] = (indptr, indices, w, d, r)
+    if n == 1:
+        assert cfg["rec_src"][1].size == 0
+    outs = {}
+    for name, kw in (("step", dict(resident=False)), ("one", dict(resident=True)),
+                     ("many", dict(resident=True, single_workgroup=False))):
+        sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=cfg["rec_src"],
+                             inp=cfg["inp_src"], i_ext=np.full(n, 400.0, np.float32), **kw)
+        sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+        bits = []
+        for steps in (0, 1, 37, 0, 100):
+            out = sim.run(steps, record_cap=1 << 14)
+            bits.append(out["bits"])
+            rec = sim.collect_record(out["record"], sort_scale=1.0)
+            assert rec["count"] == int(sim.raster(out["bits"]).sum()) and not rec["overflow"]
+        sim.check()
+        outs[name] = dict(raster=sim.raster(torch.cat(bits)).cpu().numpy(), state=sim.state.to_numpy(),
+                          ring=sim.ring.cpu().numpy())
+    assert outs["step"]["raster"].sum() >= 10 * min(n, 20)
+    for name in ("one", "many"):
+        for k in ("raster", "ring"):
+            np.testing.assert_array_equal(outs[name][k], outs["step"][k], err_msg="%s %s" % (name, k))
+        for k in outs["step"]["state"]:
+            np.testing.assert_array_equal(outs[name]["state"][k], outs["step"]["state"][k], err_msg="%s %s" % (name, k))
+
+
 def test_delay_offset_chosen_so_that_a_small_network_fits_one_workgroup():
     """450 cells whose delays are all 20 steps (bmtk's example networks at dt = 0.1 ms: 2 ms everywhere) need 21 ring
     slots, more than one workgroup's LDS holds for them; with the 19 steps all delays have in common taken off, two.
