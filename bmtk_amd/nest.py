@@ -261,8 +261,13 @@ def SetStatus(nodes, params, val=None):
     ids = _ids_of(nodes)
     plist = params if isinstance(params, (list, tuple)) else [params] * len(ids)
     for node, p in zip(ids, plist):
-        if _S.sim is not None and _S.kind[node - 1] not in (_RECORDER, _MULTIMETER):
-            raise NESTError("node parameters cannot change after the first Simulate")
+        if _S.sim is not None:
+            # what is read again at every Simulate may still change; the rest went into the device tables
+            later = {_RECORDER: None, _MULTIMETER: None, _NEURON: {"I_e"}, _CURRENT: {"amplitude_times", "amplitude_values"},
+                     _GENERATOR: {"spike_times", "origin", "precise_times", "allow_offgrid_times"}}.get(_S.kind[node - 1], set())
+            if later is not None and not set(p) <= later:
+                raise NESTError("after the first Simulate only {} of a {} can change, not {}".format(
+                    sorted(later), _S.kind[node - 1], sorted(set(p) - later)))
         _set_one(node, dict(p))
 
 
@@ -287,6 +292,8 @@ def Connect(pre, post, conn_spec=None, syn_spec=None):
     if _S.sim is not None:
         raise NESTError("connections cannot be created after the first Simulate")
     src, tgt = _ids_of(pre), _ids_of(post)
+    if len(src) == 0 and len(tgt) == 0:
+        return  # nothing to connect (a batch of edges that turned out empty)
     rule = conn_spec if isinstance(conn_spec, str) else (conn_spec or {}).get("rule", "all_to_all")
     kinds_src = {_S.kind[i - 1] for i in src}
     kinds_tgt = {_S.kind[i - 1] for i in tgt}
@@ -403,13 +410,19 @@ def _build():
                   e_l=par[_PAR["E_L"]].copy())
 
 
+def _constant_current():
+    """The neurons' own constant input current I_e (pA; glif_psc adds it to the step currents and the after-spike
+    currents in every update), as set at Create or by SetStatus since."""
+    return np.array([float(_S.params[i - 1].get("I_e", 0.0)) for i in _S.sim["neuron_ids"]], np.float32)
+
+
 def _current_at(step):
-    """Per-neuron external current (pA) used in update step `step`: a
-    step_current_generator's amplitude set at time T acts from the step that
+    """Per-neuron external current (pA) used in update step `step`: I_e plus what the step current generators
+    supply -- a step_current_generator's amplitude set at time T acts from the step that
     starts at T + delay (its connection delay is one resolution, as bmtk sets it)."""
     s = _S.sim
     dt = _S.status["resolution"]
-    cur = np.zeros(s["neuron_ids"].size, np.float32)
+    cur = _constant_current()
     t_ms = step * dt
     for g, ids in _S.cur_links:
         p = _S.params[g - 1]
@@ -467,6 +480,9 @@ def Simulate(t_ms):
     want_record = bool(_S.rec_links)
     senders, times = [], []
     mm_rows = {m: ([], [], []) for m, _ in _S.mm_links}
+    if not _S.cur_links:
+        i_e = _constant_current()
+        sim.i_ext = torch.as_tensor(i_e, device=sim.dev) if i_e.any() else None
     for a, b in zip(bounds[:-1], bounds[1:]):
         if _S.cur_links:
             sim.i_ext = torch.as_tensor(_current_at(a), device=sim.dev)

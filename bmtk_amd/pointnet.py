@@ -110,7 +110,9 @@ class PointSimulator:
         self.n_steps = int(round(self.tstop / self.dt))
         self.output = {}
         self._trains = [None] * network.n_inputs
-        self._i_ext = np.zeros(network.n, np.float64)
+        # the cells' own constant current I_e (per parameter class); current clamps add to it
+        i_e = getattr(network, "i_e", None)
+        self._i_ext = np.zeros(network.n) if i_e is None else np.asarray(i_e, np.float64)[network.class_id]
         self._clamps = []
         self._device, self._resident = device, resident
         self.spikes = None
@@ -244,7 +246,7 @@ class PointSimulator:
             marks.update(first_step(t) for t in times)
         marks = sorted(marks)
         for a, b in zip(marks[:-1], marks[1:]):
-            cur = np.zeros(self.net.n, np.float32)
+            cur = self._i_ext.astype(np.float32)
             for ids, times, values in self._clamps:
                 on = [v for t, v in zip(times, values) if first_step(t) <= a]
                 if on:

@@ -211,7 +211,8 @@ def node_parameter_classes(pop, models_dir, unsupported="raise"):
     """One GLIF3 parameter class per node type of a population.
 
     -> (par fp64 [NPARAM, classes], asc_init [2, classes], u_init [classes], class_id int32 [nodes] ordered by
-    node id, supported bool [classes], type ids [classes]).
+    node id, supported bool [classes], type ids [classes], i_e fp64 [classes]: the cells' constant input current
+    ``I_e`` in pA, which is no row of the parameter table but part of the external current).
 
     ``nest:glif_psc`` with ready NEST-unit parameters is taken as is; ``nest:glif_*`` templates with an Allen
     cell-types file (``"type": "GLIF"``) are converted first (sonata_adaptors.py:155-167).  Any other point model
@@ -244,7 +245,8 @@ def node_parameter_classes(pop, models_dir, unsupported="raise"):
     class_of_type = {t: i for i, t in enumerate(type_ids)}
     class_id = np.array([class_of_type[t] for t in pop.node_type_ids[order]], np.int32)
     assert par.shape[0] == NPARAM
-    return par, asc_init, u_init, class_id, np.array(supported), type_ids
+    i_e = np.array([float(c.get("I_e", 0.0)) for c in cells], np.float64)
+    return par, asc_init, u_init, class_id, np.array(supported), type_ids, i_e
 
 
 # ----------------------------------------------------------------------------------------------------------------
@@ -659,8 +661,9 @@ class PointNetwork:
     """
 
     def __init__(self, population, n, par, asc_init, u_init, class_id, supported, rec_edges, inp_edges, virtual,
-                 n_inputs):
+                 n_inputs, i_e=None):
         self.population, self.n = population, n
+        self.i_e = np.zeros(par.shape[1]) if i_e is None else i_e   # constant input current per class, pA
         self.par, self.asc_init, self.u_init, self.class_id, self.supported = par, asc_init, u_init, class_id, supported
         self.rec_edges, self.inp_edges = rec_edges, inp_edges  # (src, tgt, w, delay steps, receptor) or None
         self.virtual, self.n_inputs = virtual, n_inputs
@@ -707,7 +710,7 @@ def load_point_network(config, dt=None, unsupported="raise"):
     pop = real[0]
     if not np.array_equal(np.sort(pop.node_ids), np.arange(len(pop))):
         raise NotImplementedError("node ids of {} must be 0..n-1".format(pop.name))
-    par, asc_init, u_init, class_id, supported, _ = node_parameter_classes(
+    par, asc_init, u_init, class_id, supported, _, i_e = node_parameter_classes(
         pop, comp.get("point_neuron_models_dir", "."), unsupported)
     silent = ~supported[class_id]
     rec, inp, virtual, n_inputs = [], [], {}, 0
@@ -736,4 +739,4 @@ def load_point_network(config, dt=None, unsupported="raise"):
         return tuple(np.concatenate([p[i] for p in parts]) for i in range(5)) if parts else None
 
     return PointNetwork(pop.name, len(pop), par, asc_init, u_init, class_id, supported, cat(rec), cat(inp), virtual,
-                        n_inputs)
+                        n_inputs, i_e)

@@ -399,6 +399,21 @@ def _bare_simulator(dt=0.1, tstop=3500.0, n=120):
     return pointnet.PointSimulator(net_, dt, tstop)
 
 
+def test_constant_current_of_the_cell_models_is_the_base_of_every_segment():
+    """A cell model's I_e (pA, glif_psc's constant input current) is not a row of the parameter table: it is the
+    external current on which the current clamps are stacked."""
+    from types import SimpleNamespace
+    from bmtk_amd import pointnet
+    net_ = SimpleNamespace(n=6, n_inputs=0, population="cortex", virtual={}, i_e=np.array([0.0, 25.0]),
+                           class_id=np.array([0, 1, 1, 0, 1, 0], np.int32))
+    sim = pointnet.PointSimulator(net_, 0.5, 100.0)
+    sim.add_current_clamp({"input_type": "current_clamp", "module": "IClamp", "node_set": [1, 3], "amp": 100.0,
+                           "delay": 20.0, "duration": 30.0})
+    segs = [(a, b, cur.tolist()) for a, b, cur in sim._segments()]
+    assert segs == [(0, 41, [0.0, 25.0, 25.0, 0.0, 25.0, 0.0]), (41, 101, [0.0, 125.0, 25.0, 100.0, 25.0, 0.0]),
+                    (101, 200, [0.0, 25.0, 25.0, 0.0, 25.0, 0.0])]
+
+
 def test_current_clamp_amplitude_lists():
     """The amplitude times/values bmtk's IClamp module hands to a step_current_generator
     (bmtk/simulator/pointnet/modules/iclamp.py:13-39) for the inputs of examples/point_iclamp."""
