@@ -411,8 +411,8 @@ def _build():
 
 
 def _constant_current():
-    """The neurons' own constant input current I_e (pA; glif_psc adds it to the step currents and the after-spike
-    currents in every update), as set at Create or by SetStatus since."""
+    """A constant input current I_e (pA) per neuron, the parameter NEST's current-based point neurons carry, as
+    given at Create or by SetStatus since: it is added to the step currents of every update."""
     return np.array([float(_S.params[i - 1].get("I_e", 0.0)) for i in _S.sim["neuron_ids"]], np.float32)
 
 

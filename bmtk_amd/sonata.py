@@ -211,8 +211,9 @@ def node_parameter_classes(pop, models_dir, unsupported="raise"):
     """One GLIF3 parameter class per node type of a population.
 
     -> (par fp64 [NPARAM, classes], asc_init [2, classes], u_init [classes], class_id int32 [nodes] ordered by
-    node id, supported bool [classes], type ids [classes], i_e fp64 [classes]: the cells' constant input current
-    ``I_e`` in pA, which is no row of the parameter table but part of the external current).
+    node id, supported bool [classes], type ids [classes], i_e fp64 [classes]: a constant input current ``I_e``
+    in pA where a cell-model file gives one, which is no row of the parameter table but part of the external
+    current).
 
     ``nest:glif_psc`` with ready NEST-unit parameters is taken as is; ``nest:glif_*`` templates with an Allen
     cell-types file (``"type": "GLIF"``) are converted first (sonata_adaptors.py:155-167).  Any other point model

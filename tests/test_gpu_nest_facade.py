@@ -234,7 +234,7 @@ def test_multimeter_records_membrane_potential(golden_dir, tmp_path):
 
 
 def test_constant_input_current_I_e(golden_dir, tmp_path):
-    """glif_psc's own constant current I_e (pA), given at Create or set between two Simulate calls.  Below threshold
+    """A neuron's constant input current I_e (pA), given at Create or set between two Simulate calls.  Below threshold
     the potential settles at E_L + I_e / g (closed form: pA / nS = mV), which fixes the scale; above it the spike
     times follow the fp64 oracle driven with the same current, the change taking effect with the call after it."""
     from oracle import glif3_oracle as orc

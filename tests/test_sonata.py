@@ -400,7 +400,7 @@ def _bare_simulator(dt=0.1, tstop=3500.0, n=120):
 
 
 def test_constant_current_of_the_cell_models_is_the_base_of_every_segment():
-    """A cell model's I_e (pA, glif_psc's constant input current) is not a row of the parameter table: it is the
+    """A cell model's I_e (pA, a constant input current) is not a row of the parameter table: it is the
     external current on which the current clamps are stacked."""
     from types import SimpleNamespace
     from bmtk_amd import pointnet
