@@ -64,7 +64,9 @@ def test_every_driver_equals_the_oracle(seed):
     for kw in drivers:
         sim = Glif3Simulator(n, cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=rec, inp=inp,
                              i_ext=cfg["i_ext"], **kw)
-        assert sim.delay_offset == (cfg["extra"] if (has_rec or has_inp) and cfg["extra"] else 0)
+        # delays beyond the ring's reach: all that the delays have in common is taken off
+        least = min([int(t[3].min()) for t in (rec, inp) if t is not None and t[3].size] or [1])
+        assert sim.delay_offset == (least - 1 if cfg["extra"] else 0)
         if kw.get("resident"):
             assert (sim.res_groups == 1) == (kw.get("single_workgroup", True) or n <= 64)
         if has_inp:
