@@ -79,3 +79,65 @@ def test_every_driver_equals_the_oracle(seed):
         got = sim.state.to_numpy()
         for k in ("V", "asc", "y2", "ref"):
             np.testing.assert_array_equal(got[k], st[k], err_msg="%s %s" % (k, kw))
+
+
+def _larger_case(seed):
+    rng = np.random.default_rng(5000 + seed)
+    n = int(rng.choice([1025, 1500, 2000, 3333, 5000, 9000]))
+    n_in = int(rng.choice([0, 50, 400]))
+    max_delay = int(rng.choice([1, 3, 6]))
+    extra = int(rng.choice([0, 0, 2, 5, 70]))
+    classes = int(rng.choice([0, 0, 5])) or None
+    cfg = synthetic.small_glif3_network(n=n, n_in=n_in, steps=120, seed=seed, p_conn=float(rng.choice([0.0, 10.0 / n, 60.0 / n])),
+                                        in_rate=float(rng.choice([20.0, 300.0])), in_fanout=30, max_delay=max_delay,
+                                        n_classes=classes, batch=1, w_scale=6.0, in_w_scale=40.0)
+    for key in ("rec_src", "inp_src"):
+        indptr, indices, w, d, r = cfg[key]
+        cfg[key] = (indptr, indices, (np.round(w * 4.0) / 4.0 + np.sign(w) * 0.25).astype(np.float32),
+                    d.astype(np.int32) + extra, r)
+    cfg["extra"] = extra
+    # a constant current: spread out, or the same for most cells, which then fire in volleys
+    amp = float(rng.choice([300.0, 600.0, 2500.0]))
+    in_step = rng.random() < 0.4
+    cfg["i_ext"] = (np.where(rng.random(n) < 0.6, amp, rng.uniform(0.0, 300.0, n)) if in_step
+                    else rng.uniform(0.0, amp, n)).astype(np.float32)
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_many_workgroups_with_volleys_and_delay_offsets(seed):
+    """Networks of 1,025 to 9,000 neurons (several resident workgroups, spans of 64 and more), from silent stretches to
+    volleys of a thousand spikes in a step, with the part all delays have in common taken off automatically or as asked
+    (runs with slack between the workgroups): raster and state of the launch-per-step driver and of the resident
+    kernel, reading lists of fired neurons or ballots, equal the fp32 oracle's bit for bit."""
+    cfg = _larger_case(seed)
+    n, steps = cfg["n"], cfg["steps"]
+    rec = cfg["rec_src"] if cfg["rec_src"][1].size else None
+    inp = cfg["inp_src"] if cfg["n_in"] > 0 and cfg["inp_src"][1].size else None
+    L = int(max([1] + [int(t[3].max()) for t in (rec, inp) if t is not None])) + 1
+    orc.set_threads(8)
+    prop = orc.precompute(cfg["par"], cfg["h"])
+    st = orc.new_state(n, 1, np.float32)
+    ring = np.zeros((L, 4, n), np.float32)
+    want = orc.simulate(st, prop, cfg["h"], steps, class_id=cfg["class_id"], ring=ring, rec=rec, inp=inp,
+                        in_ptr=cfg["in_ptr"] if inp is not None else None,
+                        in_events=cfg["in_events"] if inp is not None else None, i_ext=cfg["i_ext"], raster=True)
+    assert want["count"] > 0
+    offsets = ["auto"] + ([cfg["extra"]] if cfg["extra"] and (rec is not None or inp is not None) else [])
+    for off in offsets:
+        for kw in (dict(resident=False), dict(resident=True), dict(resident=True, fired_lists=False)):
+            sim = Glif3Simulator(n, cfg["par"], cfg["h"], class_id=cfg["class_id"], rec=rec, inp=inp, i_ext=cfg["i_ext"],
+                                 delay_offset=off, **kw)
+            if kw["resident"]:
+                assert sim.res_groups > 1
+            if inp is not None:
+                sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+            a = sim.run(50)
+            b = sim.run(steps - 50)
+            sim.check()
+            ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
+            tag = "delay offset %s -> %d, %s" % (off, sim.delay_offset, kw)
+            np.testing.assert_array_equal(ras, want["raster"], err_msg=tag)
+            got = sim.state.to_numpy()
+            for k in ("V", "asc", "y2", "ref"):
+                np.testing.assert_array_equal(got[k], st[k], err_msg="%s %s" % (k, tag))
