@@ -366,7 +366,10 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_gl
                                 }
                             }
                         }
-                        p += kF;
+                        // a lane whose row segment has ended stays at its end: with p <= p1 at every fetch no lane
+                        // reads a record at or beyond p1 + 2*kF, which is what BMTK_BLOCKED_PAD covers, however much
+                        // longer the other rows of the visit are
+                        p = min(p + kF, p1);
                     };
                     while (true) {
                         work(cur, nxt);
@@ -826,6 +829,24 @@ extern "C" int bmtk_csr_propagate_bwd_blocked(const int32_t *blk_indptr, const b
     rc = blocked_launch(a, q, pl, false, (hipStream_t)stream);
     if (rc != BMTK_OK) return rc;
     BMTK_CHECK_LAUNCH("csr_propagate_bwd_blocked");
+    return BMTK_OK;
+}
+
+extern "C" int bmtk_csr_propagate_bwd_blocked_plan(int64_t n_neurons, int32_t batch, int32_t *plan_host)
+{
+    BMTK_REQUIRE(plan_host != nullptr, "csr_propagate_bwd_blocked_plan: plan_host is null");
+    BMTK_REQUIRE(n_neurons > 0 && n_neurons < (1ll << 24) && batch > 0 && batch % 4 == 0 && batch <= kWave,
+                 "csr_propagate_bwd_blocked_plan: n_neurons must lie in 1..2^24-1, batch be a multiple of 4 up to 64");
+    bmtk_glif3_bwd a{};
+    a.n_neurons = n_neurons;
+    a.batch = batch;
+    BlockedPlan pl{};
+    const int rc = blocked_plan(a, pl);
+    if (rc != BMTK_OK) return rc;
+    plan_host[0] = (int32_t)pl.grid;
+    plan_host[1] = pl.rows_cu;
+    plan_host[2] = pl.sweeps;
+    plan_host[3] = pl.gpw;
     return BMTK_OK;
 }
 

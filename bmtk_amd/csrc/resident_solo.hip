@@ -74,7 +74,7 @@ constexpr int kWalkRole = 0, kFetchRole = 1, kStoreRole = 2;  // what a wavefron
 constexpr int kEvCap = 128;                  // input events of a step that become items; further ones are read in place
 constexpr int kFiredCap = 512;               // fired neurons of a step that become items; further ones: overflow ballot
 constexpr int kNearSteps = 4;                // the ballots of so many steps stay in LDS (delay offsets below that)
-constexpr size_t kSoloStaticLds = 1024;      // the kernel's static LDS, rounded up
+constexpr size_t kSoloStaticLds = 2048;      // bound on the kernel's static LDS (1076 bytes and the compiler's padding)
 constexpr unsigned kNoSample = 0xFFFFFFFFu;  // a probe cell nobody writes (a NaN no update produces)
 
 struct Solo {

@@ -10,7 +10,7 @@ constexpr size_t kResLdsBytes = 160u * 1024u;                   // LDS of one gf
 constexpr size_t kResLdsExtra = kActCap * sizeof(int) + 256u;   // the list plus the kernel's static LDS (rounded up)
 // the single-workgroup form, with span elements: spike offsets and probed potentials of two steps, the items (rows to
 // walk) of two steps, its static LDS (rounded up)
-constexpr size_t solo_lds_extra(int span) { return (size_t)span * 4u * sizeof(float) + 10240u + 1024u; }
+constexpr size_t solo_lds_extra(int span) { return (size_t)span * 4u * sizeof(float) + 10240u + 2048u; }
 
 // Whole run as one cooperative launch with state in registers and the ring in
 // LDS (resident.hip).  Arguments have been validated by the caller.

@@ -511,7 +511,8 @@ def Simulate(t_ms):
             # interpolated threshold crossing (step + fraction) * resolution; ordered by time on the device
             rec = sim.collect_record(out["record"], sort_scale=dt)
             if rec["overflow"]:
-                raise NESTError("more than {} spikes in one Simulate call; simulate in shorter pieces".format(cap))
+                raise NESTError("spike record overflow in one Simulate call ({}); simulate in shorter pieces".format(
+                    sim.overflow_message(rec)))
             rec_time, rec_elem = sim.to_host(rec["time"], rec["elem"])
             times.append(rec_time)
             senders.append(s["neuron_ids"][rec_elem])

@@ -399,6 +399,17 @@ def csr_propagate_bwd_blocked(blk, n_blocks, lam_ring, n, batch, step, gz_parts=
     return gz_parts
 
 
+def blocked_plan(n, batch):
+    """Launch geometry of the blocked transposed propagation for ``n`` neurons at ``batch`` on the current device:
+    dict(grid, rows_per_workgroup, sweeps, groups_per_wavefront) (``bmtk_csr_propagate_bwd_blocked_plan``)."""
+    import ctypes
+    lib = _lib.load()
+    _dev()
+    plan = (ctypes.c_int32 * 4)()
+    _lib.check(lib.bmtk_csr_propagate_bwd_blocked_plan(n, batch, ctypes.cast(plan, ctypes.c_void_p)))
+    return dict(grid=plan[0], rows_per_workgroup=plan[1], sweeps=plan[2], groups_per_wavefront=plan[3])
+
+
 def csr_propagate_auto(active, n_active, zbits, n_src, table_src, table_tgt, ring, n_tgt, batch, step,
                        scatter_max_active=None, max_active=None):
     """Delivery with the form chosen on the device (no host synchronisation): the event-driven scatter up to

@@ -300,7 +300,7 @@ class PointSimulator:
             # node) on the device.  The pieces follow one another in time, so their order is the run's.
             r = sim.collect_record(out["record"], sort_scale=self.dt)
             if r["overflow"]:
-                raise RuntimeError("spike record overflow: {} spikes, room for {}".format(r["count"], cap))
+                raise RuntimeError("spike record overflow: " + sim.overflow_message(r))
             r_time, r_elem = sim.to_host(r["time"], r["elem"])
             elems.append(r_elem.astype(np.int64))
             times.append(r_time)

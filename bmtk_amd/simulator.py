@@ -22,7 +22,7 @@ RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static 
 # the single-workgroup form: per element the spike offsets and probed potentials of two steps (SOLO_LDS_PER_ELEMENT);
 # the items (rows to walk) of two steps and its static LDS (SOLO_LDS_EXTRA)
 SOLO_LDS_PER_ELEMENT = 4 * 4
-SOLO_LDS_EXTRA = 10240 + 1024
+SOLO_LDS_EXTRA = 10240 + 2048
 RECORD_WAYS = 64                # lists a large spike record is split into (bmtk_glif3_sim.spike_ways)
 
 
@@ -201,6 +201,15 @@ class Glif3Simulator:
         self.pull_inp_table = self.pull_inp_syn = self.pull_inp_work = self.in_hist = None
         can_pull = (self.rec is not None and not self.res_span and self.delay_offset == 0
                     and self.L * ((self.n + 31) // 32) * 4 <= PULL_MAP_BYTES)
+        # the pull form sums in 64-bit fixed point: weights must be finite and below 2^31 in size
+        def fixed_point_ok(t):
+            w = t.weights
+            return not w.numel() or bool(torch.isfinite(w).all() & (w.abs().max() < 2.0 ** 31))
+        if can_pull and (pull is True or (pull == "auto" and self.batch >= 8)):
+            if not (fixed_point_ok(self.rec) and (self.inp is None or fixed_point_ok(self.inp))):
+                if pull is True:
+                    raise ValueError("the pull form needs finite weights smaller than 2^31 in size")
+                can_pull = False   # the event-driven form propagates IEEE values as they are
         if pull is True and not can_pull:
             raise ValueError("the pull form needs a recurrent table, launch-per-step mode, delay_offset 0 and "
                              "ring_slots * n_neurons / 8 bytes of LDS (at most 40 KB)")
@@ -445,8 +454,12 @@ class Glif3Simulator:
 
     def collect_record(self, record, sort_scale=None):
         """The spike record of a ``run(..., record_cap=...)`` as one list: dict(step int32[], elem int32[], frac
-        float32[], count int, overflow bool), unordered within a step.  ``count`` is the number of spikes the run
-        produced; ``overflow`` says that some of them found no room (then the lists are incomplete).
+        float32[], count int, overflow bool, ways, way_cap, fullest), unordered within a step.  ``count`` is the
+        number of spikes the run produced; ``overflow`` says that some of them found no room (then the lists are
+        incomplete).  A record kept as ``ways`` lists overflows as soon as ONE list does -- a workgroup appends to
+        its own list of ``way_cap`` = cap / ways entries only, so activity concentrated in the neurons of a few
+        workgroups can overflow while ``count`` is far below the record's total size; ``fullest`` is the largest
+        count of a single list (``overflow_message`` words it).
         With ``sort_scale`` (the resolution in ms) the list comes back ordered by spike time
         (step + frac) * sort_scale, ties by element -- sorted on the device, where two million spikes take
         milliseconds instead of the second a host sort takes -- and ``time`` (float64, ms) is added.
@@ -466,13 +479,23 @@ class Glif3Simulator:
             first = torch.arange(ways, dtype=torch.int64, device=dev) * way_cap - (torch.cumsum(filled, 0) - filled)
             keep = torch.arange(sum(stored), dtype=torch.int64, device=dev) + torch.repeat_interleave(first, filled)
         out = dict(step=record["step"][keep], elem=record["elem"][keep], frac=record["frac"][keep],
-                   count=int(counts.sum()), overflow=bool((counts > way_cap).any()))
+                   count=int(counts.sum()), overflow=bool((counts > way_cap).any()), ways=ways, way_cap=way_cap,
+                   fullest=int(counts.max()))
         if sort_scale is not None:
             t = (out["step"].to(torch.float64) + out["frac"].to(torch.float64)) * float(sort_scale)
             by_elem = torch.argsort(out["elem"], stable=True)
             order = by_elem[torch.argsort(t[by_elem], stable=True)]
             out.update(step=out["step"][order], elem=out["elem"][order], frac=out["frac"][order], time=t[order])
         return out
+
+    @staticmethod
+    def overflow_message(rec):
+        """What a caller reports when ``collect_record`` came back with ``overflow``: the capacity that ran out is
+        that of one list, not of the record."""
+        if rec["ways"] == 1:
+            return "{} spikes, room for {}".format(rec["count"], rec["way_cap"])
+        return ("{} spikes in all; the record is kept as {} lists of {} entries (one per group of workgroups) and "
+                "the fullest list was asked to hold {}".format(rec["count"], rec["ways"], rec["way_cap"], rec["fullest"]))
 
     def to_host(self, *tensors):
         """Device tensors -> NumPy arrays through pinned host memory (torch keeps freed pinned blocks for reuse): a

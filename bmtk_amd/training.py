@@ -65,7 +65,7 @@ class Glif3Bptt:
         self.lam_y2 = torch.zeros(NREC, ne, device=dev)
         self.lam_ring = torch.zeros(sim.L, NREC, ne, device=dev)
         self.d_rec_w = torch.zeros(sim.rec.nnz, device=dev) if sim.rec is not None else None
-        can_block = sim.rec is not None and sim.batch % 4 == 0 and sim.batch <= 64 and sim.L * NREC * ne < (1 << 32)
+        can_block = sim.rec is not None and sim.batch % 4 == 0 and sim.batch <= 64 and sim.L * NREC * ne < (1 << 30)
         if blocked is None:
             blocked = can_block and sim.L * NREC * ne * 4 > self.BLOCKED_MIN_RING_BYTES
         elif blocked and not can_block:

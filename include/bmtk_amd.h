@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 16
+#define BMTK_AMD_ABI_VERSION 17
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -471,6 +471,13 @@ int bmtk_csr_propagate_bwd(const int32_t *indptr, const bmtk_synapse *packed, in
 int bmtk_csr_propagate_bwd_blocked(const int32_t *blk_indptr, const bmtk_synapse *blk_packed, int32_t blk_count,
                                    int64_t n_neurons, int32_t batch, const float *lam_ring, int32_t L, int64_t step,
                                    float *gz_parts, void *stream);
+
+/* The launch geometry the blocked form takes for a network on the current device, for callers and tests that want
+ * to know which of its paths a size exercises: plan_host[0] = workgroups (one per compute unit, workgroup b on XCD
+ * b mod 8), [1] = source rows per workgroup, [2] = sweeps over them (a sweep holds at most 16 wavefronts x 8 row
+ * groups x 64*4/batch rows in LDS), [3] = row groups per wavefront and sweep.  plan_host is a HOST pointer to four
+ * int32. */
+int bmtk_csr_propagate_bwd_blocked_plan(int64_t n_neurons, int32_t batch, int32_t *plan_host);
 
 /* Number of spikes of every element over n_steps rows of spike bits: counts[e] (int32). */
 int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_steps, int64_t ne, int32_t *counts,
