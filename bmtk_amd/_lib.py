@@ -32,6 +32,8 @@ class Glif3Sim(C.Structure):
         ("pull_inp_indptr", c_void_p), ("pull_inp_packed", c_void_p), ("pull_inp_syn", c_void_p),
         ("pull_inp_work", c_void_p), ("in_hist", c_void_p), ("in_hist_stride", c_int64),
         ("in_repeat_ptr", c_void_p), ("in_repeat_events", c_void_p),
+        ("fuse_indptr", c_void_p), ("fuse_packed", c_void_p), ("fuse_any", c_void_p),
+        ("fuse_hist_stride", c_int64), ("fuse_in_base", c_int64), ("fuse_shift", c_int32), ("fuse_wg_per_cu", c_int32),
         ("spike_bits", c_void_p), ("spike_bits_stride", c_int64),
         ("save_v", c_void_p), ("save_flags", c_void_p),
         ("probe_col", c_void_p), ("probe_v", c_void_p), ("probe_stride", c_int64), ("probe_every", c_int32),
@@ -58,7 +60,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 17  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 18  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {

@@ -41,4 +41,32 @@ __device__ __forceinline__ unsigned long long source_mask(const uint64_t *__rest
     return m;
 }
 
+// walk one row of a packed table, four 64-synapse chunks in flight at a time
+__device__ __forceinline__ void deliver_row_packed(const int32_t *__restrict__ indptr,
+                                                   const bmtk_synapse *__restrict__ syn, int j, int b, int batch,
+                                                   float *__restrict__ ring, int L, int slot0, int64_t ne,
+                                                   int idx_bits)
+{
+    const unsigned idx_mask = (1u << idx_bits) - 1u;
+    const int p0 = indptr[j], p1 = indptr[j + 1];
+    if (p1 <= p0) return;
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(syn);
+    for (int base = p0 + lane_id(); base < p1; base += 4 * kWave) {
+        uint2 s[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s[u] = rows[min(base + u * kWave, p1 - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (base + u * kWave < p1) {
+                const unsigned tdr = s[u].x;
+                int slot = slot0 + (int)(tdr >> (idx_bits + 2));
+                slot = slot >= L ? slot - L : slot;
+                const int r = (tdr >> idx_bits) & 3;
+                const int64_t i = tdr & idx_mask;
+                atomicAdd(ring + ((int64_t)(slot * GLIF3_NREC + r) * ne + i * batch + b), __uint_as_float(s[u].y));
+            }
+        }
+    }
+}
+
 }  // namespace bmtk

@@ -21,6 +21,7 @@
 
 #include "common.hpp"
 #include "propagate.hpp"
+#include "pull_common.hpp"
 
 namespace bmtk {
 
@@ -47,74 +48,6 @@ constexpr int kPullBlock = 1024;  // 16 wavefronts share one staged activity map
 // per wavefront: 4 x 64 accumulators of 8 bytes and a stage of 64 entries of 8 bytes
 constexpr size_t kPullAccBytes = (size_t)(kPullBlock / kWave) * (GLIF3_NREC + 1) * kWave * sizeof(unsigned long long);
 constexpr size_t kPullLdsMax = 80u * 1024u;  // two workgroups per compute unit: each may take half of the 160 KB of LDS
-
-// fp32 -> Q31.32 two's complement.  The size |w| is split with floor(): the integer part, and what is left, which
-// lies in [0, 1) and is exact (for a negative w, w - floor(w) = w + 1 would round); times 2^32 it is an integer
-// below 2^32 up to the bits under 2^-32, which the conversion drops.  The sign is applied to the integer.
-__device__ __forceinline__ unsigned long long to_fixed(float w)
-{
-    const float size = fabsf(w);
-    const float whole = floorf(size);
-    const unsigned lo = (unsigned)((size - whole) * 4294967296.0f);
-    const unsigned long long v = ((unsigned long long)(unsigned)whole << 32) | lo;
-    return w < 0.0f ? 0ull - v : v;
-}
-
-__device__ __forceinline__ float from_fixed(unsigned long long v)
-{
-    return (float)((double)(long long)v * (1.0 / 4294967296.0));
-}
-
-// One block of a row's synapse stream: positions [base, min(base + kPullChunks*64, p1)) of the packed table.
-constexpr int kPullChunks = 4;  // 64-synapse chunks per block
-struct PullBlock {
-    int64_t row;  // >= n_tgt: past the end
-    int base, p1;
-    bool last;    // last block of its row: the sums are stored after it
-};
-
-// The rows a wavefront owns (first, first + stride, ...) as a stream of blocks.  The bounds of the row after the
-// current one are fetched a row ahead.  Everything here is the same in all lanes (scalar registers and loads).
-struct PullCursor {
-    const int32_t *__restrict__ indptr;
-    int64_t n_tgt, stride, row;
-    int q, p1, np0, np1;
-
-    __device__ __forceinline__ void start(const int32_t *ip, int64_t n, int64_t first, int64_t step)
-    {
-        indptr = ip;
-        n_tgt = n;
-        stride = step;
-        row = first;
-        q = p1 = np0 = np1 = 0;
-        if (row < n_tgt) {
-            q = indptr[row];
-            p1 = indptr[row + 1];
-        }
-        if (row + stride < n_tgt) {
-            np0 = indptr[row + stride];
-            np1 = indptr[row + stride + 1];
-        }
-    }
-    __device__ __forceinline__ PullBlock next()
-    {
-        PullBlock b{row, q, p1, false};
-        if (row < n_tgt) {
-            q += kPullChunks * kWave;
-            if (q >= p1) {
-                b.last = true;
-                row += stride;
-                q = np0;
-                p1 = np1;
-                if (row + stride < n_tgt) {
-                    np0 = indptr[row + stride];
-                    np1 = indptr[row + stride + 1];
-                }
-            }
-        }
-        return b;
-    }
-};
 
 // kWords64: batch == 64, so that the trial mask of source j is word j of a history row; otherwise the general
 // bit-field read (any batch, tiles of 64 trials over blockIdx.y).

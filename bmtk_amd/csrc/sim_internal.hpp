@@ -20,4 +20,7 @@ int simulate_resident(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, h
 // whole synapse rows walked by a wavefront (resident_solo.hip).
 int simulate_resident_solo(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream);
 
+// Batched runs, one launch per step with the pull of a step's arrivals and the update fused (simulate_fused.hip).
+int simulate_fused(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipStream_t stream);
+
 }  // namespace bmtk

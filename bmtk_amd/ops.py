@@ -271,6 +271,33 @@ class SynapseTable:
                             self.delays[order].contiguous(), self.receptors[order].contiguous(), n_rows=n_cols,
                             max_row=int(counts.max().item()) if counts.numel() else 0)
 
+    @staticmethod
+    def joined_by_target(rec, inp, n_tgt, in_base):
+        """The joint target-major table of the fused batched driver (``bmtk_glif3_sim.fuse_*`` of
+        include/bmtk_amd.h) from the source-major recurrent table ``rec`` and input table ``inp`` (either may be
+        None): row = target neuron, index field = source in the joint space -- neuron j is j, input source k is
+        ``in_base + k``.  Rows keep the recurrent synapses first, each part in (source, position) order."""
+        parts = []
+        for t, base in ((rec, 0), (inp, in_base)):
+            if t is None or t.nnz == 0:
+                continue
+            dev = t.indices.device
+            rows = torch.repeat_interleave(torch.arange(t.n_rows, device=dev, dtype=torch.int64),
+                                           (t.indptr[1:] - t.indptr[:-1]).long()) + base
+            parts.append((t.indices.long(), rows, t.weights, t.delays, t.receptors))
+        if not parts:
+            raise ValueError("no synapses to join")
+        tgt = torch.cat([p[0] for p in parts])
+        order = torch.sort(tgt, stable=True).indices
+        counts = torch.bincount(tgt, minlength=n_tgt)
+        indptr = torch.zeros(n_tgt + 1, dtype=torch.int32, device=tgt.device)
+        indptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+
+        def col(k, dtype):
+            return torch.cat([p[k] for p in parts])[order].to(dtype).contiguous()
+        return SynapseTable(indptr, col(1, torch.int32), col(2, torch.float32), col(3, torch.uint8),
+                            col(4, torch.uint8), n_rows=n_tgt, max_row=int(counts.max().item()))
+
     def blocked(self, n_cols, n_blocks):
         """The table regrouped by column range for the transposed propagation of the backward pass
         (``bmtk_glif3_bwd.blk_*`` of include/bmtk_amd.h): columns are cut into ``n_blocks`` equal ranges and the

@@ -16,6 +16,9 @@ from .ops import Glif3State, SpikeCompactor, SynapseTable, _dev, _p, _stream, gl
 
 
 PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what is left of 80 KB beside its accumulators
+FUSE_LDS_BYTES = 80 * 1024      # LDS of one workgroup of the fused batched driver (kFuseLdsMax of csrc/simulate_fused.hip)
+FUSE_WAVES = 16                 # wavefronts of one of its workgroups (kFuseWaves)
+FUSE_BATCHES = (8, 16, 32, 64)  # lane = trial, whole bytes of spike bits per neuron
 RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
 RES_ACT_ENTRIES = 8192          # active-row list of the resident kernel (kActCap of csrc/resident.hip), 4 B each
 RES_LDS_EXTRA = RES_ACT_ENTRIES * 4 + 256   # the list plus the kernel's static LDS (rounded up)
@@ -65,6 +68,13 @@ class Glif3Simulator:
                 as a short list beside its ballots, and the others read the lists instead of expanding the whole
                 network's ballots (steps in which a list does not suffice are read from the ballots); False: always
                 from the ballots.  Same results either way.
+    fused       launch-per-step mode, batch 8, 16, 32 or 64, delay_offset 0: one launch per step in which a
+                wavefront sums what arrives at a neuron -- over recurrent and input synapses, from a joint
+                target-major table and a joint history of spike and input-event bits -- and advances the neuron's
+                trials, lane = trial; no arrival sum passes through device memory.  "auto": whenever ``pull`` would
+                apply and the batch is one of those; takes any number of sources (above what the activity map in
+                LDS holds, one bit of the map stands for 2, 4, ... sources).  False: the pull form as separate
+                launches (below).  ``ring`` then holds only the few input ids repeated within a step.
     pull        launch-per-step mode only: sum the recurrent arrivals of a step in one pass over a target-major
                 copy of the table from the spike-bit history, instead of pushing them into the ring with global
                 atomics as spikes occur -- the faster form for batched runs.  "auto": batch >= 8 (and delay_offset
@@ -82,7 +92,7 @@ class Glif3Simulator:
 
     def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
                  asc_init=None, u_init=None, i_ext=None, device=None, resident="auto", delay_offset="auto",
-                 pull="auto", single_workgroup=True, fired_lists=True):
+                 pull="auto", single_workgroup=True, fired_lists=True, fused="auto", fuse_wg_per_cu=0):
         self.lib = _lib.load()
         self.dev = device or _dev()
         self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
@@ -199,6 +209,13 @@ class Glif3Simulator:
             self._setup_resident(required=(resident is True))
         self.pull_table = self.pull_syn = self.pull_work = None
         self.pull_inp_table = self.pull_inp_syn = self.pull_inp_work = self.in_hist = None
+        self.fuse_table = self.fuse_any = None
+        self.fuse_wg_per_cu = int(fuse_wg_per_cu)
+        can_fuse = ((self.rec is not None or self.inp is not None) and not self.res_span and self.delay_offset == 0
+                    and self.delay_bits == 6 and self.batch in FUSE_BATCHES and pull is not False)
+        if fused is True and not can_fuse:
+            raise ValueError("the fused form needs a synapse table, launch-per-step mode, delay_offset 0, delays "
+                             "within 63 steps and a batch of 8, 16, 32 or 64")
         can_pull = (self.rec is not None and not self.res_span and self.delay_offset == 0
                     and self.L * ((self.n + 31) // 32) * 4 <= PULL_MAP_BYTES)
         # the pull form sums in 64-bit fixed point: weights must be finite and below 2^31 in size
@@ -213,7 +230,15 @@ class Glif3Simulator:
         if pull is True and not can_pull:
             raise ValueError("the pull form needs a recurrent table, launch-per-step mode, delay_offset 0 and "
                              "ring_slots * n_neurons / 8 bytes of LDS (at most 40 KB)")
-        if can_pull and (pull is True or (pull == "auto" and self.batch >= 8)):
+        if can_fuse and fused and (fused is True or pull is True or self.batch >= 8):
+            tables = [t for t in (self.rec, self.inp) if t is not None]
+            if all(fixed_point_ok(t) for t in tables):
+                self._setup_fused()
+            elif fused is True:
+                raise ValueError("the fused form needs finite weights smaller than 2^31 in size")
+        if self.fuse_table is not None:
+            pass
+        elif can_pull and (pull is True or (pull == "auto" and self.batch >= 8)):
             self.pull_table = self.rec.transposed(self.n)
             self.pull_syn = torch.zeros(NREC, self.ne, device=self.dev)
             need = self.lib.bmtk_csr_propagate_pull_workspace_bytes(self.L, self.n)
@@ -228,6 +253,46 @@ class Glif3Simulator:
                 self.pull_inp_work = torch.zeros(need // 4 + 1, dtype=torch.int32, device=self.dev)
                 self.in_hist_stride = n_words(self.n_inputs * self.batch) + 1
                 self.in_hist = torch.zeros(self.L * self.in_hist_stride, dtype=torch.int64, device=self.dev)
+
+    def _setup_fused(self):
+        """Joint target-major table, joint history and activity map of the fused batched driver."""
+        n, batch, n_in = self.n, self.batch, self.n_inputs if self.inp is not None else 0
+        self.fuse_in_base = -(-n * batch // 64) * 64 // batch
+        if self.fuse_in_base + n_in >= 2 ** 24:
+            return
+        self.fuse_table = SynapseTable.joined_by_target(self.rec, self.inp, n, self.fuse_in_base)
+        self.fuse_hist_stride = self.fuse_in_base * batch // 64 + n_words(n_in * batch) + 1
+        self.hist_slots = self.L + 2
+        self.work_bits = torch.zeros(self.hist_slots * self.fuse_hist_stride, dtype=torch.int64, device=self.dev)
+        # one bit of the activity map per 2^shift sources: the smallest shift whose map fits the LDS beside the
+        # accumulators (16 wavefronts x (4 x batch sums + a stage of 64 synapses) x 8 bytes)
+        fixed = FUSE_WAVES * (NREC * batch + 64) * 8
+        self.fuse_shift = 0
+        while fixed + (self.L - 1) * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
+            self.fuse_shift += 1
+        self.fuse_any = self._new_fuse_any()
+
+    def set_fuse_shift(self, shift):
+        """Fused form: one bit of the activity map per 2^shift sources (the constructor picks the smallest shift
+        whose map fits the LDS).  Before the first run only."""
+        if self.fuse_table is None or self.step:
+            raise ValueError("set_fuse_shift applies to the fused form before its first run")
+        fixed = FUSE_WAVES * (NREC * self.batch + 64) * 8
+        old, self.fuse_shift = self.fuse_shift, int(shift)
+        if not 0 <= self.fuse_shift <= 16 or fixed + (self.L - 1) * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
+            self.fuse_shift = old
+            raise ValueError("shift must lie in 0..16 and leave the activity map within the LDS")
+        self.fuse_any = self._new_fuse_any()
+
+    def _new_fuse_any(self):
+        # the activity map (one row per history row) and, behind it, the map of ring cells that hold something
+        # (one row per ring slot, a bit per neuron)
+        return torch.zeros(self.hist_slots * self._fuse_any_words() + self.L * (-(-self.n // 32)), dtype=torch.int32,
+                           device=self.dev)
+
+    def _fuse_any_words(self):
+        groups = -(-(self.fuse_in_base + (self.n_inputs if self.inp is not None else 0)) // (1 << self.fuse_shift))
+        return -(-groups // 32)
 
     def _setup_resident(self, required):
         """Resident mode keeps state in registers and the ring in LDS for a whole
@@ -328,7 +393,7 @@ class Glif3Simulator:
         self.in_steps = in_ptr.numel() - 1
         self.in_duplicates = repeat is not None
         self.in_repeat_ptr = self.in_repeat_events = None
-        if repeat is not None and self.pull_inp_table is not None:
+        if repeat is not None and (self.pull_inp_table is not None or self.fuse_table is not None):
             where = repeat.nonzero().flatten() + 1         # positions of the second and later occurrences
             self.in_repeat_events = in_events[where].contiguous()
             self.in_repeat_ptr = torch.searchsorted(where, in_ptr).to(torch.int64).contiguous()
@@ -360,6 +425,13 @@ class Glif3Simulator:
                 s.in_hist, s.in_hist_stride = _p(self.in_hist), self.in_hist_stride
                 if self.in_repeat_ptr is not None:
                     s.in_repeat_ptr, s.in_repeat_events = _p(self.in_repeat_ptr), _p(self.in_repeat_events)
+        if self.fuse_table is not None:
+            s.n_inputs = self.n_inputs if self.inp is not None else 0   # the history's layout, events or not
+            s.fuse_indptr, s.fuse_packed = _p(self.fuse_table.indptr), _p(self.fuse_table.packed())
+            s.fuse_any, s.fuse_hist_stride, s.fuse_in_base = _p(self.fuse_any), self.fuse_hist_stride, self.fuse_in_base
+            s.fuse_shift, s.fuse_wg_per_cu = self.fuse_shift, self.fuse_wg_per_cu
+            if self.in_repeat_ptr is not None:
+                s.in_repeat_ptr, s.in_repeat_events = _p(self.in_repeat_ptr), _p(self.in_repeat_events)
         if self.res_span:
             s.res_span, s.res_groups, s.res_sync = self.res_span, self.res_groups, _p(self.res_sync)
             s.res_spin_limit = int(self.spin_limit)

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 17
+#define BMTK_AMD_ABI_VERSION 18
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -299,6 +299,30 @@ typedef struct bmtk_glif3_sim {
      * ring. */
     const int64_t *in_repeat_ptr;        /* [total steps + 1] */
     const int32_t *in_repeat_events;
+    /* Fused form of the batched driver (optional; launch-per-step mode, batch 8, 16, 32 or 64, delay_offset 0,
+     * hist_slots == ring_slots + 2; takes precedence over pull_*): ONE launch per step in which a wavefront owns a
+     * target neuron at a time -- it sums what arrives at the neuron in step t-1 over recurrent AND input synapses in
+     * one pass over a joint target-major table (64-bit fixed point in LDS, as bmtk_csr_propagate_pull), folds the
+     * sums into y1 and advances the neuron's `batch` trials through step t, lane = trial; no arrival sum passes
+     * through device memory.  The joint table's index field names a source of the joint space: neuron j is j,
+     * input source k is fuse_in_base + k, fuse_in_base = ceil(n_neurons*batch/64)*64/batch.  work_bits is then the
+     * joint history [hist_slots][fuse_hist_stride]: bit j*batch+b of row t % hist_slots = source j fired (or had an
+     * input event) in trial b of step t; the driver writes the input part of row t from in_ptr / in_events in the
+     * launch of step t.  Repeated ids of a step go through the ring as events (in_repeat_*, with inp_indptr /
+     * inp_packed), as in the pull form.  fuse_any is the "some trial fired" map of the joint sources, one bit per
+     * group of 2^fuse_shift sources and history row; a coarser map (larger shift) costs mask fetches for silent
+     * sources but is what lets any number of sources fit the LDS: (ring_slots-1) * fuse_any_words * 4 bytes beside
+     * the accumulators must stay within 80 KB. */
+    const int32_t *fuse_indptr;        /* [n_neurons + 1] */
+    const bmtk_synapse *fuse_packed;   /* rows = targets, index field = joint source */
+    uint32_t *fuse_any;                /* [hist_slots][fuse_any_words] followed by [ring_slots][ceil(n_neurons/32)]
+                                        * words (a bit per neuron and ring slot: the slot holds an arrival of a
+                                        * repeated id for the neuron), zeroed with work_bits before the first run;
+                                        * fuse_any_words = ceil(ceil((fuse_in_base + n_inputs) / 2^fuse_shift) / 32) */
+    int64_t fuse_hist_stride;          /* words per row of work_bits: >= fuse_in_base*batch/64 + ceil(n_inputs*batch/64) + 1 */
+    int64_t fuse_in_base;
+    int32_t fuse_shift;                /* 0..16 */
+    int32_t fuse_wg_per_cu;            /* persistent workgroups per compute unit, 0 = the library's choice */
     /* outputs */
     uint64_t *spike_bits;        /* [n_steps][words] spike bits per step, words = ceil(ne/64); or NULL.
                                   * Row k belongs to step step0+k of the call that wrote it. */

@@ -271,11 +271,14 @@ def test_v1_scale_forward_run_against_both_oracles():
     assert agree[np.float64] >= 0.999, agree
 
 
-def test_training_size_forward_run_is_bit_identical_to_the_oracle():
+@pytest.mark.parametrize("fused", [True, False])
+def test_training_size_forward_run_is_bit_identical_to_the_oracle(fused):
     """The forward pass of the training configuration at its own size -- 51,978 neurons x batch 32, 52 M recurrent
-    and 8 M input synapses, 17,400 Poisson inputs at 5 Hz, per-step record on -- through the batched driver (pull
-    form for recurrent and input synapses, repeat lists for ids that occur twice in a step).  Quarter-pA weights:
-    raster, state and the recorded potentials must equal the fp32 oracle's bit for bit."""
+    and 8 M input synapses, 17,400 Poisson inputs at 5 Hz, per-step record on -- through the batched driver: pull
+    and update fused in one launch per step over the joint table (what a simulator picks at this batch), and as
+    separate launches (pull form for recurrent and input synapses); repeat lists for ids that occur twice in a step
+    either way.  Quarter-pA weights: raster, state and the recorded potentials must equal the fp32 oracle's bit for
+    bit."""
     n, n_in, batch, steps = N52K, 17400, 32, 120
     rng = np.random.default_rng(4)
     par = synthetic.random_cells(rng, n)
@@ -284,8 +287,11 @@ def test_training_size_forward_run_is_bit_identical_to_the_oracle():
     inp = synthetic.device_input_table(n_in, n, 8_000_000, seed=4, w_scale=2.0)
     inp = (inp[0], inp[1], _quarter(inp[2]), inp[3], inp[4])
     in_ptr, in_ev = ops.poisson_events(n_in, 5.0, 1.0, steps, batch=batch, seed=5)
-    sim = Glif3Simulator(n, par, 1.0, batch=batch, rec=by_src, inp=inp, resident=False)
-    assert sim.pull_table is not None and sim.pull_inp_table is not None
+    sim = Glif3Simulator(n, par, 1.0, batch=batch, rec=by_src, inp=inp, resident=False, fused="auto" if fused else False)
+    if fused:
+        assert sim.fuse_table is not None and sim.pull_table is None and sim.fuse_shift == 0
+    else:
+        assert sim.pull_table is not None and sim.pull_inp_table is not None
     sim.set_input_events(in_ptr, in_ev)
     assert sim.in_duplicates and sim.in_repeat_events.numel() > 0   # a few ids occur twice within a step
     a = sim.run(50, save_state=True)

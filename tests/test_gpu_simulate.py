@@ -300,10 +300,10 @@ def test_pull_form_of_the_per_step_driver(batch):
     cfg["inp_src"] = _integer_weights(cfg["inp_src"])
     want, st, _ = _oracle_run(cfg, np.float32, batch=batch)
     assert want["count"] > 1000 * batch // 4
-    for pull in (True, False):
+    for pull, fused in ((True, False), (False, False)) + (((True, True),) if batch in (32, 64) else ()):
         sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
-                             inp=cfg["inp_src"], ring_slots=cfg["L"], resident=False, pull=pull)
-        assert (sim.pull_table is not None) == pull
+                             inp=cfg["inp_src"], ring_slots=cfg["L"], resident=False, pull=pull, fused=fused)
+        assert (sim.pull_table is not None) == (pull and not fused) and (sim.fuse_table is not None) == fused
         sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
         a = sim.run(150)
         b = sim.run(250)
@@ -314,7 +314,9 @@ def test_pull_form_of_the_per_step_driver(batch):
             np.testing.assert_array_equal(got[k], st[k], err_msg=k)
     auto = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
                           resident=False)
-    assert (auto.pull_table is not None) == (batch >= 8)
+    # batched runs pull; batches whose trials fill whole bytes of spike bits take the fused form of it
+    assert (auto.fuse_table is not None) == (batch in (8, 16, 32, 64))
+    assert (auto.pull_table is not None) == (batch >= 8 and auto.fuse_table is None)
 
 
 def test_resident_pull_with_more_fired_rows_than_its_list_holds():
@@ -423,7 +425,7 @@ def _with_duplicate_events(cfg, rng, batch):
     return np.asarray(new_ptr, np.int64), np.concatenate(chunks).astype(np.int32)
 
 
-@pytest.mark.parametrize("batch,resident", [(1, False), (1, True), (1, "many"), (8, False)])
+@pytest.mark.parametrize("batch,resident", [(1, False), (1, True), (1, "many"), (8, False), (8, "unfused"), (32, False)])
 def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     """Two spikes of one generator inside one resolution step are two deliveries.  Every driver must count them:
     the launch-per-step driver, the resident one, and the batched driver, whose pull form of the inputs (bit rows:
@@ -440,6 +442,9 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     assert want["count"] > 1.05 * plain["count"] > 500 * batch      # the repeats matter
     if resident == "many":       # 700 neurons on a dozen workgroups instead of one
         kw = dict(resident=True, single_workgroup=False)
+    elif resident == "unfused":  # the batched driver with pull and update as separate launches
+        kw = dict(resident=False, fused=False)
+        resident = False
     else:
         kw = dict(resident=resident)
     sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
@@ -450,7 +455,10 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     a, b = sim.run(120), sim.run(180)
     sim.check()
     if batch >= 8:
-        assert sim.pull_table is not None and sim.pull_inp_table is not None
+        if kw.get("fused", True):
+            assert sim.fuse_table is not None and sim.pull_table is None
+        else:
+            assert sim.pull_table is not None and sim.pull_inp_table is not None
         n_rep = in_events.size - sum(np.unique(in_events[in_ptr[t]:in_ptr[t + 1]]).size for t in range(in_ptr.size - 1))
         assert sim.in_repeat_events.numel() == n_rep > 0 and int(sim.in_repeat_ptr[-1]) == n_rep
     ras = np.concatenate([sim.raster(a["bits"]).cpu().numpy(), sim.raster(b["bits"]).cpu().numpy()])
