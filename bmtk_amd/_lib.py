@@ -60,7 +60,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 18  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 19  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -80,8 +80,9 @@ SIGNATURES = {
                                              c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "bmtk_csr_propagate_gather": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
-    "bmtk_csr_propagate_auto": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int32] + [c_void_p] * 10 +
-                                [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p]),
+    "bmtk_csr_propagate_auto_workspace_bytes": (c_int64, [c_int32, c_int64]),
+    "bmtk_csr_propagate_auto": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int64, c_int32] +
+                                [c_void_p] * 7 + [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "bmtk_csr_propagate_pull_workspace_bytes": (c_int64, [c_int32, c_int64]),
     "bmtk_csr_propagate_pull": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
                                           c_int64, c_int64, c_void_p, c_void_p]),

@@ -314,16 +314,12 @@ __global__ __launch_bounds__(kBlock) void compact_write_fused_kernel(const uint6
 // the ring.
 // ---------------------------------------------------------------------------
 
-// cnt_max: the kernel does nothing when more than that many elements are active (the caller then runs the
-// row-wise form in the same stream, see bmtk_csr_propagate_auto)
 __global__ __launch_bounds__(kBlock) void scatter_kernel(const int32_t *__restrict__ active,
                                                          const int32_t *__restrict__ n_active, int batch, Table t,
-                                                         float *__restrict__ ring, int L, int64_t ne, int slot0,
-                                                         int cnt_max)
+                                                         float *__restrict__ ring, int L, int64_t ne, int slot0)
 {
     const int n_waves = gridDim.x * (kBlock / kWave);
     const int cnt = *n_active;
-    if (cnt > cnt_max) return;
     for (int k = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; k < cnt; k += n_waves) {
         const int e = active[k];
         const int j = batch == 1 ? e : (int)((uint32_t)e / (uint32_t)batch);
@@ -341,13 +337,11 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const int32_t *__restri
 // in stored synapse order: deterministic and equal to a scalar loop.
 // ---------------------------------------------------------------------------
 
-// gate: when given, the kernel only runs if more than gate_min elements are active (*gate)
 __global__ __launch_bounds__(kBlock) void gather_kernel(const uint64_t *__restrict__ zbits, int batch, Table t,
                                                         float *__restrict__ ring, int L, int64_t n_tgt, int64_t ne,
-                                                        int slot0, const int32_t *__restrict__ gate, int gate_min)
+                                                        int slot0)
 {
     extern __shared__ float lds[];
-    if (gate && *gate <= gate_min) return;
     const int lane = lane_id();
     const int wave_in_block = threadIdx.x / kWave;
     float *acc = lds + (size_t)wave_in_block * L * GLIF3_NREC * kWave;
@@ -576,48 +570,8 @@ int bmtk_csr_propagate_scatter(const int32_t *active, const int32_t *n_active, i
     const unsigned grid = (unsigned)((waves + kBlock / kWave - 1) / (kBlock / kWave));
     Table t{indptr, indices, weights, delays, receptors};
     hipLaunchKernelGGL(scatter_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, active, n_active, batch, t,
-                       ring, L, n_tgt * (int64_t)batch, (int)(step % L), 0x7fffffff);
+                       ring, L, n_tgt * (int64_t)batch, (int)(step % L));
     BMTK_CHECK_LAUNCH("csr_propagate_scatter");
-    return BMTK_OK;
-}
-
-int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_active, int64_t max_active,
-                            const uint64_t *zbits, int64_t n_src, int32_t batch,
-                            const int32_t *src_indptr, const int32_t *src_indices, const float *src_weights,
-                            const uint8_t *src_delays, const uint8_t *src_receptors,
-                            const int32_t *tgt_indptr, const int32_t *tgt_indices, const float *tgt_weights,
-                            const uint8_t *tgt_delays, const uint8_t *tgt_receptors,
-                            float *ring, int32_t L, int64_t n_tgt, int64_t step, int64_t scatter_max_active, void *stream)
-{
-    BMTK_REQUIRE(active && n_active && zbits && ring, "csr_propagate_auto: pointers must be non-null");
-    BMTK_REQUIRE(src_indptr && src_indices && src_weights && src_delays && src_receptors && tgt_indptr && tgt_indices &&
-                     tgt_weights && tgt_delays && tgt_receptors,
-                 "csr_propagate_auto: both forms of the table are needed");
-    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && n_src > 0 && step >= 0, "csr_propagate_auto: bad batch, sizes or step");
-    BMTK_REQUIRE(L > 1 && L <= 16, "csr_propagate_auto: ring_slots must lie in 2..16");
-    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31), "csr_propagate_auto: n_tgt*batch must stay below 2^31");
-    BMTK_REQUIRE(scatter_max_active >= 0 && scatter_max_active < (1ll << 31), "csr_propagate_auto: bad threshold");
-    const int64_t ne = n_tgt * (int64_t)batch;
-    const int slot0 = (int)(step % L);
-    // both kernels are enqueued; each looks at the active count on the device and one of them returns at once
-    const int64_t bound = max_active < scatter_max_active ? max_active : scatter_max_active;
-    if (bound > 0) {
-        const int64_t waves = bound < 8192 ? bound : 8192;
-        const unsigned grid = (unsigned)((waves + kBlock / kWave - 1) / (kBlock / kWave));
-        Table t{src_indptr, src_indices, src_weights, src_delays, src_receptors};
-        hipLaunchKernelGGL(scatter_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, active, n_active, batch, t,
-                           ring, L, ne, slot0, (int)scatter_max_active);
-    }
-    if (max_active > scatter_max_active) {
-        const unsigned rows_per_block = kBlock / kWave;
-        const dim3 grid((unsigned)((n_tgt + rows_per_block - 1) / rows_per_block), (unsigned)((batch + kWave - 1) / kWave));
-        BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_auto: batch too large");
-        const size_t lds = (size_t)rows_per_block * L * GLIF3_NREC * kWave * sizeof(float);
-        Table t{tgt_indptr, tgt_indices, tgt_weights, tgt_delays, tgt_receptors};
-        hipLaunchKernelGGL(gather_kernel, grid, dim3(kBlock), lds, (hipStream_t)stream, zbits, batch, t, ring, L, n_tgt, ne,
-                           slot0, n_active, (int)scatter_max_active);
-    }
-    BMTK_CHECK_LAUNCH("csr_propagate_auto");
     return BMTK_OK;
 }
 
@@ -637,7 +591,7 @@ int bmtk_csr_propagate_gather(const uint64_t *zbits, int64_t n_src, int32_t batc
     const size_t lds = (size_t)rows_per_block * L * GLIF3_NREC * kWave * sizeof(float);
     Table t{indptr, indices, weights, delays, receptors};
     hipLaunchKernelGGL(gather_kernel, grid, dim3(kBlock), lds, (hipStream_t)stream, zbits, batch, t, ring, L, n_tgt,
-                       n_tgt * (int64_t)batch, (int)(step % L), (const int32_t *)nullptr, 0);
+                       n_tgt * (int64_t)batch, (int)(step % L));
     BMTK_CHECK_LAUNCH("csr_propagate_gather");
     return BMTK_OK;
 }

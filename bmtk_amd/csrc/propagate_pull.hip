@@ -59,14 +59,29 @@ constexpr size_t kPullLdsMax = 80u * 1024u;  // two workgroups per compute unit:
 // one gather of 64 masks, one conversion, one bit walk with every lane busy.  At 1 Hz that is once per row
 // instead of sixteen times.  The per-synapse part uses 32-bit offsets against scalar base pointers and unsigned
 // wrap-around for the history row of a delay.
-template <bool kWords64>
+//
+// kAuto: the kernel serves bmtk_csr_propagate_auto.  `ctrl` then says, per history row, whether the row's spikes
+// are left to this kernel at all (the others were pushed into the ring as events when they occurred): with no such
+// row among the L-1 the arrival step looks back on, the kernel returns at once.  And `syn` is the ring slot of the
+// arrival step, which may already hold what pushed spikes sent there: ctrl says so, and the sums are then added to
+// the cells instead of replacing them.
+constexpr int kAutoRows = 64;  // ctrl: int32 pulled[kAutoRows], then int32 slot_holds[kAutoRows]
+template <bool kWords64, bool kAuto>
 __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride, int L,
                                                          int batch, const int32_t *__restrict__ indptr,
                                                          const bmtk_synapse *__restrict__ packed,
                                                          float *__restrict__ syn, int64_t n_tgt, int64_t ne,
-                                                         int slot_now, const uint32_t *__restrict__ any_map, int n_w32)
+                                                         int slot_now, const uint32_t *__restrict__ any_map, int n_w32,
+                                                         const int32_t *__restrict__ ctrl)
 {
     extern __shared__ unsigned long long pull_lds[];  // accumulators, stages, then the activity map [L][n_w32]
+    bool add_to_cells = false;
+    if (kAuto) {
+        int pulled = 0;
+        for (int d = 1; d < L; ++d) pulled |= ctrl[(slot_now + L - d) % L];
+        if (!pulled) return;
+        add_to_cells = ctrl[kAutoRows + slot_now] != 0;
+    }
     // (the wavefront's number through a scalar register, so that rows, bounds and base pointers stay scalar)
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     unsigned long long(*acc)[kWave] = reinterpret_cast<unsigned long long(*)[kWave]>(pull_lds) + wave * GLIF3_NREC;
@@ -82,10 +97,13 @@ __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__r
     const char *__restrict__ hist_bytes = reinterpret_cast<const char *>(hist);
     // Block of the table: 64-bit words at a scalar base, 8 * (lane + u*64) bytes on.  Lanes past the end of the
     // row read its last synapse again (and are ignored later): no branch, the four loads go out back to back.
+    // A block past the end or an empty one reads the table's first record the same way: every call issues exactly
+    // four loads, which is what lets a turn wait for ITS block only and leave the younger ones in flight (the wait
+    // is a count of loads still out, fixed at compile time).
     auto fetch = [&](unsigned long long *dst, const PullBlock &blk) {
-        if (blk.row >= n_tgt || blk.base >= blk.p1) return;
-        const char *__restrict__ src = reinterpret_cast<const char *>(packed) + (size_t)blk.base * 8u;
-        const unsigned last = (unsigned)(blk.p1 - blk.base) - 1u;
+        const bool some = blk.row < n_tgt && blk.base < blk.p1;
+        const char *__restrict__ src = reinterpret_cast<const char *>(packed) + (some ? (size_t)blk.base * 8u : (size_t)0);
+        const unsigned last = some ? (unsigned)(blk.p1 - blk.base) - 1u : 0u;
 #pragma unroll
         for (int u = 0; u < kPullChunks; ++u)
             // streamed once per step: keep it from displacing the spike history in L2
@@ -157,23 +175,70 @@ __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__r
             flush();
 #pragma unroll
             for (int r = 0; r < GLIF3_NREC; ++r) {
-                if ((int)lane < width) syn[(int64_t)r * ne + cb.row * batch + tile0 + lane] = from_fixed(acc[r][lane]);
+                if ((int)lane < width) {
+                    float *cell = syn + ((int64_t)r * ne + cb.row * batch + tile0 + lane);
+                    const float sum = from_fixed(acc[r][lane]);
+                    *cell = (kAuto && add_to_cells) ? *cell + sum : sum;
+                }
                 acc[r][lane] = 0ull;
             }
         }
         cb = cursor.next();
         fetch(cd, cb);
     };
-    // the buffers take turns in place, so that no register copy ties the arrival of a later block to the work on
-    // this one
-    while (true) {
+    // The buffers take turns in place, so that no register copy ties the arrival of a later block to the work on
+    // this one.  One way out of the loop, after a whole round: with a way out after every turn the compiler joins
+    // them in one block before the loop's head, from where it looks as if a turn could follow directly on the fetch
+    // of its own buffer, and every turn would wait for all loads in flight.  The turns past a wavefront's last
+    // block (at most two) see empty blocks of no row.
+    do {
         turn(b0, d0);
-        if (b1.row >= n_tgt) break;
         turn(b1, d1);
-        if (b2.row >= n_tgt) break;
         turn(b2, d2);
-        if (b0.row >= n_tgt) break;
+    } while (b0.row < n_tgt);
+}
+
+// bmtk_csr_propagate_auto, first launch: the spikes of step `step` as events, if they are few.  Every workgroup
+// reads the number of active elements and decides the same way; up to cnt_max the elements' rows are walked and
+// their weights pushed into the ring (fp32 atomics), above it nothing happens here and the step is left to the
+// pull kernel.  One thread records the decision: ctrl[row] = 1 when the history row of the step is to be pulled,
+// and which ring slots hold pushed arrivals (the slot of the step itself, consumed by now, holds none).
+__global__ __launch_bounds__(kBlock) void auto_push_kernel(const int32_t *__restrict__ active,
+                                                           const int32_t *__restrict__ n_active, int batch, Table t,
+                                                           float *__restrict__ ring, int L, int64_t ne, int slot0,
+                                                           int cnt_max, int32_t *__restrict__ ctrl)
+{
+    const int n_waves = gridDim.x * (kBlock / kWave);
+    const int cnt = *n_active;
+    const bool push = cnt <= cnt_max;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        ctrl[slot0] = push ? 0 : 1;
+        ctrl[kAutoRows + slot0] = 0;
+        if (push && cnt > 0)
+            for (int d = 1; d < L; ++d) ctrl[kAutoRows + (slot0 + d) % L] = 1;
     }
+    if (!push) return;
+    for (int k = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; k < cnt; k += n_waves) {
+        const int e = active[k];
+        const int j = batch == 1 ? e : (int)((uint32_t)e / (uint32_t)batch);
+        deliver_row(t, j, e - j * batch, batch, ring, L, slot0, ne);
+    }
+}
+
+// ... second launch: the row of the step in the activity map -- from the history row when the step is to be
+// pulled, empty when its spikes were pushed (the pull kernel then finds nothing of that step)
+__global__ __launch_bounds__(kBlock) void auto_anymap_kernel(const uint64_t *__restrict__ hist_row, int batch,
+                                                             int64_t n_src, int n_w32, uint32_t *__restrict__ any_row,
+                                                             const int32_t *__restrict__ pulled)
+{
+    const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    bool any = false;
+    if (*pulled && j < n_src) {
+        for (int t0 = 0; t0 < batch && !any; t0 += kWave)
+            any = source_mask(hist_row, (int)j, batch, t0, min(kWave, batch - t0)) != 0ull;
+    }
+    const unsigned long long m = __ballot(any);
+    if ((lane_id() & 31) == 0 && j < (int64_t)n_w32 * 32) any_row[j >> 5] = (uint32_t)(m >> (lane_id() & 32));
 }
 
 }  // namespace bmtk
@@ -222,7 +287,8 @@ extern "C" int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_
     static bool asked[2][64];
     if (dev >= 0 && dev < 64 && !asked[batch == kWave][dev]) {
         const hipError_t err = hipFuncSetAttribute(
-            batch == kWave ? reinterpret_cast<const void *>(pull_kernel<true>) : reinterpret_cast<const void *>(pull_kernel<false>),
+            batch == kWave ? reinterpret_cast<const void *>(pull_kernel<true, false>)
+                           : reinterpret_cast<const void *>(pull_kernel<false, false>),
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPullLdsMax);
         if (err != hipSuccess) {
             set_error("csr_propagate_pull: cannot reserve %zu bytes of LDS: %s", kPullLdsMax, hipGetErrorString(err));
@@ -231,11 +297,98 @@ extern "C" int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_
         asked[batch == kWave][dev] = true;
     }
     if (batch == kWave)
-        hipLaunchKernelGGL(pull_kernel<true>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
-                           batch, indptr, packed, syn, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
+        hipLaunchKernelGGL((pull_kernel<true, false>), grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist,
+                           hist_stride, L, batch, indptr, packed, syn, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L),
+                           any_map, n_w32, (const int32_t *)nullptr);
     else
-        hipLaunchKernelGGL(pull_kernel<false>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
-                           batch, indptr, packed, syn, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
+        hipLaunchKernelGGL((pull_kernel<false, false>), grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist,
+                           hist_stride, L, batch, indptr, packed, syn, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L),
+                           any_map, n_w32, (const int32_t *)nullptr);
     BMTK_CHECK_LAUNCH("csr_propagate_pull");
+    return BMTK_OK;
+}
+
+extern "C" int64_t bmtk_csr_propagate_auto_workspace_bytes(int32_t L, int64_t n_src)
+{
+    if (L <= 0 || n_src <= 0) return 0;
+    return (int64_t)L * ((n_src + 31) / 32) * 4 + 2 * bmtk::kAutoRows * 4;
+}
+
+extern "C" int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_active, int64_t max_active,
+                                       const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src,
+                                       int32_t batch, const int32_t *src_indptr, const int32_t *src_indices,
+                                       const float *src_weights, const uint8_t *src_delays, const uint8_t *src_receptors,
+                                       const int32_t *tgt_indptr, const bmtk_synapse *tgt_packed, float *ring,
+                                       int64_t n_tgt, int64_t step, int64_t scatter_max_active, void *workspace,
+                                       void *stream)
+{
+    using namespace bmtk;
+    BMTK_REQUIRE(active && n_active && spike_hist && ring && workspace, "csr_propagate_auto: pointers must be non-null");
+    BMTK_REQUIRE(src_indptr && src_indices && src_weights && src_delays && src_receptors && tgt_indptr && tgt_packed,
+                 "csr_propagate_auto: both forms of the table are needed");
+    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && n_src > 0 && step >= 0, "csr_propagate_auto: bad batch, sizes or step");
+    BMTK_REQUIRE(L > 1 && L <= kAutoRows, "csr_propagate_auto: L must lie in 2..64");
+    BMTK_REQUIRE(hist_stride >= (n_src * (int64_t)batch + 63) / 64 + 1,
+                 "csr_propagate_auto: hist_stride must hold ceil(n_src*batch/64)+1 words");
+    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31) && n_src < (1ll << 24), "csr_propagate_auto: network too large");
+    BMTK_REQUIRE((int64_t)L * hist_stride < (1ll << 29) && hist_stride < (1ll << 24),
+                 "csr_propagate_auto: spike history beyond 4 GiB");
+    BMTK_REQUIRE(scatter_max_active >= 0 && scatter_max_active < (1ll << 31) && max_active >= 0,
+                 "csr_propagate_auto: bad threshold or bound");
+    const int n_w32 = (int)((n_src + 31) / 32);
+    const size_t lds = (size_t)L * n_w32 * 4 + kPullAccBytes;
+    BMTK_REQUIRE(lds <= kPullLdsMax, "csr_propagate_auto: L * n_src too large for the activity map in LDS");
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t *any_map = (uint32_t *)workspace;
+    int32_t *ctrl = (int32_t *)(any_map + (size_t)L * n_w32);
+    const int64_t ne = n_tgt * (int64_t)batch;
+    const int slot0 = (int)(step % L);
+    {   // the step's spikes as events, if they are few (the launch also records the decision)
+        const int64_t bound = max_active < scatter_max_active ? max_active : scatter_max_active;
+        const int64_t waves = bound < 1 ? 1 : (bound < 8192 ? bound : 8192);
+        const unsigned grid = (unsigned)((waves + kBlock / kWave - 1) / (kBlock / kWave));
+        Table t{src_indptr, src_indices, src_weights, src_delays, src_receptors};
+        hipLaunchKernelGGL(auto_push_kernel, dim3(grid), dim3(kBlock), 0, st, active, n_active, batch, t, ring, L, ne, slot0,
+                           (int)scatter_max_active, ctrl);
+    }
+    hipLaunchKernelGGL(auto_anymap_kernel, dim3((unsigned)(((int64_t)n_w32 * 32 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
+                       spike_hist + (int64_t)slot0 * hist_stride, batch, n_src, n_w32, any_map + (size_t)slot0 * n_w32,
+                       ctrl + slot0);
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    static int cu_count[64];
+    int n_cu = (dev >= 0 && dev < 64) ? cu_count[dev] : 0;
+    if (n_cu <= 0) {
+        n_cu = 256;
+        (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (dev >= 0 && dev < 64) cu_count[dev] = n_cu;
+    }
+    const unsigned rows_per_block = kPullBlock / kWave;
+    const unsigned want = (unsigned)((n_tgt + rows_per_block - 1) / rows_per_block);
+    const unsigned cap = (unsigned)n_cu * 2u;
+    const dim3 grid(want < cap ? want : cap, (unsigned)((batch + kWave - 1) / kWave));
+    BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_auto: batch too large");
+    static bool asked[2][64];
+    if (dev >= 0 && dev < 64 && !asked[batch == kWave][dev]) {
+        const hipError_t err = hipFuncSetAttribute(
+            batch == kWave ? reinterpret_cast<const void *>(pull_kernel<true, true>)
+                           : reinterpret_cast<const void *>(pull_kernel<false, true>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPullLdsMax);
+        if (err != hipSuccess) {
+            set_error("csr_propagate_auto: cannot reserve %zu bytes of LDS: %s", kPullLdsMax, hipGetErrorString(err));
+            return BMTK_E_LAUNCH;
+        }
+        asked[batch == kWave][dev] = true;
+    }
+    // everything that arrives in step + 1 from the steps that were not pushed, into the ring slot of that step
+    const int slot_arrive = (int)((step + 1) % L);
+    float *cells = ring + (int64_t)slot_arrive * GLIF3_NREC * ne;
+    if (batch == kWave)
+        hipLaunchKernelGGL((pull_kernel<true, true>), grid, dim3(kPullBlock), lds, st, spike_hist, hist_stride, L, batch,
+                           tgt_indptr, tgt_packed, cells, n_tgt, ne, slot_arrive, any_map, n_w32, (const int32_t *)ctrl);
+    else
+        hipLaunchKernelGGL((pull_kernel<false, true>), grid, dim3(kPullBlock), lds, st, spike_hist, hist_stride, L, batch,
+                           tgt_indptr, tgt_packed, cells, n_tgt, ne, slot_arrive, any_map, n_w32, (const int32_t *)ctrl);
+    BMTK_CHECK_LAUNCH("csr_propagate_auto");
     return BMTK_OK;
 }

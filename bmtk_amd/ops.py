@@ -437,38 +437,55 @@ def blocked_plan(n, batch):
     return dict(grid=plan[0], rows_per_workgroup=plan[1], sweeps=plan[2], groups_per_wavefront=plan[3])
 
 
-def csr_propagate_auto(active, n_active, zbits, n_src, table_src, table_tgt, ring, n_tgt, batch, step,
-                       scatter_max_active=None, max_active=None):
-    """Delivery with the form chosen on the device (no host synchronisation): the event-driven scatter up to
-    ``scatter_max_active`` active elements, the row-wise gather above.  Default threshold: a fifth of the source
-    rows per 64 trials, the measured break-even of the two kernels on one MI355X."""
-    lib = _lib.load()
-    L = ring.shape[0]
-    if ring.numel() != L * NREC * n_tgt * batch or table_tgt.n_rows != n_tgt or table_src.n_rows != n_src:
-        raise ValueError("ring must be [L, 4, n_tgt*batch]; tables must have one row per source / per target")
-    if scatter_max_active is None:
-        scatter_max_active = max(1, n_src // 5) * max(1, batch // 64)
-    if max_active is None:
-        max_active = active.numel()
-    _lib.check(lib.bmtk_csr_propagate_auto(
-        _p(active, torch.int32, None, "active"), _p(n_active, torch.int32, 1, "n_active"), max_active,
-        _p(zbits, torch.int64, n_words(n_src * batch) + 1, "zbits"), n_src, batch, *table_src.pointers(),
-        *table_tgt.pointers(), _p(ring, torch.float32), L, n_tgt, int(step), int(scatter_max_active), _stream()))
+class AutoPropagator:
+    """Step-by-step delivery with the form chosen on the device (``bmtk_csr_propagate_auto``): few spikes are pushed
+    into the ring as events through the source-major table, many are left to the pull over the target-major table
+    and the spike history.  Owns the workspace (activity map of the last L steps, record of the pushed steps).
+
+    ``hist`` is the caller's spike history, int64 [L, words+1]: before ``step(k, ...)`` row k % L must hold the
+    spike bits of step k.  After the call ring slot (k + 1) % L holds everything that arrives in step k + 1; the
+    caller consumes and clears it before the next call.  Default threshold: 2,000 active elements per 52 M synapses
+    of table, the measured break-even on one MI355X."""
+
+    def __init__(self, table_src, table_tgt, hist, ring, n_src, n_tgt, batch, scatter_max_active=None):
+        self.lib = _lib.load()
+        L = hist.shape[0]
+        if ring.numel() != L * NREC * n_tgt * batch or table_tgt.n_rows != n_tgt or table_src.n_rows != n_src:
+            raise ValueError("ring must be [L, 4, n_tgt*batch]; tables must have one row per source / per target")
+        if table_tgt.max_delay() >= L:
+            raise ValueError("spike history of {} steps is shorter than the largest delay".format(L))
+        self.src, self.tgt, self.hist, self.ring = table_src, table_tgt, hist, ring
+        self.L, self.n_src, self.n_tgt, self.batch = L, n_src, n_tgt, batch
+        if scatter_max_active is None:
+            scatter_max_active = max(1, int(2000 * table_tgt.nnz / 52e6))
+        self.scatter_max_active = int(scatter_max_active)
+        need = self.lib.bmtk_csr_propagate_auto_workspace_bytes(L, n_src)
+        self.workspace = torch.zeros(need // 4 + 1, dtype=torch.int32, device=ring.device)
+
+    def step(self, k, active, n_active, max_active=None):
+        if max_active is None:
+            max_active = active.numel()
+        _lib.check(self.lib.bmtk_csr_propagate_auto(
+            _p(active, torch.int32, None, "active"), _p(n_active, torch.int32, 1, "n_active"), max_active,
+            _p(self.hist, torch.int64), self.hist.shape[1], self.L, self.n_src, self.batch, *self.src.pointers(),
+            _p(self.tgt.indptr), _p(self.tgt.packed()), _p(self.ring, torch.float32), self.n_tgt, int(k),
+            self.scatter_max_active, _p(self.workspace), _stream()))
+
+    def pulled_steps(self):
+        """Which of the history rows are left to the pull kernel (bool [L]; synchronises) -- for tests and
+        profiles."""
+        n_w32 = (self.n_src + 31) // 32
+        return self.workspace[self.L * n_w32:self.L * n_w32 + self.L].cpu().numpy() != 0
 
 
-def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_active=None, zbits=None, n_src=None,
-                      table_tgt=None, scatter_max_active=None):
-    """``mode`` "scatter" (source-major table + active list), "gather" (target-major table + spike bits) or
-    "auto" (``table`` source-major and ``table_tgt`` target-major, active list and spike bits: the device picks
-    by the active count, see ``csr_propagate_auto``)."""
+def csr_propagate_fwd(mode, table, ring, n_tgt, batch, step, active=None, n_active=None, zbits=None, n_src=None):
+    """``mode`` "scatter" (source-major table + active list) or "gather" (target-major table + spike bits); the
+    form chosen on the device needs state from step to step, see ``AutoPropagator``."""
     if mode == "scatter":
         return csr_propagate_scatter(active, n_active, table, ring, n_tgt, batch, step)
     if mode == "gather":
         return csr_propagate_gather(zbits, n_src, table, ring, n_tgt, batch, step)
-    if mode == "auto":
-        return csr_propagate_auto(active, n_active, zbits, n_src, table, table_tgt, ring, n_tgt, batch, step,
-                                  scatter_max_active)
-    raise ValueError("mode must be 'scatter', 'gather' or 'auto'")
+    raise ValueError("mode must be 'scatter' or 'gather'")
 
 
 def poisson_events(n_sources, rate_hz, dt_ms, n_steps, batch=1, seed=1, t_start_ms=0.0, t_stop_ms=None,

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 18
+#define BMTK_AMD_ABI_VERSION 19
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -120,22 +120,6 @@ int bmtk_csr_propagate_gather(const uint64_t *zbits, int64_t n_src, int32_t batc
                               const uint8_t *delays, const uint8_t *receptors,
                               float *ring, int32_t L, int64_t n_tgt, int64_t step, void *stream);
 
-/* The same delivery with the form chosen ON THE DEVICE from the number of active elements, without a host
- * synchronisation: up to scatter_max_active active elements the event-driven form runs (its cost grows with the
- * number of events), above it the row-wise form (its cost is a pass over the table).  Both kernels are enqueued and
- * one of them returns at once, so the call costs one empty launch more than the form it picks.  The caller supplies
- * both views of one step's spikes -- the active list with its device-side count and the spike bits -- and both forms
- * of the table.  On one MI355X with 51,978 neurons, in-degree 1000 and batch 64 the two forms cost the same near
- * 10,000 active elements (3 Hz). */
-int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_active, int64_t max_active,
-                            const uint64_t *zbits, int64_t n_src, int32_t batch,
-                            const int32_t *src_indptr, const int32_t *src_indices, const float *src_weights,
-                            const uint8_t *src_delays, const uint8_t *src_receptors,
-                            const int32_t *tgt_indptr, const int32_t *tgt_indices, const float *tgt_weights,
-                            const uint8_t *tgt_delays, const uint8_t *tgt_receptors,
-                            float *ring, int32_t L, int64_t n_tgt, int64_t step, int64_t scatter_max_active,
-                            void *stream);
-
 /* One packed synapse: tdr = index | receptor << 24 | delay << 26 (index < 2^24, delay < 64 steps). */
 typedef struct bmtk_synapse {
     uint32_t tdr;
@@ -163,6 +147,34 @@ int64_t bmtk_csr_propagate_pull_workspace_bytes(int32_t L, int64_t n_src);
 int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src, int32_t batch,
                             const int32_t *indptr, const bmtk_synapse *packed, float *syn, int64_t n_tgt,
                             int64_t t_arrive, void *workspace, void *stream);
+
+/* Delivery step by step with the form chosen ON THE DEVICE from the number of active elements, without a host
+ * synchronisation -- the switch NEST does not need (it is always event-driven) and a GPU does: pushing events costs
+ * one fp32 atomic each (about 2e10 per second on one MI355X, whatever the rate), the pull form a pass over the whole
+ * table (about 100 us for 52 M synapses, whatever the rate), so few spikes are pushed and many are pulled.
+ * Call once per step, in order, after the step's spikes are known:
+ *   - spike_hist row (step mod L) holds the spike bits of `step` (the caller wrote them), active / *n_active the
+ *     same spikes as a list (bmtk_spikes_compact*);
+ *   - up to scatter_max_active active elements the spikes are pushed into `ring` through the SOURCE-major table
+ *     (as bmtk_csr_propagate_scatter) and their history row is struck from the pull's view; above it they are left
+ *     to the pull kernel, which sums, over the packed TARGET-major table, what the steps not pushed send to step
+ *     + 1 and writes (or, where pushed spikes already sent something, adds) it into ring slot (step + 1) mod L.
+ *     When none of the L-1 steps the arrival step looks back on was left to it, the pull kernel returns at once.
+ *   After the call ring slot (step + 1) mod L holds everything that arrives in step + 1, whatever mix of forms
+ *   delivered it; the caller consumes and CLEARS that slot before the next call (bmtk_glif3_step_fwd with
+ *   clear_syn does), as with the event-driven form.  Later slots hold the pushed part only.
+ * workspace: bmtk_csr_propagate_auto_workspace_bytes(L, n_src) bytes, zeroed before the first call and then left
+ * to the library (the activity map of the last L steps and the record of which steps were pushed).  Limits as for
+ * bmtk_csr_propagate_pull.  On one MI355X with 51,978 neurons, in-degree 1000 and batch 64 the two forms cost the
+ * same near 2,000 active elements per step (0.6 Hz). */
+int64_t bmtk_csr_propagate_auto_workspace_bytes(int32_t L, int64_t n_src);
+int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_active, int64_t max_active,
+                            const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src, int32_t batch,
+                            const int32_t *src_indptr, const int32_t *src_indices, const float *src_weights,
+                            const uint8_t *src_delays, const uint8_t *src_receptors,
+                            const int32_t *tgt_indptr, const bmtk_synapse *tgt_packed,
+                            float *ring, int64_t n_tgt, int64_t step, int64_t scatter_max_active, void *workspace,
+                            void *stream);
 
 /* Packed synapse format used by the fused simulation: one 8-byte record per
  * synapse, {uint32 tdr, float weight} with tdr = index | receptor << 24 |

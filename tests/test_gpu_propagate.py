@@ -211,27 +211,47 @@ def test_table_from_edges_on_the_device_equals_the_host_build():
         ops.SynapseTable.from_edges(src, tgt + n_cols, w, d, r, n_rows, n_cols)
 
 
-@pytest.mark.parametrize("batch", [1, 64])
-def test_auto_delivery_picks_a_form_on_the_device_and_both_give_the_oracle_ring(batch):
-    """`csr_propagate_fwd("auto")`: the active count decides on the device between the event-driven and the row-wise
-    form.  Quarter-pA weights: whichever runs, the ring must equal the fp32 oracle's bit for bit -- with a
-    threshold below, at and above the actual count, and with nothing active."""
+@pytest.mark.parametrize("batch", [1, 24, 64])
+def test_auto_delivery_picks_a_form_on_the_device_and_the_ring_is_the_oracles(batch):
+    """``ops.AutoPropagator`` (bmtk_csr_propagate_auto): step by step the active count decides on the device whether
+    a step's spikes are pushed into the ring as events or left to the pull over the spike history.  A run whose
+    activity goes from nothing to 20 % and back mixes the two forms in every way -- pushed steps between pulled
+    ones, arrival slots that hold pushed weights when the pull adds its sums, stretches with nothing to pull.
+    Quarter-pA weights: after every call the arrival slot must equal the fp32 oracle's bit for bit, whatever the
+    mix, also with thresholds that force one form throughout."""
     rng = np.random.default_rng(33)
-    n, L = 500, 6
+    n, L, T = 500, 6, 40
     src, tgt, w, d, r = _edges(rng, n, n, 30000)
     w = (np.round(w * 4) / 4 + np.sign(w) * 0.25).astype(np.float32)
     by_src = net.coo_to_csr(src, tgt, w, d, r, n_rows=n, major="source")
     by_tgt = net.csr_transpose(by_src, n)
     t_src, t_tgt = ops.SynapseTable.from_numpy(by_src), ops.SynapseTable.from_numpy(by_tgt)
-    comp = ops.SpikeCompactor(n * batch)
-    for p in (0.0, 0.01, 0.2):
-        z = (rng.random(n * batch) < p).astype(np.uint8)
-        count = int(z.sum())
-        want = np.zeros((L, 4, n * batch), np.float32)
-        orc.gather_rows(z, batch, by_tgt, want, n, 4)
-        for thr in (0, max(count - 1, 0), count, count + 1, None):
-            ring = torch.zeros(L, 4, n * batch, device="cuda")
-            ids, cnt = comp(to_dev(z))
-            ops.csr_propagate_fwd("auto", t_src, ring, n, batch, 4, active=ids, n_active=cnt, zbits=to_dev(bits_of(z)),
-                                  n_src=n, table_tgt=t_tgt, scatter_max_active=thr)
-            np.testing.assert_array_equal(ring.cpu().numpy(), want, err_msg="p=%g threshold=%s" % (p, thr))
+    ne = n * batch
+    comp = ops.SpikeCompactor(ne)
+    rates = [0.0, 0.0, 0.002, 0.2, 0.002, 0.0, 0.2, 0.2, 0.01, 0.002] * 4
+    zs = [(rng.random(ne) < rates[k]).astype(np.uint8) for k in range(T)]
+    counts = sorted(int(z.sum()) for z in zs)
+    mid = counts[len(counts) // 2]
+    for thr in (mid, 0, ne, counts[-1] - 1):
+        want = np.zeros((L, 4, ne), np.float32)
+        hist = torch.zeros(L, ops.n_words(ne) + 1, dtype=torch.int64, device="cuda")
+        ring = torch.zeros(L, 4, ne, device="cuda")
+        auto = ops.AutoPropagator(t_src, t_tgt, hist, ring, n, n, batch, scatter_max_active=thr)
+        seen = set()
+        for k in range(T):
+            orc.gather_rows(zs[k], batch, by_tgt, want, n, k)
+            hist[k % L] = to_dev(bits_of(zs[k]))
+            ids, cnt = comp(to_dev(zs[k]))
+            auto.step(k, ids, cnt)
+            seen.add(bool(auto.pulled_steps()[k % L]))
+            slot = (k + 1) % L
+            np.testing.assert_array_equal(ring[slot].cpu().numpy(), want[slot], err_msg="step %d threshold %d" % (k, thr))
+            ring[slot].zero_()        # the consumer's part: the slot is read and cleared before the next call
+            want[slot] = 0.0
+        assert np.abs(want).max() > 0 or thr == mid
+        if thr == mid:
+            assert seen == {True, False}      # both forms ran
+        elif thr == 0:
+            assert seen == {True} or 0 in counts
+        elif thr == ne:
+            assert seen == {False}
