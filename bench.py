@@ -349,6 +349,44 @@ def bench_bptt(torch, steps=600):
     return entries
 
 
+def bench_batched_v1(torch, batch=8, steps=300):
+    """The V1-scale network as a batched run, 230,924 neurons x 8 trials, from the settled state, through the
+    launch-per-step driver in the form the simulator picks by itself at this batch and rate (spikes pushed into the
+    ring as events: 0.02 events per synapse and step) and through the fused pull form (248 k sources, so one bit of
+    its activity map stands for several).  Algorithmic bytes: 18 B per synaptic event + 103 B per element update."""
+    import numpy as np
+    from bmtk_amd import ops, synthetic, training
+    from bmtk_amd.simulator import Glif3Simulator
+    rng = np.random.default_rng(3)
+    par = synthetic.random_cells(rng, N_CLASSES)
+    class_id = rng.integers(0, N_CLASSES, N_V1).astype(np.int32)
+    _, by_src, _ = synthetic.device_network(N_V1, MEAN_IN, "lognormal", seed=3)
+    inp = synthetic.device_input_table(N_IN, N_V1, N_IN_SYN, seed=4, w_scale=IN_W_SCALE)
+    in_ptr, in_ev = ops.poisson_events(N_IN, IN_RATE_HZ, 1.0, 600 + 2 * steps, batch=batch, seed=5)
+    out = []
+    for form, kw in (("the simulator's choice", dict()), ("fused pull form", dict(fused=True))):
+        sim = Glif3Simulator(N_V1, par, 1.0, batch=batch, class_id=class_id, rec=by_src, inp=inp, resident=False, **kw)
+        sim.set_input_events(in_ptr, in_ev)
+        sim.run(600, spike_bits=False)
+        sim.run(steps // 4, spike_bits=False)
+        res = {}
+        wall, dev = time_region(torch, lambda: res.update(out=sim.run(steps)))
+        spikes = int(training.spike_counts(res["out"]["bits"], sim.ne).sum().item())
+        rec_ev, inp_ev = count_events(torch, sim, res["out"]["bits"], 600 + steps // 4)
+        per = dev / steps
+        alg = (rec_ev + inp_ev) / steps * B_PER_EVENT + sim.ne * B_PER_UPDATE_CLASS
+        out.append({"kernel": "sim_fused_kernel" if sim.fuse_table is not None else "sim_step_kernel",
+                    "workload": "V1-scale batched run: 230,924 neurons x %d trials, %d steps, %s" % (batch, steps, form),
+                    "activity_map_sources_per_bit": 1 << sim.fuse_shift if sim.fuse_table is not None else None,
+                    "us_per_sim_step": per * 1e6, "neuron_updates_per_s": sim.ne / per,
+                    "synaptic_events_per_s": (rec_ev + inp_ev) / dev, "mean_rate_hz": spikes / (sim.ne * steps * 1e-3),
+                    "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                                 "what": "18 B per synaptic event + 103 B per element update"}})
+        del sim
+    return out
+
+
 def bench_small_network(torch):
     """The size of the reference's own examples: configuration 0's 450 neurons, which ONE workgroup holds (the
     single-workgroup form of the resident kernel), with the spike record on as the front ends run it."""
@@ -511,6 +549,9 @@ def kernel_summary(kernels):
                                 "forward_us_per_step": k["forward_s"] / 600 * 1e6,
                                 "backward_frac": r.get("frac"), "forward_frac": k["roofline_forward"]["frac"],
                                 "weight_grad_events_per_s": k["weight_grad_events_per_s"]}
+        elif w.startswith("V1-scale batched run"):
+            out["v1_scale_batch_8, " + ("fused pull form" if "fused" in w else "the simulator's choice")] = {"us_per_sim_step": k["us_per_sim_step"], "neuron_updates_per_s": k["neuron_updates_per_s"],
+                                       "synaptic_events_per_s": k["synaptic_events_per_s"], "frac": r.get("frac")}
         elif w.startswith("transposed propagation"):
             out.setdefault("transposed_propagation_us", {})[k["kernel"]] = round(k["us_per_launch"], 1)
     return out
@@ -527,7 +568,7 @@ def main():
                     help="simulation steps per pass (the configuration's 3000)")
     ap.add_argument("--cpu-steps", type=int, default=3000, help="steps of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the isolated-kernel measurements")
-    ap.add_argument("--kernels", default="state,compaction,propagation,bptt",
+    ap.add_argument("--kernels", default="state,compaction,propagation,bptt,batched_v1",
                     help="which isolated-kernel measurements to run (comma-separated)")
     ap.add_argument("--propagation-modes", default=",".join(PROPAGATION_MODES),
                     help="delivery forms the propagation group times (profiler runs leave out 'auto', which launches "
@@ -563,7 +604,7 @@ def main():
         sys.exit("bench.py: --propagation-modes takes %s" % ", ".join(PROPAGATION_MODES))
     groups = {"state": bench_state_update, "compaction": bench_compaction,
               "propagation": lambda t: bench_propagation(t, modes=modes), "bptt": bench_bptt,
-              "small": bench_small_network}   # (the headline run reports "small" with its front-end entries)
+              "small": bench_small_network, "batched_v1": bench_batched_v1}   # (the headline run reports "small" with its front-end entries)
     want = [g for g in args.kernels.split(",") if g]
     unknown = set(want) - set(groups)
     if unknown:

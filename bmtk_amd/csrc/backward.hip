@@ -213,6 +213,7 @@ __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, B
 // over the ranges seen so far waits in LDS (16 bytes per lane and row, lane-private, so no barriers), which is
 // what bounds the rows of a sweep: 16 wavefronts x gpw row groups x 64/lp rows.  The eight XCDs each see every
 // row for their own ranges and write a partial sum of their own, gz[x][ne]; the state adjoint adds the eight.
+__device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves);
 constexpr int kBlkThreads = 1024;
 constexpr int kBlkWaves = kBlkThreads / kWave;
 constexpr int kBlkMaxGroups = 8;  // row groups per wavefront and sweep: one byte of trial masks each in a 64-bit register
@@ -229,9 +230,9 @@ __device__ __forceinline__ float dpp_move(float x)
 // kNe24: n_neurons*batch < 2^24, so that the cell arithmetic can use 24-bit multiplies; kWide: lp >= 8
 template <bool kGrad, bool kNe24, bool kWide>
 __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_glif3_bwd a, BwdStep q, int lp, int rows_cu,
-                                                                         int sweeps, int gpw)
+                                                                         int sweeps, int gpw, int use_order, int do_inp)
 {
-    extern __shared__ float4 blk_acc[];  // [kBlkWaves][gpw][kWave]
+    extern __shared__ float4 blk_acc[];  // [kBlkWaves][gpw][kWave], then the row order (uint16 per place)
     constexpr int kF = kBlkInFlight;
     const int batch = a.batch;
     const int64_t n = a.n_neurons, ne = n * batch;
@@ -259,13 +260,66 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_gl
         return (elem << 2) + lane_off;
     };
     float4 *acc = blk_acc + (size_t)wave * gpw * kWave + lane;
+    // Which row a lane group works on.  The workgroup's rows are taken in groups of `per` (a wavefront's lane groups
+    // side by side), group g by wavefront g % 16 as its (g / 16)-th.  With the gradient riding along, the rows
+    // whose source fired in this step come first in that order (a list in LDS, built once per launch): a wavefront
+    // runs the gradient's extra work whenever ONE of its rows fired, so with a tenth of the rows firing and eight
+    // rows side by side more than half of all visits ran it, seven eighths idle; gathered into the first groups
+    // the fired rows fill a tenth of the visits, dealt out evenly over the wavefronts.
+    uint16_t *order = reinterpret_cast<uint16_t *>(blk_acc + (size_t)kBlkWaves * gpw * kWave);
+    const int places = sweeps * kBlkWaves * gpw * per;
+    if (kGrad && use_order) {
+        __shared__ unsigned scan_l[2][kBlkWaves];
+        const uint64_t *__restrict__ bits = a.spike_bits + q.row * a.spike_bits_stride;
+        // a thread looks at rows threadIdx.x, threadIdx.x + 1024, ... (at most 16): fired or not, one bit each
+        unsigned fm = 0u, n_mine = 0u;
+        for (int i = 0; (int)threadIdx.x + i * kBlkThreads < rows_cu; ++i) {
+            const int64_t j = row_lo + threadIdx.x + i * kBlkThreads;
+            if (j < row_hi && trial_mask(bits, j, batch, 0, batch) != 0ull) fm |= 1u << i;
+            ++n_mine;
+        }
+        const unsigned c1 = (unsigned)__popc(fm), c0 = n_mine - c1;
+        const unsigned in1 = wave_inclusive_scan(c1), in0 = wave_inclusive_scan(c0);
+        if (lane == kWave - 1) {
+            scan_l[0][wave] = in0;
+            scan_l[1][wave] = in1;
+        }
+        __syncthreads();
+        unsigned base0 = 0u, base1 = 0u, total1 = 0u;
+#pragma unroll
+        for (int w = 0; w < kBlkWaves; ++w) {
+            if (w < wave) {
+                base0 += scan_l[0][w];
+                base1 += scan_l[1][w];
+            }
+            total1 += scan_l[1][w];
+        }
+        unsigned p1 = base1 + in1 - c1, p0 = total1 + base0 + in0 - c0;  // next place among the fired / the others
+        for (unsigned i = 0; i < n_mine; ++i) {
+            const unsigned local = threadIdx.x + i * kBlkThreads;
+            if ((fm >> i) & 1u)
+                order[p1++] = (uint16_t)local;
+            else
+                order[p0++] = (uint16_t)local;
+        }
+        for (int i = rows_cu + (int)threadIdx.x; i < places; i += kBlkThreads) order[i] = 0xFFFFu;  // places without a row
+        __syncthreads();
+    }
+    // row of lane group `grp` in the wavefront's k-th group of sweep sw (row_hi and beyond: none)
+    auto row_of = [&](int sw, int k) -> int64_t {
+        const int place = ((sw * gpw + k) * kBlkWaves + wave) * per + grp;
+        if (kGrad && use_order) {
+            const unsigned local = order[place];
+            return local == 0xFFFFu ? row_hi : row_lo + local;
+        }
+        return place < rows_cu ? row_lo + place : row_hi;
+    };
     for (int sw = 0; sw < sweeps; ++sw) {
-        const int64_t jw = row_lo + ((int64_t)sw * kBlkWaves + wave) * gpw * per + grp;  // this lane's row of group 0
         // per row group one byte: bits 0-3 the lane's trials with a non-zero surrogate derivative in this step,
         // bits 4-7 those in which the source fired (kGrad)
         unsigned long long masks = 0ull;
         for (int k = 0; k < gpw; ++k) {
-            const int64_t j = jw + (int64_t)k * per;
+            const int64_t j = row_of(sw, k);
             unsigned act = 0u, mine = 0u;
             if (j < row_hi && lane_on) {
                 const int64_t e = j * batch + b4;
@@ -293,7 +347,7 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_gl
             p = p1 = 0;
             if (ph >= P) return;
             const bool want = ((masks >> (8 * k)) & 0xFFull) != 0ull;
-            const int64_t j = jw + (int64_t)k * per;
+            const int64_t j = row_of(sw, k);
             if ((__ballot(want) & grp_lanes) != 0ull && j < row_hi) {
                 const int32_t *__restrict__ ip = a.blk_indptr + (int64_t)(x * P + ph) * n + j;
                 p = ip[0];
@@ -419,7 +473,7 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_gl
             }
         }
         for (int k = 0; k < gpw; ++k) {
-            const int64_t j = jw + (int64_t)k * per;
+            const int64_t j = row_of(sw, k);
             if (j < row_hi && lane_on) {
                 const unsigned act = (unsigned)(masks >> (8 * k)) & 0xFu;
                 const float4 t = acc[k * kWave];
@@ -429,14 +483,18 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_gl
             }
         }
     }
+    // The input-weight gradient of the same step (it reads the same adjoint slots): a few thousand runs of events,
+    // each a chain of dependent reads for one wavefront.  Done here by whichever wavefronts are through with their
+    // rows, it disappears in this kernel's tail; beside the state adjoint it lengthened that launch by 20 us.
+    if (do_inp) bwd_inp_grad_waves(a, q, (int)blockIdx.x * kBlkWaves + wave, (int)gridDim.x * kBlkWaves);
 }
 
 // state adjoint of one step, one thread per element; writes the adjoint of
 // this step's arrivals into ring slot t
-__global__ __launch_bounds__(kBlock) void bwd_state_kernel(bmtk_glif3_bwd a, BwdStep q)
+__device__ __forceinline__ void bwd_state_block(const bmtk_glif3_bwd &a, const BwdStep &q, int64_t block)
 {
     const int64_t ne = a.n_neurons * (int64_t)a.batch;
-    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t e = block * kBlock + threadIdx.x;
     if (e >= ne) return;
     const int64_t n = a.batch == 1 ? e : (int64_t)((uint32_t)e / (uint32_t)a.batch);
     const int64_t col = a.class_id ? (int64_t)a.class_id[n] : n;
@@ -539,16 +597,21 @@ __global__ __launch_bounds__(kBlock) void bwd_rec_grad_kernel(bmtk_glif3_bwd a, 
 #define BWD_INP_GRID 1024
 #endif
 constexpr int kInpGradGrid = BWD_INP_GRID;
-__global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, BwdStep q)
+// (a workgroup of any size: wavefront `wave` of `n_waves`)
+__device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves);
+__device__ __forceinline__ void bwd_inp_grad_block(const bmtk_glif3_bwd &a, const BwdStep &q, int block, int n_blocks)
+{
+    bwd_inp_grad_waves(a, q, block * (kBlock / kWave) + threadIdx.x / kWave, n_blocks * (kBlock / kWave));
+}
+__device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves)
 {
     const int batch = a.batch;
     const int64_t ne = a.n_neurons * (int64_t)batch;
     const int L = a.ring_slots;
     const int slot0 = (int)(q.t % L);
     const int64_t k0 = a.in_ptr[q.t], k1 = a.in_ptr[q.t + 1];
-    const int n_waves = gridDim.x * (kBlock / kWave);
     const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.inp_packed);
-    for (int64_t k = k0 + blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; k < k1; k += n_waves) {
+    for (int64_t k = k0 + wave; k < k1; k += n_waves) {
         const int ev = a.in_events[k];
         const int j = batch == 1 ? ev : (int)((uint32_t)ev / (uint32_t)batch);
         if (k > k0 && (batch == 1 ? a.in_events[k - 1] : (int)((uint32_t)a.in_events[k - 1] / (uint32_t)batch)) == j)
@@ -587,6 +650,18 @@ __global__ __launch_bounds__(kBlock) void bwd_inp_grad_kernel(bmtk_glif3_bwd a, 
                 if (base + u * kWave < p1) a.d_inp_w[base + u * kWave] = old[u] + acc[u];
         }
     }
+}
+
+// The state adjoint of step t and the input-weight gradient of the same step in one launch, side by side: the
+// gradient reads the adjoint slots t+1 .. t+L-1 and the step's events, the state adjoint writes slot t -- neither
+// needs the other.  The gradient's workgroups (a chain of dependent reads per event run, few wavefronts) take the
+// lowest block ids so that they start first and run under the streaming state adjoint instead of after it.
+__global__ __launch_bounds__(kBlock) void bwd_state_kernel(bmtk_glif3_bwd a, BwdStep q, int n_inp_blocks)
+{
+    if ((int)blockIdx.x < n_inp_blocks)
+        bwd_inp_grad_block(a, q, (int)blockIdx.x, n_inp_blocks);
+    else
+        bwd_state_block(a, q, (int64_t)blockIdx.x - n_inp_blocks);
 }
 
 __global__ __launch_bounds__(kBlock) void fill_zero_kernel(float *x, int64_t n)
@@ -629,9 +704,10 @@ const void *blocked_variant(bool grad, bool ne24, bool wide)
 // launch geometry of bwd_gather_blocked_kernel for a network on the current device
 struct BlockedPlan {
     unsigned grid;
-    int lp, rows_cu, sweeps, gpw;
+    int lp, rows_cu, sweeps, gpw, use_order;
     size_t lds;
 };
+constexpr size_t kBlkLdsMax = 160u * 1024u - 256u;  // a compute unit's LDS less the kernel's static part
 
 int blocked_plan(const bmtk_glif3_bwd &a, BlockedPlan &pl)
 {
@@ -657,13 +733,17 @@ int blocked_plan(const bmtk_glif3_bwd &a, BlockedPlan &pl)
     pl.rows_cu = (int)rows_cu;
     pl.grid = (unsigned)cus * 8u;
     pl.lds = (size_t)kBlkWaves * pl.gpw * kWave * sizeof(float4);
+    // the row order list (gradient riding along): two bytes per place, where it fits (up to 16 rows per thread)
+    const size_t order_bytes = (size_t)pl.sweeps * kBlkWaves * pl.gpw * per * sizeof(uint16_t);
+    pl.use_order = (pl.lds + order_bytes <= kBlkLdsMax && rows_cu <= 16 * kBlkThreads && rows_cu < 0xFFFF) ? 1 : 0;
+    if (pl.use_order) pl.lds += order_bytes;
     static bool asked[8][64];
     const void *variants[8];
     for (int g = 0; g < 8; ++g) variants[g] = blocked_variant(g & 4, g & 2, g & 1);
     for (int g = 0; g < 8; ++g) {
         if (dev < 0 || dev >= 64 || asked[g][dev]) continue;
         const hipError_t err = hipFuncSetAttribute(
-            variants[g], hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kBlkWaves * kBlkMaxGroups * kWave * sizeof(float4)));
+            variants[g], hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlkLdsMax);
         if (err != hipSuccess) {
             set_error("transposed propagation: cannot reserve LDS: %s", hipGetErrorString(err));
             return BMTK_E_LAUNCH;
@@ -685,13 +765,15 @@ int blocked_check(const bmtk_glif3_bwd &a, const char *who)
     return BMTK_OK;
 }
 
-int blocked_launch(const bmtk_glif3_bwd &a, const BwdStep &q, const BlockedPlan &pl, bool grad, hipStream_t st)
+int blocked_launch(const bmtk_glif3_bwd &a, const BwdStep &q, const BlockedPlan &pl, bool grad, bool inp_grad,
+                   hipStream_t st)
 {
     const bool ne24 = a.n_neurons * (int64_t)a.batch < (1ll << 24);
     bmtk_glif3_bwd args = a;
     BwdStep step = q;
-    int lp = pl.lp, rows_cu = pl.rows_cu, sweeps = pl.sweeps, gpw = pl.gpw;
-    void *params[] = {&args, &step, &lp, &rows_cu, &sweeps, &gpw};
+    int lp = pl.lp, rows_cu = pl.rows_cu, sweeps = pl.sweeps, gpw = pl.gpw, use_order = pl.use_order;
+    int do_inp = inp_grad ? 1 : 0;
+    void *params[] = {&args, &step, &lp, &rows_cu, &sweeps, &gpw, &use_order, &do_inp};
     const hipError_t err = hipLaunchKernel(blocked_variant(grad, ne24, pl.lp >= 8), dim3(pl.grid), dim3(kBlkThreads),
                                            params, pl.lds, st);
     if (err != hipSuccess) {
@@ -748,7 +830,7 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
         // their own (several wavefronts would share a row).
         const bool fused = blocked ? a.d_blk_w != nullptr : (a.d_rec_w && tiles == 1);
         if (blocked) {
-            const int rc = blocked_launch(a, q, pl, fused, st);
+            const int rc = blocked_launch(a, q, pl, fused, inp_grad, st);
             if (rc != BMTK_OK) return rc;
         } else if (has_rec && a.batch % 4 == 0 && a.batch <= kWave) {
             if (fused)
@@ -763,9 +845,9 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
         } else {
             hipLaunchKernelGGL(fill_zero_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a.gz, ne);
         }
-        hipLaunchKernelGGL(bwd_state_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q);
+        const int n_inp_blocks = (inp_grad && !blocked) ? kInpGradGrid : 0;  // (the blocked kernel took it along)
+        hipLaunchKernelGGL(bwd_state_kernel, dim3(elem_grid + n_inp_blocks), dim3(kBlock), 0, st, a, q, n_inp_blocks);
         if (a.d_rec_w && !fused) hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
-        if (inp_grad) hipLaunchKernelGGL(bwd_inp_grad_kernel, dim3(kInpGradGrid), dim3(kBlock), 0, st, a, q);
     }
     BMTK_CHECK_LAUNCH("glif3_simulate_bwd");
     return BMTK_OK;
@@ -826,7 +908,7 @@ extern "C" int bmtk_csr_propagate_bwd_blocked(const int32_t *blk_indptr, const b
     if (rc == BMTK_OK) rc = blocked_plan(a, pl);
     if (rc != BMTK_OK) return rc;
     BwdStep q{step, 0, 8};
-    rc = blocked_launch(a, q, pl, false, (hipStream_t)stream);
+    rc = blocked_launch(a, q, pl, false, false, (hipStream_t)stream);
     if (rc != BMTK_OK) return rc;
     BMTK_CHECK_LAUNCH("csr_propagate_bwd_blocked");
     return BMTK_OK;

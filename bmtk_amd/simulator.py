@@ -16,6 +16,7 @@ from .ops import Glif3State, SpikeCompactor, SynapseTable, _dev, _p, _stream, gl
 
 
 PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what is left of 80 KB beside its accumulators
+PULL_MIN_DENSITY = 0.06         # synaptic events per synapse and step from which "auto" pulls instead of pushing
 FUSE_LDS_BYTES = 80 * 1024      # LDS of one workgroup of the fused batched driver (kFuseLdsMax of csrc/simulate_fused.hip)
 FUSE_WAVES = 16                 # wavefronts of one of its workgroups (kFuseWaves)
 FUSE_BATCHES = (8, 16, 32, 64)  # lane = trial, whole bytes of spike bits per neuron
@@ -68,17 +69,23 @@ class Glif3Simulator:
                 as a short list beside its ballots, and the others read the lists instead of expanding the whole
                 network's ballots (steps in which a list does not suffice are read from the ballots); False: always
                 from the ballots.  Same results either way.
+    expected_rate_hz  what "auto" decides ``pull`` / ``fused`` by.  Pushing spikes into the ring costs an atomic per
+                synaptic event, pulling a pass over the whole table per step whatever the activity; a synapse
+                carries batch * rate * h events per step, and on one MI355X the pass is the cheaper of the two from
+                about 0.06 events per synapse and step (measured: 51,978 neurons x 32 trials at 3.2 Hz pull 168 us
+                against 340 pushed; 230,924 neurons x 8 and x 16 at 2.8 Hz pushed 132 / 237 us against 321 / 358
+                pulled).  Default 3 Hz: batches from 20 at 1 ms steps.
     fused       launch-per-step mode, batch 8, 16, 32 or 64, delay_offset 0: one launch per step in which a
                 wavefront sums what arrives at a neuron -- over recurrent and input synapses, from a joint
                 target-major table and a joint history of spike and input-event bits -- and advances the neuron's
-                trials, lane = trial; no arrival sum passes through device memory.  "auto": whenever ``pull`` would
-                apply and the batch is one of those; takes any number of sources (above what the activity map in
+                trials, lane = trial; no arrival sum passes through device memory.  "auto": whenever ``pull``
+                "auto" would pull and the batch is one of those; takes any number of sources (above what the activity map in
                 LDS holds, one bit of the map stands for 2, 4, ... sources).  False: the pull form as separate
                 launches (below).  ``ring`` then holds only the few input ids repeated within a step.
     pull        launch-per-step mode only: sum the recurrent arrivals of a step in one pass over a target-major
                 copy of the table from the spike-bit history, instead of pushing them into the ring with global
-                atomics as spikes occur -- the faster form for batched runs.  "auto": batch >= 8 (and delay_offset
-                0, network small enough for the activity map in LDS).  Recurrent arrivals still ahead at the end
+                atomics as spikes occur -- the faster form for batched runs.  "auto": by ``expected_rate_hz``
+                (and delay_offset 0, network small enough for the activity map in LDS).  Recurrent arrivals still ahead at the end
                 of a run then live in the history, and ``ring`` holds the input arrivals only.
     delay_offset  B steps taken off every delay before the tables are built; spikes and input events are
                 then handed to the tables B steps late from a history of spike bits, which gives the same
@@ -92,7 +99,8 @@ class Glif3Simulator:
 
     def __init__(self, n_neurons, par, h, batch=1, class_id=None, rec=None, inp=None, ring_slots=None,
                  asc_init=None, u_init=None, i_ext=None, device=None, resident="auto", delay_offset="auto",
-                 pull="auto", single_workgroup=True, fired_lists=True, fused="auto", fuse_wg_per_cu=0):
+                 pull="auto", single_workgroup=True, fired_lists=True, fused="auto", fuse_wg_per_cu=0,
+                 expected_rate_hz=3.0):
         self.lib = _lib.load()
         self.dev = device or _dev()
         self.n, self.batch, self.h = int(n_neurons), int(batch), float(h)
@@ -222,7 +230,9 @@ class Glif3Simulator:
         def fixed_point_ok(t):
             w = t.weights
             return not w.numel() or bool(torch.isfinite(w).all() & (w.abs().max() < 2.0 ** 31))
-        if can_pull and (pull is True or (pull == "auto" and self.batch >= 8)):
+        # events per synapse and step at the expected rate: from PULL_MIN_DENSITY on a pass over the table is cheaper
+        dense = self.batch * float(expected_rate_hz) * 1e-3 * self.h >= PULL_MIN_DENSITY
+        if can_pull and (pull is True or (pull == "auto" and dense)):
             if not (fixed_point_ok(self.rec) and (self.inp is None or fixed_point_ok(self.inp))):
                 if pull is True:
                     raise ValueError("the pull form needs finite weights smaller than 2^31 in size")
@@ -230,7 +240,7 @@ class Glif3Simulator:
         if pull is True and not can_pull:
             raise ValueError("the pull form needs a recurrent table, launch-per-step mode, delay_offset 0 and "
                              "ring_slots * n_neurons / 8 bytes of LDS (at most 40 KB)")
-        if can_fuse and fused and (fused is True or pull is True or self.batch >= 8):
+        if can_fuse and fused and (fused is True or pull is True or dense):
             tables = [t for t in (self.rec, self.inp) if t is not None]
             if all(fixed_point_ok(t) for t in tables):
                 self._setup_fused()
@@ -238,7 +248,7 @@ class Glif3Simulator:
                 raise ValueError("the fused form needs finite weights smaller than 2^31 in size")
         if self.fuse_table is not None:
             pass
-        elif can_pull and (pull is True or (pull == "auto" and self.batch >= 8)):
+        elif can_pull and (pull is True or (pull == "auto" and dense)):
             self.pull_table = self.rec.transposed(self.n)
             self.pull_syn = torch.zeros(NREC, self.ne, device=self.dev)
             need = self.lib.bmtk_csr_propagate_pull_workspace_bytes(self.L, self.n)

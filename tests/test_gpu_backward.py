@@ -107,9 +107,9 @@ def test_weight_gradients_with_input_ids_repeated_within_a_step(batch):
     assert in_events.size > 1.15 * cfg["in_events"].size
     prop = orc.precompute(cfg["par"], h)
     sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
-                         resident=False)
+                         resident=False, pull=batch >= 8)
     sim.set_input_events(in_ptr, in_events)
-    assert sim.in_duplicates and (batch < 8 or sim.in_repeat_ptr is not None)
+    assert sim.in_duplicates and (batch < 8 or (sim.fuse_table is not None and sim.in_repeat_ptr is not None))
     fwd = sim.run(T, save_state=True)
     ras = sim.raster(fwd["bits"]).cpu().numpy()
     a = np.random.default_rng(6).normal(size=(T, n * batch))

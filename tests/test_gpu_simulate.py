@@ -314,9 +314,11 @@ def test_pull_form_of_the_per_step_driver(batch):
             np.testing.assert_array_equal(got[k], st[k], err_msg=k)
     auto = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
                           resident=False)
-    # batched runs pull; batches whose trials fill whole bytes of spike bits take the fused form of it
-    assert (auto.fuse_table is not None) == (batch in (8, 16, 32, 64))
-    assert (auto.pull_table is not None) == (batch >= 8 and auto.fuse_table is None)
+    # at the expected 3 Hz and 1 ms steps batches from 20 pull, in the fused form (trials fill whole bytes of bits)
+    assert (auto.fuse_table is not None) == (batch in (32, 64)) and auto.pull_table is None
+    busy = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
+                          resident=False, expected_rate_hz=40.0)
+    assert (busy.pull_table is not None) == (batch == 3) and (busy.fuse_table is not None) == (batch != 3)
 
 
 def test_resident_pull_with_more_fired_rows_than_its_list_holds():
@@ -443,10 +445,10 @@ def test_repeated_input_events_within_a_step_are_all_delivered(batch, resident):
     if resident == "many":       # 700 neurons on a dozen workgroups instead of one
         kw = dict(resident=True, single_workgroup=False)
     elif resident == "unfused":  # the batched driver with pull and update as separate launches
-        kw = dict(resident=False, fused=False)
+        kw = dict(resident=False, fused=False, pull=True)
         resident = False
     else:
-        kw = dict(resident=resident)
+        kw = dict(resident=resident, pull=True) if batch >= 8 else dict(resident=resident)
     sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=batch, class_id=cfg["class_id"], rec=cfg["rec_src"],
                          inp=cfg["inp_src"], ring_slots=cfg["L"], **kw)
     assert sim.res_groups == (0 if not resident else 1 if resident is True else 11)
