@@ -387,6 +387,44 @@ def bench_batched_v1(torch, batch=8, steps=300):
     return out
 
 
+def bench_lds(torch, clock_ghz=2.4):
+    """What the LDS and the path between workgroups cost (the figures the resident kernels' design quotes):
+    additions into a 92 KB LDS array in five forms with 64, 8 and 1 active lanes per wavefront, in clocks per
+    wavefront instruction on a compute unit at a nominal 2.4 GHz, and the time a word takes from one workgroup to
+    another through device memory, on one XCD and across two."""
+    from bmtk_amd import _lib
+    from bmtk_amd.ops import _p, _stream
+    lib = _lib.load()
+    n_blocks, rounds = 256, 2000
+    out_buf = torch.empty(n_blocks * 1024, device="cuda")
+    names = {0: "ds_add_f32", 1: "ds_add_u32", 2: "ds_add_u64", 3: "float add by compare-and-swap loop", 4: "plain store"}
+    entries = []
+    for op in range(5):
+        row = {}
+        for active in (64, 8, 1):
+            call = lambda: _lib.check(lib.bmtk_microbench_lds(op, active, rounds, n_blocks, _p(out_buf), _stream()))
+            call()
+            _, dev = time_region(torch, lambda: [call() for _ in range(5)])
+            clk = dev / 5 * clock_ghz * 1e9 / (16.0 * rounds)     # 16 wavefronts per compute unit, one workgroup each
+            row[str(active) + " lanes"] = {"clocks_per_wavefront_instruction": clk, "clocks_per_lane": clk / active}
+        entries.append({"kernel": "lds_add_kernel", "workload": "LDS addition, " + names[op], "result": row,
+                        "clock_ghz_assumed": clock_ghz})
+    flags = torch.zeros(1024, dtype=torch.int32, device="cuda")
+    xcc = torch.zeros(4, dtype=torch.int32, device="cuda")
+    hop_rounds = 20000
+    for a, b, what in ((0, 8, "workgroups 0 and 8"), (0, 1, "workgroups 0 and 1")):
+        best = None
+        for _ in range(3):
+            flags.zero_(); xcc.zero_()
+            _, dev = time_region(torch, lambda: _lib.check(lib.bmtk_microbench_hop(_p(flags), _p(xcc), a, b, hop_rounds,
+                                                                                   1_000_000, _stream())))
+            best = dev if best is None else min(best, dev)
+        x = xcc.cpu().tolist()
+        entries.append({"kernel": "hop_kernel", "workload": "word passed between two workgroups through device memory, " + what,
+                        "xcd_of_each": x[:2], "gave_up": bool(x[2]), "us_per_hop": best / hop_rounds / 2 * 1e6})
+    return entries
+
+
 def bench_small_network(torch):
     """The size of the reference's own examples: configuration 0's 450 neurons, which ONE workgroup holds (the
     single-workgroup form of the resident kernel), with the spike record on as the front ends run it."""
@@ -604,7 +642,7 @@ def main():
         sys.exit("bench.py: --propagation-modes takes %s" % ", ".join(PROPAGATION_MODES))
     groups = {"state": bench_state_update, "compaction": bench_compaction,
               "propagation": lambda t: bench_propagation(t, modes=modes), "bptt": bench_bptt,
-              "small": bench_small_network, "batched_v1": bench_batched_v1}   # (the headline run reports "small" with its front-end entries)
+              "small": bench_small_network, "batched_v1": bench_batched_v1, "lds": bench_lds}   # (the headline run reports "small" with its front-end entries)
     want = [g for g in args.kernels.split(",") if g]
     unknown = set(want) - set(groups)
     if unknown:

@@ -15,7 +15,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB = os.path.join(PKG, "libbmtk_amd.so")
-SOURCES = ["kernels.hip", "propagate_pull.hip", "simulate.hip", "simulate_fused.hip", "resident.hip", "resident_solo.hip", "backward.hip", "poisson.hip"]
+SOURCES = ["kernels.hip", "propagate_pull.hip", "simulate.hip", "simulate_fused.hip", "resident.hip", "resident_solo.hip", "backward.hip", "poisson.hip", "microbench.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
          "-munsafe-fp-atomics", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wall", "-Wno-unused-function"]

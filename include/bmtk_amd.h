@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 19
+#define BMTK_AMD_ABI_VERSION 20
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -518,6 +518,23 @@ int bmtk_csr_propagate_bwd_blocked_plan(int64_t n_neurons, int32_t batch, int32_
 /* Number of spikes of every element over n_steps rows of spike bits: counts[e] (int32). */
 int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_steps, int64_t ne, int32_t *counts,
                       void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Two measurements the kernels' design rests on, kept in the library so that they can be repeated
+ * (bench.py --kernels lds).  No counterpart in the reference.
+ *
+ * bmtk_microbench_lds: n_blocks workgroups of 1024 threads; in each of `rounds` rounds, `active_lanes` lanes of every
+ * wavefront add to a pseudo-random cell of a 92,160-byte LDS array.  op 0: float atomic (ds_add_f32), 1: 32-bit
+ * integer atomic, 2: 64-bit integer atomic, 3: float add by a compare-and-swap loop, 4: plain store.  out: n_blocks *
+ * 1024 floats (checksums).  The caller times the launch; time * clock / (16 * rounds) = clocks per wavefront
+ * instruction on a compute unit.
+ * bmtk_microbench_hop: workgroups block_a and block_b (0..15; workgroups go round the XCDs, so 0 and 8 share one, 0
+ * and 1 do not) pass a counter back and forth `rounds` times through two words of `flags` (at least 512 bytes,
+ * zeroed by the caller) with relaxed agent-scope loads and stores; time / rounds = two hops.  xcc (3 words, zeroed
+ * by the caller): the XCD each ran on, and 1 in xcc[2] if a wait ran out after spin_limit polls (both then leave). */
+int bmtk_microbench_lds(int32_t op, int32_t active_lanes, int32_t rounds, int32_t n_blocks, float *out, void *stream);
+int bmtk_microbench_hop(uint32_t *flags, uint32_t *xcc, int32_t block_a, int32_t block_b, int32_t rounds,
+                        uint32_t spin_limit, void *stream);
 
 #ifdef __cplusplus
 }
