@@ -106,6 +106,37 @@ __device__ __forceinline__ unsigned load_agent(const unsigned *p)
 // its stores -- the write-through, device-coherent ballot store among them -- have been acknowledged.  A release
 // fence of workgroup scope does NOT do this: on this target it waits for LDS and scalar operations only, because
 // the wavefronts of a workgroup share one vector cache.
+//
+// THE GRID BARRIER'S CONTRACT.  Four kinds of words in device memory are written by one workgroup and read by
+// others during a launch; every such access is a relaxed atomic of AGENT scope (it passes the compute unit's
+// vector cache and the XCD's L2 and is served where all XCDs see the same value), and the order between them is
+// made by hand, because HIP's memory model offers no fence of the needed kind that does not also invalidate the
+// XCD's L2 every step:
+//   work_bits   (ballots)   written by: lane 0 of every wavefront that owns elements, right after its update of
+//                           step t (row t % hist).  Read by: every workgroup's pull of step t, after it has seen
+//                           the barrier of step t complete.
+//   res_fired   (lists)     written by: the first 16 threads of a workgroup after the workgroup has met (row t %
+//                           hist, the workgroup's 16 places).  Read by: every workgroup's pull of step t, as above.
+//   arrival counters        written by: thread 0 of a workgroup, one increment per step, on the counter of (step,
+//                           the workgroup's XCD), AFTER every wavefront of the workgroup has executed
+//                           wait_vector_memory() and the workgroup has passed __syncthreads().  Read by: one look
+//                           per workgroup and step (the eight counters of the step added up), repeated within a
+//                           bounded spin.
+//   abort word              written by: any workgroup whose spin ran out.  Read by: every workgroup inside its spin
+//                           and at the start of a launch.  Sticky: only the host clears it.
+// The one ordering that makes the barrier a barrier: a workgroup's ballot and list stores of step t are
+// ACKNOWLEDGED (wait_vector_memory in every wavefront that stored, then the workgroup barrier) before its arrival
+// for step t is sent.  A reader that has counted all arrivals of step t therefore loads ballots and lists that
+// are already where agent-scope loads look.  Nothing else is assumed: readers do not rely on the order of two
+// stores of another workgroup, and no acquire fence runs inside the loop (every read of another workgroup's words
+// is an agent-scope load, which is not served from a copy that an earlier read left in the compute unit's cache).
+// If the wait before the arrival were lost (a compiler that moved or dropped the asm, a fence mistaken for it),
+// a reader could see the arrival before a ballot word and miss a spike of that step: the tests that run many
+// workgroups for many steps against a driver without this barrier would differ in single synaptic segments --
+// tests/test_gpu_simulate.py::test_v1_scale_resident_equals_per_step_launches and
+// ::test_lists_of_fired_neurons_equal_the_ballots, tests/test_gpu_random_networks.py::
+// test_many_workgroups_with_volleys_and_delay_offsets, tests/test_gpu_fullsize.py::
+// test_v1_scale_forward_run_against_both_oracles.
 __device__ __forceinline__ void wait_vector_memory()
 {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -1,25 +1,29 @@
 // Batched forward simulation, one launch per step, pull and update fused.
 //
-// A wavefront owns a target neuron at a time and its lanes are the neuron's
-// trials (batch 8, 16, 32 or 64).  For step t it
-//   1. streams the neuron's row of the joint target-major table (recurrent
-//      synapses and input synapses, lane = synapse), keeps the synapses whose
-//      source fired in some trial of the emitting step t-1-delay (a bit map of
-//      the last L-1 steps in LDS), fetches those sources' trial masks from the
-//      joint history and adds the weights into 64-bit fixed-point sums in LDS,
-//      one per (receptor, trial): everything that arrives at the neuron in
-//      step t-1, exact and independent of the order of the additions;
+// A wavefront advances 64 elements at a time: the 64 / batch neurons of a group
+// with all their trials (batch 8, 16, 32 or 64), lane = (neuron of the group,
+// trial).  For step t it
+//   1. streams the rows of the group's neurons in the joint target-major table
+//      (recurrent synapses and input synapses, lane = synapse), keeps the
+//      synapses whose source fired in some trial of the emitting step
+//      t-1-delay (a bit map of the last L-1 steps in LDS), fetches those
+//      sources' trial masks from the joint history and adds the weights into
+//      64-bit fixed-point sums in LDS, one per (receptor, neuron of the group,
+//      trial): everything that arrives at these neurons in step t-1, exact and
+//      independent of the order of the additions;
 //   2. folds the sums into y1 (NEST adds the arrivals of step t-1 at the end of
 //      that step; nothing reads y1 before the update of step t, so adding them
 //      at the top of that update performs the same two rounded operations);
-//   3. advances the neuron's trials through step t (lane = trial; the
-//      propagators are the same in all lanes) and writes its spike bits into
-//      row t of the history, where the launches of steps t+2 .. t+L find them.
+//   3. advances the 64 elements through step t with every lane at work and
+//      256-byte rows of state, and writes their spike bits -- one 64-bit word --
+//      into row t of the history, where the launches of steps t+2 .. t+L find
+//      them.
 // No arrival sum passes through device memory and no launch stands between the
-// pull and the update.  Other workgroups of the same launch turn the input
-// events of step t into bits of the same history row, and deliver the few ids
-// that occur twice within a step (bits hold an id once) as events into the
-// ring, which the update folds along.
+// pull and the update.  A workgroup owns a run of consecutive groups and its
+// wavefronts take them one by one from a counter in LDS; two of them first turn
+// the workgroup's share of the input events of step t into bits of the same
+// history row, and deliver the few ids that occur twice within a step (bits
+// hold an id once) as events into the ring, which the update folds along.
 #include "common.hpp"
 #include "glif3_update.hpp"
 #include "propagate.hpp"
@@ -29,61 +33,203 @@
 namespace bmtk {
 
 constexpr int kFuseBlock = 1024;
-constexpr int kFuseAhead = 3;  // table blocks of 2 KB per wavefront, in flight or at hand (4 and 5: no faster)
 constexpr int kFuseWaves = kFuseBlock / kWave;
-constexpr size_t kFuseLdsMax = 80u * 1024u;  // half a compute unit's LDS: the few workgroups of the other roles fit beside
+#ifndef FUSE_AHEAD
+#define FUSE_AHEAD 3
+#endif
+constexpr int kFuseAhead = FUSE_AHEAD;  // table blocks of 2 KB per wavefront, in flight or at hand (4 and 5: no faster)
+constexpr size_t kFuseLdsMax = 150u * 1024u;  // one workgroup per compute unit
 
 struct FusedLaunch {
     int64_t t;           // step being updated (closing launch: one past the last step)
     int64_t out_row;     // row of spike_bits / save_v / save_flags
     int64_t probe_row;   // row of probe_v, -1: not a sampled step
     int64_t n_in_words;  // 64-bit words of the input part of a history row
-    int n_main, n_inb, n_rep;  // workgroups per role, in this order of block ids
+    int n_main;          // workgroups
     int do_update;       // 0 in the closing launch: pull and fold only
     int fold;            // the arrivals of step t-1 are pulled and folded (every launch but a call's first)
     int use_ring;        // ring slot t-1 may hold arrivals (ids repeated within a step)
+    int in_bits;         // the input events of step t become bits of history row t
+    int repeats;         // the repeated ids of step t-1 are delivered as events
     int H;               // rows of the history
     int n_w32;           // words per row of the activity map
     int shift;           // sources per bit of the activity map: 2^shift
 };
 
-// the spike bits of one neuron's trials: bits [row*kBatch, (row+1)*kBatch) of a history row
-template <int kBatch>
-__device__ __forceinline__ void store_trial_bits(uint64_t *__restrict__ words, int64_t row, unsigned long long m)
-{
-    if (kBatch == 64)
-        words[row] = m;
-    else if (kBatch == 32)
-        reinterpret_cast<uint32_t *>(words)[row] = (uint32_t)m;
-    else if (kBatch == 16)
-        reinterpret_cast<uint16_t *>(words)[row] = (uint16_t)m;
-    else
-        reinterpret_cast<uint8_t *>(words)[row] = (uint8_t)m;
-}
+// One block of the synapse stream a wavefront works through: positions [base, min(base + 256, p1)) of the packed
+// table, all of one row.
+struct FuseBlockDesc {
+    int row;       // -1: past the end (an empty block of no row)
+    int base, p1;
+    bool first;    // first block of the first row of its group: the group's state is asked for
+    bool last;     // last block of its row: the row's synapses are complete after it
+    bool closes;   // ... and the row is the last of its group: the group is closed after it
+};
+
+// The groups a wavefront takes from its workgroup's counter, as a stream of blocks.  The bounds of the row after the
+// current one (which may belong to the next group, taken from the counter a group ahead) are fetched a row ahead.
+// Everything here is the same in all lanes.
+template <int kRows>
+struct GroupCursor {
+    const int32_t *__restrict__ indptr;
+    int *counter;
+    int n, g_end;
+    int grp, row, row_end;  // group and row at hand, one past the group's last row
+    int q, p1;              // what is left of the row
+    int ngrp;               // the group after (>= g_end: none)
+    int nrow, np0, np1;     // the row after (-1: none) and its bounds
+    bool at_start;
+
+    __device__ __forceinline__ int grab()
+    {
+        int g = 0;
+        if (lane_id() == 0) g = atomicAdd(counter, 1);
+        return __builtin_amdgcn_readfirstlane(g);
+    }
+    __device__ __forceinline__ void look_ahead()
+    {
+        nrow = -1;
+        if (row >= 0 && row + 1 < row_end)
+            nrow = row + 1;
+        else if (ngrp < g_end)
+            nrow = ngrp * kRows;
+        if (nrow >= 0) {
+            np0 = indptr[nrow];
+            np1 = indptr[nrow + 1];
+        }
+    }
+    __device__ __forceinline__ void start(const int32_t *ip, int n_rows, int groups_end, int *ctr)
+    {
+        indptr = ip;
+        counter = ctr;
+        n = n_rows;
+        g_end = groups_end;
+        grp = grab();
+        ngrp = grab();
+        row = -1;
+        row_end = q = p1 = np0 = np1 = 0;
+        at_start = true;
+        if (grp < g_end) {
+            row = grp * kRows;
+            row_end = min(n, row + kRows);
+            q = indptr[row];
+            p1 = indptr[row + 1];
+        }
+        look_ahead();
+    }
+    __device__ __forceinline__ FuseBlockDesc next()
+    {
+        if (row < 0) return FuseBlockDesc{-1, 0, 0, false, false, false};
+        FuseBlockDesc b{row, q, p1, at_start, false, false};
+        at_start = false;
+        q += kPullChunks * kWave;
+        if (q >= p1) {
+            b.last = true;
+            b.closes = row + 1 == row_end;
+            const bool new_group = b.closes;
+            row = nrow;
+            q = np0;
+            p1 = np1;
+            if (new_group) {
+                at_start = true;
+                grp = ngrp;
+                row_end = min(n, (grp + 1) * kRows);
+                if (row >= 0) ngrp = grab();
+            }
+            look_ahead();
+        }
+        return b;
+    }
+};
 
 template <int kBatch>
 __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s, FusedLaunch q)
 {
     extern __shared__ unsigned long long fuse_lds[];  // accumulators, stages, then the activity map [L-1][n_w32]
-    static_assert(kBatch == 8 || kBatch == 16 || kBatch == 32 || kBatch == 64, "lane = trial, whole bytes of spike bits");
+    __shared__ int next_group;
+    static_assert(kBatch == 8 || kBatch == 16 || kBatch == 32 || kBatch == 64, "whole neurons per wavefront");
+    constexpr int kRows = kWave / kBatch;  // neurons of a group
     const int bid = (int)blockIdx.x;
-    const int64_t n = s.n_neurons, ne = n * kBatch;
+    const int n = (int)s.n_neurons;
+    const int64_t ne = (int64_t)n * kBatch;
     const int L = s.ring_slots, H = q.H;
     const unsigned lane = (unsigned)lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     uint64_t *__restrict__ hist_t = s.work_bits + (q.t % H) * s.fuse_hist_stride;  // the row this launch writes
     uint32_t *__restrict__ any_t = s.fuse_any + (q.t % H) * q.n_w32;
+    unsigned long long *acc = fuse_lds + wave * (GLIF3_NREC * kWave);  // [receptor][neuron of the group, trial]
+    uint2 *stage = reinterpret_cast<uint2 *>(fuse_lds + kFuseWaves * GLIF3_NREC * kWave) + wave * kWave;
+    uint32_t *any_l = reinterpret_cast<uint32_t *>(fuse_lds + kFuseWaves * (GLIF3_NREC + 1) * kWave);
+    // ring map: bit i of row (u % L) = some ring cell of neuron i in slot u % L holds an arrival (set where repeated
+    // ids are delivered, cleared by the neuron's owner when it takes the cells along); behind the H rows of the
+    // activity map
+    const int ring_map_words = (n + 31) >> 5;
+    uint32_t *__restrict__ ring_map = s.fuse_any + (int64_t)H * q.n_w32;
+    uint32_t *__restrict__ ring_map_prev = ring_map + (int64_t)((q.t + L - 1) % L) * ring_map_words;
 
-    if (bid >= q.n_main + q.n_inb) {
+    // the workgroup's run of groups, and the counter its wavefronts take them from
+    const int n_groups = (n + kRows - 1) / kRows;
+    const int per_wg = (n_groups + q.n_main - 1) / q.n_main;
+    const int g_first = bid * per_wg, g_end = min(n_groups, g_first + per_wg);
+    if (threadIdx.x == 0) next_group = g_first;
+    // the activity row of the step after this one starts empty (no launch reads it before it is written)
+    {
+        uint32_t *__restrict__ next = s.fuse_any + ((q.t + 1) % H) * q.n_w32;
+        for (int i = bid * kFuseBlock + (int)threadIdx.x; i < q.n_w32; i += q.n_main * kFuseBlock) next[i] = 0u;
+    }
+    if (q.fold) {
+        // the activity maps of the steps t-2 .. t-L (delays 1 .. L-1), one after the other
+        for (int dd = 0; dd < L - 1; ++dd) {
+            const int64_t u = q.t - 2 - dd;
+            const uint32_t *__restrict__ src = s.fuse_any + (((u % H) + H) % H) * q.n_w32;
+            for (int i = threadIdx.x; i < q.n_w32; i += kFuseBlock) any_l[dd * q.n_w32 + i] = src[i];
+        }
+    }
+    __syncthreads();
+
+    if (wave == kFuseWaves - 1 && q.in_bits) {
+        // ---- the workgroup's share of the input events of step t as bits of history row t: a lane per 64-bit
+        //      word; the events of a step are ascending, so a word's events are one run of the list, found by
+        //      bisection.  (Read from the launch of step t+2 on.)  The wavefront then takes groups like the others,
+        //      which have taken a few more meanwhile. ----
+        const int64_t k0 = s.in_ptr[q.t], k1 = s.in_ptr[q.t + 1];
+        const int64_t in_word0 = s.fuse_in_base * kBatch / 64;
+        for (int64_t w = (int64_t)bid * kWave + lane; w < q.n_in_words; w += (int64_t)q.n_main * kWave) {
+            const int64_t lo = w * 64;
+            int64_t a = k0, b = k1;
+            while (a < b) {
+                const int64_t mid = (a + b) >> 1;
+                if ((int64_t)s.in_events[mid] < lo)
+                    a = mid + 1;
+                else
+                    b = mid;
+            }
+            unsigned long long bits = 0ull;
+            for (; a < k1; ++a) {
+                const int64_t ev = s.in_events[a];
+                if (ev >= lo + 64) break;
+                bits |= 1ull << (ev - lo);
+            }
+            hist_t[in_word0 + w] = bits;
+            if (bits != 0ull) {
+                const unsigned long long field = kBatch == 64 ? ~0ull : ((1ull << kBatch) - 1ull);
+#pragma unroll
+                for (int f = 0; f < kRows; ++f) {
+                    if ((bits >> (f * (kBatch & 63))) & field) {
+                        const unsigned g = (unsigned)(s.fuse_in_base + w * kRows + f) >> q.shift;
+                        atomicOr(any_t + (g >> 5), 1u << (g & 31u));
+                    }
+                }
+            }
+        }
+    }
+    if (wave == kFuseWaves - 2 && q.repeats) {
         // ---- ids that occur more than once among the input events of step t-1: the occurrences after the first,
         //      as events into the ring (slots t .. t+L-2; this launch folds and clears slot t-1) ----
         const int slot0 = (int)((q.t - 1) % L);
         const int64_t k0 = s.in_repeat_ptr[q.t - 1], k1 = s.in_repeat_ptr[q.t];
-        const int n_waves = q.n_rep * kFuseWaves;
-        const int wave = (bid - q.n_main - q.n_inb) * kFuseWaves + threadIdx.x / kWave;
-        const int ring_map_words = (int)((n + 31) >> 5);
-        uint32_t *__restrict__ ring_map = s.fuse_any + (int64_t)H * q.n_w32;
         const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(s.inp_packed);
-        for (int64_t k = k0 + wave; k < k1; k += n_waves) {
+        for (int64_t k = k0 + bid; k < k1; k += q.n_main) {
             const int e = s.in_repeat_events[k];
             const int j = (int)((uint32_t)e / (uint32_t)kBatch), b = e - j * kBatch;
             const int p1 = s.inp_indptr[j + 1];
@@ -97,73 +243,19 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
                 atomicOr(ring_map + (int64_t)slot * ring_map_words + (i >> 5), 1u << (i & 31));
             }
         }
-        return;
     }
 
-    if (bid >= q.n_main) {
-        // ---- the input events of step t as bits of history row t: one thread per 64-bit word; the events of a
-        //      step are ascending, so a word's events are one run of the list, found by bisection ----
-        const int64_t w = (int64_t)(bid - q.n_main) * kFuseBlock + threadIdx.x;
-        if (w >= q.n_in_words) return;
-        const int64_t k0 = s.in_ptr[q.t], k1 = s.in_ptr[q.t + 1];
-        const int64_t lo = w * 64;
-        int64_t a = k0, b = k1;
-        while (a < b) {
-            const int64_t mid = (a + b) >> 1;
-            if ((int64_t)s.in_events[mid] < lo)
-                a = mid + 1;
-            else
-                b = mid;
-        }
-        unsigned long long bits = 0ull;
-        for (; a < k1; ++a) {
-            const int64_t ev = s.in_events[a];
-            if (ev >= lo + 64) break;
-            bits |= 1ull << (ev - lo);
-        }
-        const int64_t in_word0 = s.fuse_in_base * kBatch / 64;
-        hist_t[in_word0 + w] = bits;
-        if (bits != 0ull) {
-            constexpr int kPerWord = 64 / kBatch;  // sources per word
-            const unsigned long long field = kBatch == 64 ? ~0ull : ((1ull << kBatch) - 1ull);
-#pragma unroll
-            for (int f = 0; f < kPerWord; ++f) {
-                if ((bits >> (f * (kBatch & 63))) & field) {
-                    const unsigned g = (unsigned)(s.fuse_in_base + w * kPerWord + f) >> q.shift;
-                    atomicOr(any_t + (g >> 5), 1u << (g & 31u));
-                }
-            }
-        }
-        return;
-    }
-
-    // ---- a neuron at a time: pull, fold, update ----
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
-    constexpr int kAccWords = GLIF3_NREC * kBatch;  // per wavefront
-    unsigned long long *acc = fuse_lds + wave * kAccWords;  // [receptor][trial]
-    uint2 *stage = reinterpret_cast<uint2 *>(fuse_lds + kFuseWaves * kAccWords) + wave * kWave;
-    uint32_t *any_l = reinterpret_cast<uint32_t *>(fuse_lds + kFuseWaves * (kAccWords + kWave));
-    // the activity row of the step after this one starts empty (no launch reads it before it is written)
-    {
-        uint32_t *__restrict__ next = s.fuse_any + ((q.t + 1) % H) * q.n_w32;
-        for (int i = bid * kFuseBlock + (int)threadIdx.x; i < q.n_w32; i += q.n_main * kFuseBlock) next[i] = 0u;
-    }
-    const bool on = kBatch == 64 || lane < (unsigned)kBatch;  // this lane holds a trial
+    // ---- a group at a time: pull, fold, update ----
     const unsigned uw32 = (unsigned)q.n_w32, ushift = (unsigned)q.shift, umax_dd = (unsigned)(L - 2);
-    Glif3Elem st;  // the state of the row at hand, asked for when its first block turns up
-    float prop_col = 0.0f;  // ... and its propagators: lane k holds row k of the neuron's column
-    unsigned ring_word = 0u;  // ... and the word of the ring map that holds the row's bit
-    const unsigned prop_row_bytes = (unsigned)(s.prop_stride * sizeof(float));
-    // ring map: bit i of row (u % L) = some ring cell of neuron i in slot u % L holds an arrival (set by the
-    // workgroups that deliver repeated ids, cleared by the neuron's owner when it takes the cells along); it lies
-    // behind the H rows of the activity map
-    const int ring_map_words = (int)((n + 31) >> 5);
-    uint32_t *__restrict__ ring_map = s.fuse_any + (int64_t)H * q.n_w32;
-    uint32_t *__restrict__ ring_map_prev = ring_map + (int64_t)((q.t + L - 1) % L) * ring_map_words;
-    static_assert(GLIF3_NPROP <= kWave, "a column of the propagator table in one wavefront register");
+    const unsigned sub_lane = lane / (unsigned)kBatch;  // this lane's neuron within a group
+    // Asked for when a group's first block turns up, used when the group is closed: the state of its 64 elements,
+    // their propagators (every lane its neuron's column) and the word of the ring map that holds the group's bits.
+    Glif3Elem st;
+    Glif3Prop pr;
+    unsigned ring_word = 0u;
 
     // Element accesses: a scalar base (array + plane k of ne elements) and this lane's 32-bit byte offset
-    // (n_neurons * batch < 2^30, checked by the caller), which is the address form that needs no 64-bit lane arithmetic.
+    // (n_neurons * batch < 2^30, checked by the caller), the address form that needs no 64-bit lane arithmetic.
     const size_t plane = (size_t)ne * sizeof(float);
     auto ldf = [&](const float *base, int k, unsigned boff) {
         return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) + k * plane + boff);
@@ -171,30 +263,50 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
     auto stf = [&](float *base, int k, unsigned boff, float v) {
         *reinterpret_cast<float *>(reinterpret_cast<char *>(base) + k * plane + boff) = v;
     };
-    // what is left to do for a neuron once its arrival sums are known
-    auto finish_row = [&](int64_t row, float (&a)[GLIF3_NREC]) {
-        const unsigned e = (unsigned)(row * kBatch) + lane, boff = e * 4u;
-        if (q.use_ring && q.fold && ((ring_word >> ((unsigned)row & 31u)) & 1u)) {
-            // an id repeated within a step reached this neuron's ring cells of step t-1 (rare): take them along
-            if (on) {
-                float *prev = s.ring + (int64_t)((q.t + L - 1) % L) * GLIF3_NREC * ne;
-                float v[GLIF3_NREC];
+    // All lanes load, whatever they hold (the lanes past the last neuron of the network load the last neuron's
+    // values and keep them to themselves): a load under a condition would have to be waited for at once, where the
+    // two ways meet again.
+    auto load_group = [&](int grp) {
+        const int row = min(grp * kRows + (int)sub_lane, n - 1);
+        const unsigned e = (unsigned)row * (unsigned)kBatch + (lane & (unsigned)(kBatch - 1));
+        const unsigned boff = e * 4u;
+        const int64_t col = s.class_id ? (int64_t)s.class_id[row] : (int64_t)row;
+        pr.load(s.prop, s.prop_stride, col);
+        if (q.use_ring) ring_word = ring_map_prev[(grp * kRows) >> 5];
+        if (q.do_update) {
+            st.V = ldf(s.V, 0, boff);
+            st.ref = *reinterpret_cast<const int32_t *>(reinterpret_cast<const char *>(s.ref) + boff);
 #pragma unroll
-                for (int k = 0; k < GLIF3_NREC; ++k) v[k] = ldf(prev, k, boff);
+            for (int k = 0; k < GLIF3_NASC; ++k) st.asc[k] = ldf(s.asc, k, boff);
 #pragma unroll
-                for (int k = 0; k < GLIF3_NREC; ++k) {
-                    stf(prev, k, boff, 0.0f);
-                    a[k] = v[k] + a[k];
-                }
+            for (int k = 0; k < GLIF3_NREC; ++k) {
+                st.y1[k] = ldf(s.y1, k, boff);
+                st.y2[k] = ldf(s.y2, k, boff);
             }
-            if (lane == 0) atomicAnd(ring_map_prev + (row >> 5), ~(1u << ((unsigned)row & 31u)));
         }
-        Glif3Prop p;  // the same in all lanes
-        p.load_from_lanes(prop_col);
+    };
+    // what is left to do for a group once its arrival sums are known
+    auto finish_group = [&](int grp, float (&a)[GLIF3_NREC]) {
+        const int row = grp * kRows + (int)sub_lane;
+        const bool on = row < n;  // this lane holds an element
+        const unsigned e = (unsigned)(grp * kRows) * (unsigned)kBatch + lane, boff = e * 4u;
+        if (q.use_ring && q.fold && on && ((ring_word >> ((unsigned)row & 31u)) & 1u)) {
+            // an id repeated within a step reached this neuron's ring cells of step t-1 (rare): take them along
+            float *prev = s.ring + (int64_t)((q.t + L - 1) % L) * GLIF3_NREC * ne;
+            float v[GLIF3_NREC];
+#pragma unroll
+            for (int k = 0; k < GLIF3_NREC; ++k) v[k] = ldf(prev, k, boff);
+#pragma unroll
+            for (int k = 0; k < GLIF3_NREC; ++k) {
+                stf(prev, k, boff, 0.0f);
+                a[k] = v[k] + a[k];
+            }
+            if ((lane & (unsigned)(kBatch - 1)) == 0u) atomicAnd(ring_map_prev + (row >> 5), ~(1u << ((unsigned)row & 31u)));
+        }
         if (!q.do_update) {
             if (on && q.fold) {
 #pragma unroll
-                for (int k = 0; k < GLIF3_NREC; ++k) stf(s.y1, k, boff, ldf(s.y1, k, boff) + a[k] * p.psc0[k]);
+                for (int k = 0; k < GLIF3_NREC; ++k) stf(s.y1, k, boff, ldf(s.y1, k, boff) + a[k] * pr.psc0[k]);
             }
             return;
         }
@@ -203,12 +315,12 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
         if (on) {
             if (q.fold) {
 #pragma unroll
-                for (int k = 0; k < GLIF3_NREC; ++k) st.y1[k] = st.y1[k] + a[k] * p.psc0[k];
+                for (int k = 0; k < GLIF3_NREC; ++k) st.y1[k] = st.y1[k] + a[k] * pr.psc0[k];
             }
             const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
             const float I = s.i_ext ? ldf(s.i_ext, 0, boff) : 0.0f;
             const int ref_before = st.ref;
-            spike = glif3_update(st, p, s.h, zero, I, &frac);
+            spike = glif3_update(st, pr, s.h, zero, I, &frac);
             stf(s.V, 0, boff, st.V);
             *reinterpret_cast<int32_t *>(reinterpret_cast<char *>(s.ref) + boff) = st.ref;
 #pragma unroll
@@ -229,11 +341,15 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
                                                               (ref_before > 0 && st.ref == 0 ? BMTK_F_RESET : 0));
             }
         }
+        // the group's 64 elements are one word of spike bits
         const unsigned long long m = __ballot(spike);
         if (lane == 0) {
-            store_trial_bits<kBatch>(hist_t, row, m);
-            if (s.spike_bits) store_trial_bits<kBatch>(s.spike_bits + q.out_row * s.spike_bits_stride, row, m);
-            if (m != 0ull) {
+            hist_t[grp] = m;
+            if (s.spike_bits) s.spike_bits[q.out_row * s.spike_bits_stride + grp] = m;
+        }
+        if (m != 0ull && on && (lane & (unsigned)(kBatch - 1)) == 0u) {
+            const unsigned long long field = kBatch == 64 ? ~0ull : ((1ull << kBatch) - 1ull);
+            if ((m >> (sub_lane * (unsigned)(kBatch & 63))) & field) {
                 const unsigned g = (unsigned)row >> ushift;
                 atomicOr(any_t + (g >> 5), 1u << (g & 31u));
             }
@@ -256,45 +372,19 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
             }
         }
     };
-    // Asked for when a row's first block turns up, used when the row is closed: its propagator column (lane k
-    // fetches row k; the lanes beyond the table fetch the last row again), the state of its trials, and the word
-    // of the map of ring cells that hold something.  All lanes load, whatever they hold: see flush_issue.
-    auto load_row = [&](int64_t row, int64_t col) {
-        prop_col = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(s.prop + col) +
-                                                    min(lane, (unsigned)(GLIF3_NPROP - 1)) * prop_row_bytes);
-        if (q.use_ring) ring_word = ring_map_prev[row >> 5];
-        if (q.do_update) {
-            const unsigned boff = ((unsigned)(row * kBatch) + (on ? lane : 0u)) * 4u;
-            st.V = ldf(s.V, 0, boff);
-            st.ref = *reinterpret_cast<const int32_t *>(reinterpret_cast<const char *>(s.ref) + boff);
-#pragma unroll
-            for (int k = 0; k < GLIF3_NASC; ++k) st.asc[k] = ldf(s.asc, k, boff);
-#pragma unroll
-            for (int k = 0; k < GLIF3_NREC; ++k) {
-                st.y1[k] = ldf(s.y1, k, boff);
-                st.y2[k] = ldf(s.y2, k, boff);
-            }
-        }
-    };
 
-    const int64_t first_row = (int64_t)bid * kFuseWaves + wave, row_stride = (int64_t)q.n_main * kFuseWaves;
     if (!q.fold) {
         // a call's first launch: the closing launch of the call before it has folded everything that arrived
-        for (int64_t row = first_row; row < n; row += row_stride) {
+        for (int grp = 0;;) {
+            if (lane == 0) grp = atomicAdd(&next_group, 1);
+            grp = __builtin_amdgcn_readfirstlane(grp);
+            if (grp >= g_end) break;
             float a[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
-            load_row(row, s.class_id ? (int64_t)s.class_id[row] : row);
-            finish_row(row, a);
+            load_group(grp);
+            finish_group(grp, a);
         }
         return;
     }
-
-    // the activity maps of the steps t-2 .. t-L (delays 1 .. L-1), one after the other
-    for (int dd = 0; dd < L - 1; ++dd) {
-        const int64_t u = q.t - 2 - dd;
-        const uint32_t *__restrict__ src = s.fuse_any + (((u % H) + H) % H) * q.n_w32;
-        for (int i = threadIdx.x; i < q.n_w32; i += kFuseBlock) any_l[dd * q.n_w32 + i] = src[i];
-    }
-    __syncthreads();
 
     const unsigned hrow_bytes = (unsigned)s.fuse_hist_stride * 8u;  // H * stride * 8 < 2^32 (checked by the caller)
     const unsigned uH = (unsigned)H, uprev = (unsigned)((q.t - 1) % H);
@@ -305,8 +395,8 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
     // A block past the end or an empty one reads the table's first record the same way: every call issues exactly
     // four loads, which is what lets a turn wait for ITS block only and leave the younger ones in flight (the wait
     // is a count of loads still out, fixed at compile time).
-    auto fetch = [&](unsigned long long *dst, const PullBlock &blk) {
-        const bool some = blk.row < n && blk.base < blk.p1;
+    auto fetch = [&](unsigned long long *dst, const FuseBlockDesc &blk) {
+        const bool some = blk.row >= 0 && blk.base < blk.p1;
         const char *__restrict__ src = reinterpret_cast<const char *>(packed) + (some ? (size_t)blk.base * 8u : (size_t)0);
         const unsigned last = some ? (unsigned)(blk.p1 - blk.base) - 1u : 0u;
 #pragma unroll
@@ -319,9 +409,9 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
     // over).  The buffers take turns in place -- a register copy of a block still on its way would wait for it --
     // (and a buffer chosen at run time would leave the compiler no way to tell which loads a turn may leave in
     // flight: it then waits for all of them), so the loop body holds one turn per buffer.
-    PullCursor cursor;
-    cursor.start(s.fuse_indptr, n, first_row, row_stride, s.class_id);
-    PullBlock dq[kFuseAhead];
+    GroupCursor<kRows> cursor;
+    cursor.start(s.fuse_indptr, n, g_end, &next_group);
+    FuseBlockDesc dq[kFuseAhead];
     unsigned long long d[kFuseAhead][kPullChunks];
 #pragma unroll
     for (int k = 0; k < kFuseAhead; ++k) {
@@ -330,23 +420,21 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
         dq[k] = cursor.next();
         fetch(d[k], dq[k]);
     }
-    if (dq[0].row >= n) return;
-    if (on) {
+    if (dq[0].row < 0) return;
 #pragma unroll
-        for (int r = 0; r < GLIF3_NREC; ++r) acc[r * kBatch + lane] = 0ull;
-    }
+    for (int r = 0; r < GLIF3_NREC; ++r) acc[r * kWave + lane] = 0ull;
     int staged = 0;  // entries in the stage (same in all lanes)
     // A flush of the stage has two halves a turn apart, so that the masks travel while the wavefront works on the
     // next block: the first takes the staged synapses into registers and asks for their sources' trial masks, the
-    // second converts the weights and adds.  A row's closing work (sums, fold, update) waits for its last flush
-    // the same way and is done in the turn after the row's last block.
+    // second converts the weights and adds.  A group's closing work (sums, fold, update) waits for its last flush
+    // the same way and is done in the turn after the group's last block.  A flush holds synapses of one row.
     int pend_n = 0;           // synapses of the flush under way (same in all lanes)
+    unsigned pend_col = 0u;   // ... and the first column of their neuron in the accumulators
     uint2 pend_e = make_uint2(0u, 0u);
     unsigned long long pend_m = 0ull;
-    int64_t fin_row = -1;     // the row whose closing work is due
-    auto flush_issue = [&]() {
-        // every lane loads (the lanes without a synapse the mask of source 0 in the row of step t-1, and ignore it):
-        // a load under a condition would have to be waited for at once, where the two ways meet again
+    int fin_grp = -1;         // the group whose closing work is due
+    auto flush_issue = [&](int row) {
+        // every lane loads (the lanes without a synapse the mask of source 0 in the row of step t-1, and ignore it)
         const uint2 e = stage[lane];  // {source | receptor << 24 | delay << 26, weight}
         pend_e = (int)lane < staged ? e : make_uint2(0u, 0u);
         const unsigned src = pend_e.x & 0xFFFFFFu;
@@ -362,11 +450,12 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
         else
             pend_m = *reinterpret_cast<const uint8_t *>(cell);
         pend_n = staged;
+        pend_col = (unsigned)(row % kRows) * (unsigned)kBatch;
         staged = 0;
     };
     auto flush_complete = [&]() {
         if ((int)lane < pend_n) {
-            unsigned long long *a = acc + ((pend_e.x >> 24) & 3u) * kBatch;
+            unsigned long long *a = acc + ((pend_e.x >> 24) & 3u) * kWave + pend_col;
             const unsigned long long w = to_fixed(__uint_as_float(pend_e.y));
             unsigned long long mm = pend_m;
             while (mm) {
@@ -377,23 +466,21 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
         }
         pend_n = 0;
     };
-    // the flush under way, then the closing work of the row it belonged to
+    // the flush under way, then the closing work of the group it belonged to
     auto resolve = [&]() {
         flush_complete();
-        float a[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (on) {
+        float a[GLIF3_NREC];
 #pragma unroll
-            for (int r = 0; r < GLIF3_NREC; ++r) {
-                a[r] = from_fixed(acc[r * kBatch + lane]);
-                acc[r * kBatch + lane] = 0ull;
-            }
+        for (int r = 0; r < GLIF3_NREC; ++r) {
+            a[r] = from_fixed(acc[r * kWave + lane]);
+            acc[r * kWave + lane] = 0ull;
         }
-        finish_row(fin_row, a);
-        fin_row = -1;
+        finish_group(fin_grp, a);
+        fin_grp = -1;
     };
     // one turn: the block `cb` with its table words `cd`; afterwards the buffer takes the block kFuseAhead ahead
-    auto turn = [&](PullBlock &cb, unsigned long long *cd) {
-        const unsigned left = cb.base < cb.p1 ? (unsigned)(cb.p1 - cb.base) : 0u;
+    auto turn = [&](FuseBlockDesc &cb, unsigned long long *cd) {
+        const unsigned left = (cb.row >= 0 && cb.base < cb.p1) ? (unsigned)(cb.p1 - cb.base) : 0u;
         // activity bits of the four chunks (LDS reads, no branch between them)
         unsigned word[kPullChunks], bit[kPullChunks];
 #pragma unroll
@@ -411,25 +498,25 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
             hit[u] = lane + u * kWave < left && ((word[u] >> bit[u]) & 1u);
             who[u] = __ballot(hit[u]);
         }
-        // the row before: its last masks were asked for a turn ago, its closing work comes before any synapse of
-        // this row is added (the one place of a turn where a row is closed)
-        if (fin_row >= 0) resolve();
-        if (cb.first) load_row(cb.row, cb.col);  // (after that row's closing work, which used the same registers)
+        // the group before: its last masks were asked for a turn ago, its closing work comes before any synapse of
+        // this group is added (the one place of a turn where a group is closed)
+        if (fin_grp >= 0) resolve();
+        if (cb.first) load_group(cb.row / kRows);  // (after that group's closing work, which used the same registers)
 #pragma unroll
         for (int u = 0; u < kPullChunks; ++u) {
             const int cnt = __popcll(who[u]);
             if (cnt == 0) continue;
             if (staged + cnt > kWave) {
                 flush_complete();
-                flush_issue();
+                flush_issue(cb.row);
             }
             if (hit[u]) stage[staged + lane_prefix(who[u])] = make_uint2((unsigned)cd[u], (unsigned)(cd[u] >> 32));
             staged += cnt;
         }
         if (cb.last) {
-            flush_complete();  // a flush of this row still under way
-            flush_issue();
-            fin_row = cb.row;
+            flush_complete();  // a flush of this row (or the row before, of the same group) still under way
+            flush_issue(cb.row);
+            if (cb.closes) fin_grp = cb.row / kRows;
         }
         cb = cursor.next();
         fetch(cd, cb);
@@ -441,13 +528,13 @@ __global__ __launch_bounds__(kFuseBlock) void sim_fused_kernel(bmtk_glif3_sim s,
     do {
 #pragma unroll
         for (int k = 0; k < kFuseAhead; ++k) turn(dq[k], d[k]);
-    } while (dq[0].row < n);
-    if (fin_row >= 0) resolve();
+    } while (dq[0].row >= 0);
+    if (fin_grp >= 0) resolve();
 }
 
-size_t fused_lds_bytes(int batch, int L, int n_w32)
+size_t fused_lds_bytes(int L, int n_w32)
 {
-    return (size_t)kFuseWaves * (GLIF3_NREC * batch + kWave) * sizeof(unsigned long long) + (size_t)(L - 1) * n_w32 * 4u;
+    return (size_t)kFuseWaves * (GLIF3_NREC + 1) * kWave * sizeof(unsigned long long) + (size_t)(L - 1) * n_w32 * 4u;
 }
 
 const void *fused_variant(int batch)
@@ -466,8 +553,8 @@ int simulate_fused(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipS
     BMTK_REQUIRE(batch == 8 || batch == 16 || batch == 32 || batch == 64,
                  "glif3_simulate_fwd: the fused form runs batches of 8, 16, 32 or 64");
     BMTK_REQUIRE(s.fuse_indptr && s.fuse_any, "glif3_simulate_fwd: the fused form needs fuse_indptr and fuse_any");
-    BMTK_REQUIRE(s.n_neurons * (int64_t)batch < (1ll << 30) && GLIF3_NPROP * s.prop_stride < (1ll << 30),
-                 "glif3_simulate_fwd: the fused form addresses fewer than 2^30 elements and propagator entries");
+    BMTK_REQUIRE(s.n_neurons * (int64_t)batch < (1ll << 30),
+                 "glif3_simulate_fwd: the fused form addresses fewer than 2^30 elements");
     BMTK_REQUIRE(s.delay_offset == 0 && (s.delay_bits == 0 || s.delay_bits == 6) && s.hist_slots == L + 2,
                  "glif3_simulate_fwd: the fused form needs delay_offset 0, the standard packing and hist_slots == ring_slots + 2");
     BMTK_REQUIRE(s.fuse_shift >= 0 && s.fuse_shift <= 16, "glif3_simulate_fwd: fuse_shift must lie in 0..16");
@@ -484,7 +571,7 @@ int simulate_fused(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipS
     BMTK_REQUIRE((int64_t)(L + 2) * s.fuse_hist_stride < (1ll << 29), "glif3_simulate_fwd: joint history beyond 4 GiB");
     const int64_t groups = (in_base + n_in + (1ll << s.fuse_shift) - 1) >> s.fuse_shift;
     const int n_w32 = (int)((groups + 31) / 32);
-    const size_t lds = fused_lds_bytes(batch, L, n_w32);
+    const size_t lds = fused_lds_bytes(L, n_w32);
     BMTK_REQUIRE(lds <= kFuseLdsMax, "glif3_simulate_fwd: the activity map does not fit in LDS; use a larger fuse_shift");
     BMTK_REQUIRE(!s.in_repeat_ptr || (s.in_repeat_events && s.inp_indptr && s.inp_packed),
                  "glif3_simulate_fwd: repeat lists need in_repeat_events and the source-major input table");
@@ -512,7 +599,8 @@ int simulate_fused(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipS
     }
     FusedLaunch q{};
     const int per_cu = s.fuse_wg_per_cu > 0 ? s.fuse_wg_per_cu : 1;
-    const int64_t want = (s.n_neurons + kFuseWaves - 1) / kFuseWaves;
+    const int64_t n_groups = (s.n_neurons * batch + kWave - 1) / kWave;
+    const int64_t want = (n_groups + kFuseWaves - 1) / kFuseWaves;
     const int64_t cap = (int64_t)n_cu * per_cu;
     q.n_main = (int)(want < cap ? want : cap);
     q.H = L + 2;
@@ -529,12 +617,12 @@ int simulate_fused(const bmtk_glif3_sim &s, int64_t step0, int64_t n_steps, hipS
             q.probe_row = (q.t + 1) / s.probe_every - step0 / s.probe_every - 1;
         q.do_update = closing ? 0 : 1;
         q.fold = k > 0 ? 1 : 0;
-        q.n_inb = (has_inp && !closing && n_in_words > 0) ? (int)((n_in_words + kFuseBlock - 1) / kFuseBlock) : 0;
-        q.n_rep = (s.in_repeat_ptr && k > 0 && q.t >= 1) ? 4 : 0;
+        q.in_bits = (has_inp && !closing && n_in_words > 0) ? 1 : 0;
+        q.repeats = (s.in_repeat_ptr && k > 0 && q.t >= 1) ? 1 : 0;
         bmtk_glif3_sim args = s;
         FusedLaunch launch = q;
         void *params[] = {&args, &launch};
-        const hipError_t err = hipLaunchKernel(kernel, dim3((unsigned)(q.n_main + q.n_inb + q.n_rep)), dim3(kFuseBlock),
+        const hipError_t err = hipLaunchKernel(kernel, dim3((unsigned)q.n_main), dim3(kFuseBlock),
                                                params, lds, stream);
         if (err != hipSuccess) {
             set_error("glif3_simulate_fwd: launch failed: %s", hipGetErrorString(err));

@@ -17,7 +17,7 @@ from .ops import Glif3State, SpikeCompactor, SynapseTable, _dev, _p, _stream, gl
 
 PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what is left of 80 KB beside its accumulators
 PULL_MIN_DENSITY = 0.06         # synaptic events per synapse and step from which "auto" pulls instead of pushing
-FUSE_LDS_BYTES = 80 * 1024      # LDS of one workgroup of the fused batched driver (kFuseLdsMax of csrc/simulate_fused.hip)
+FUSE_LDS_BYTES = 150 * 1024     # LDS of one workgroup of the fused batched driver (kFuseLdsMax of csrc/simulate_fused.hip)
 FUSE_WAVES = 16                 # wavefronts of one of its workgroups (kFuseWaves)
 FUSE_BATCHES = (8, 16, 32, 64)  # lane = trial, whole bytes of spike bits per neuron
 RES_LDS_BYTES = 160 * 1024      # LDS of one gfx950 compute unit
@@ -275,8 +275,8 @@ class Glif3Simulator:
         self.hist_slots = self.L + 2
         self.work_bits = torch.zeros(self.hist_slots * self.fuse_hist_stride, dtype=torch.int64, device=self.dev)
         # one bit of the activity map per 2^shift sources: the smallest shift whose map fits the LDS beside the
-        # accumulators (16 wavefronts x (4 x batch sums + a stage of 64 synapses) x 8 bytes)
-        fixed = FUSE_WAVES * (NREC * batch + 64) * 8
+        # accumulators (16 wavefronts x (4 x 64 sums + a stage of 64 synapses) x 8 bytes)
+        fixed = FUSE_WAVES * (NREC * 64 + 64) * 8
         self.fuse_shift = 0
         while fixed + (self.L - 1) * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
             self.fuse_shift += 1
@@ -287,7 +287,7 @@ class Glif3Simulator:
         whose map fits the LDS).  Before the first run only."""
         if self.fuse_table is None or self.step:
             raise ValueError("set_fuse_shift applies to the fused form before its first run")
-        fixed = FUSE_WAVES * (NREC * self.batch + 64) * 8
+        fixed = FUSE_WAVES * (NREC * 64 + 64) * 8
         old, self.fuse_shift = self.fuse_shift, int(shift)
         if not 0 <= self.fuse_shift <= 16 or fixed + (self.L - 1) * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
             self.fuse_shift = old

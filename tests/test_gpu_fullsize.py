@@ -314,11 +314,11 @@ def test_training_size_forward_run_is_bit_identical_to_the_oracle(fused):
 
 
 def test_fused_batched_driver_at_120k_neurons_batch_16():
-    """120,000 neurons x batch 16 with 3,000 Poisson inputs: more sources than the activity map of the fused batched
-    driver holds at one source per bit (the simulator then lets a bit stand for two sources, which costs mask
-    fetches for silent sources and nothing else), more neurons than its 256 workgroups take at a time (7,500 rows
-    per workgroup round).  Quarter-pA weights: raster and state equal the fp32 oracle's bit for bit over 60 steps
-    in two calls."""
+    """120,000 neurons x batch 16 with 3,000 Poisson inputs through the fused batched driver: 30,000 groups of four
+    neurons, 117 per workgroup, taken one by one from the workgroup's counter; with the activity map at one source
+    per bit and at two (what a simulator picks by itself once the sources outgrow the LDS: a bit then stands for
+    several sources, which costs mask fetches for silent sources and nothing else).  Quarter-pA weights: raster and
+    state equal the fp32 oracle's bit for bit over 60 steps in two calls."""
     n, n_in, batch, steps = 120000, 3000, 16, 60
     rng = np.random.default_rng(6)
     par = synthetic.random_cells(rng, 40)
@@ -328,21 +328,24 @@ def test_fused_batched_driver_at_120k_neurons_batch_16():
     inp = synthetic.device_input_table(n_in, n, 1_500_000, seed=9, w_scale=25.0)
     inp = (inp[0], inp[1], _quarter(inp[2]), inp[3], inp[4])
     in_ptr, in_ev = ops.poisson_events(n_in, 20.0, 1.0, steps, batch=batch, seed=10)
-    sim = Glif3Simulator(n, par, 1.0, batch=batch, class_id=class_id, rec=by_src, inp=inp, resident=False, fused=True)
-    assert sim.fuse_table is not None and sim.fuse_shift >= 1
-    sim.set_input_events(in_ptr, in_ev)
-    a = sim.run(25)
-    b = sim.run(steps - 25)
-    ras = torch.cat([sim.raster(a["bits"]), sim.raster(b["bits"])]).cpu().numpy()
     prop = orc.precompute(par, 1.0)
     orc.set_threads(orc.max_threads())
     st = orc.new_state(n, batch, np.float32)
-    ring = np.zeros((sim.L, 4, n * batch), np.float32)
+    ring = np.zeros((6, 4, n * batch), np.float32)
     want = orc.simulate(st, prop, 1.0, steps, batch=batch, class_id=class_id, ring=ring,
                         rec=tuple(t.cpu().numpy() for t in by_src), inp=tuple(t.cpu().numpy() for t in inp),
                         in_ptr=in_ptr.cpu().numpy(), in_events=in_ev.cpu().numpy(), raster=True)
     assert want["count"] > 50_000
-    np.testing.assert_array_equal(ras, want["raster"])
-    got = sim.state.to_numpy()
-    for k in ("V", "asc", "y1", "y2", "ref"):
-        np.testing.assert_array_equal(got[k], st[k], err_msg=k)
+    for shift in (0, 1):
+        sim = Glif3Simulator(n, par, 1.0, batch=batch, class_id=class_id, rec=by_src, inp=inp, resident=False, fused=True)
+        assert sim.fuse_table is not None and sim.fuse_shift == 0 and sim.L == 6
+        if shift:
+            sim.set_fuse_shift(shift)
+        sim.set_input_events(in_ptr, in_ev)
+        a = sim.run(25)
+        b = sim.run(steps - 25)
+        ras = torch.cat([sim.raster(a["bits"]), sim.raster(b["bits"])]).cpu().numpy()
+        np.testing.assert_array_equal(ras, want["raster"], err_msg="shift %d" % shift)
+        got = sim.state.to_numpy()
+        for k in ("V", "asc", "y1", "y2", "ref"):
+            np.testing.assert_array_equal(got[k], st[k], err_msg="%s shift %d" % (k, shift))
