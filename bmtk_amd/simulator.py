@@ -272,13 +272,14 @@ class Glif3Simulator:
             return
         self.fuse_table = SynapseTable.joined_by_target(self.rec, self.inp, n, self.fuse_in_base)
         self.fuse_hist_stride = self.fuse_in_base * batch // 64 + n_words(n_in * batch) + 1
-        self.hist_slots = self.L + 2
+        self.hist_slots = self.L + 4         # two steps per launch: rows read, written and cleared ahead
+        self.ring = torch.zeros(self.L + 2, NREC, self.ne, device=self.dev)   # (its ring: two slots more)
         self.work_bits = torch.zeros(self.hist_slots * self.fuse_hist_stride, dtype=torch.int64, device=self.dev)
         # one bit of the activity map per 2^shift sources: the smallest shift whose map fits the LDS beside the
-        # accumulators (16 wavefronts x (4 x 64 sums + a stage of 64 synapses) x 8 bytes)
-        fixed = FUSE_WAVES * (NREC * 64 + 64) * 8
+        # accumulators (16 wavefronts x 2 arrival steps x (4 x 64 sums + a stage of 64 synapses) x 8 bytes)
+        fixed = FUSE_WAVES * 2 * (NREC * 64 + 64) * 8
         self.fuse_shift = 0
-        while fixed + (self.L - 1) * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
+        while fixed + self.L * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
             self.fuse_shift += 1
         self.fuse_any = self._new_fuse_any()
 
@@ -287,9 +288,9 @@ class Glif3Simulator:
         whose map fits the LDS).  Before the first run only."""
         if self.fuse_table is None or self.step:
             raise ValueError("set_fuse_shift applies to the fused form before its first run")
-        fixed = FUSE_WAVES * (NREC * 64 + 64) * 8
+        fixed = FUSE_WAVES * 2 * (NREC * 64 + 64) * 8
         old, self.fuse_shift = self.fuse_shift, int(shift)
-        if not 0 <= self.fuse_shift <= 16 or fixed + (self.L - 1) * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
+        if not 0 <= self.fuse_shift <= 16 or fixed + self.L * self._fuse_any_words() * 4 > FUSE_LDS_BYTES:
             self.fuse_shift = old
             raise ValueError("shift must lie in 0..16 and leave the activity map within the LDS")
         self.fuse_any = self._new_fuse_any()
@@ -297,7 +298,7 @@ class Glif3Simulator:
     def _new_fuse_any(self):
         # the activity map (one row per history row) and, behind it, the map of ring cells that hold something
         # (one row per ring slot, a bit per neuron)
-        return torch.zeros(self.hist_slots * self._fuse_any_words() + self.L * (-(-self.n // 32)), dtype=torch.int32,
+        return torch.zeros(self.hist_slots * self._fuse_any_words() + (self.L + 2) * (-(-self.n // 32)), dtype=torch.int32,
                            device=self.dev)
 
     def _fuse_any_words(self):

@@ -312,22 +312,24 @@ typedef struct bmtk_glif3_sim {
     const int64_t *in_repeat_ptr;        /* [total steps + 1] */
     const int32_t *in_repeat_events;
     /* Fused form of the batched driver (optional; launch-per-step mode, batch 8, 16, 32 or 64, delay_offset 0,
-     * hist_slots == ring_slots + 2; takes precedence over pull_*): ONE launch per step in which a wavefront takes
-     * 64 / batch target neurons at a time -- it sums what arrives at them in step t-1 over recurrent AND input
-     * synapses in one pass over a joint target-major table (64-bit fixed point in LDS, as bmtk_csr_propagate_pull),
-     * folds the sums into y1 and advances the neurons' trials through step t, lane = (neuron, trial); no arrival
-     * sum passes through device memory.  The joint table's index field names a source of the joint space: neuron j is j,
+     * hist_slots == ring_slots + 4, `ring` of ring_slots + 2 slots; takes precedence over pull_*): one launch per TWO
+     * steps in which a wavefront takes 64 / batch target neurons at a time -- in one pass over a joint target-major
+     * table it sums what arrives at them in step t-1 and in step t over recurrent AND input synapses (64-bit fixed
+     * point in LDS, as bmtk_csr_propagate_pull; both only depend on spikes up to step t-1, delays being at least one
+     * step), folds the first sums into y1, advances the neurons' trials through step t, folds the second and
+     * advances them through step t+1, lane = (neuron, trial); no arrival sum passes through device memory and the
+     * table is read once per two steps.  The joint table's index field names a source of the joint space: neuron j is j,
      * input source k is fuse_in_base + k, fuse_in_base = ceil(n_neurons*batch/64)*64/batch.  work_bits is then the
      * joint history [hist_slots][fuse_hist_stride]: bit j*batch+b of row t % hist_slots = source j fired (or had an
      * input event) in trial b of step t; the driver writes the input part of row t from in_ptr / in_events in the
      * launch of step t.  Repeated ids of a step go through the ring as events (in_repeat_*, with inp_indptr /
      * inp_packed), as in the pull form.  fuse_any is the "some trial fired" map of the joint sources, one bit per
      * group of 2^fuse_shift sources and history row; a coarser map (larger shift) costs mask fetches for silent
-     * sources but is what lets any number of sources fit the LDS: (ring_slots-1) * fuse_any_words * 4 bytes beside
-     * the 40 KB of accumulators must stay within 150 KB. */
+     * sources but is what lets any number of sources fit the LDS: ring_slots * fuse_any_words * 4 bytes beside
+     * the 80 KB of accumulators must stay within 150 KB. */
     const int32_t *fuse_indptr;        /* [n_neurons + 1] */
     const bmtk_synapse *fuse_packed;   /* rows = targets, index field = joint source */
-    uint32_t *fuse_any;                /* [hist_slots][fuse_any_words] followed by [ring_slots][ceil(n_neurons/32)]
+    uint32_t *fuse_any;                /* [hist_slots][fuse_any_words] followed by [ring_slots + 2][ceil(n_neurons/32)]
                                         * words (a bit per neuron and ring slot: the slot holds an arrival of a
                                         * repeated id for the neuron), zeroed with work_bits before the first run;
                                         * fuse_any_words = ceil(ceil((fuse_in_base + n_inputs) / 2^fuse_shift) / 32) */
