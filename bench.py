@@ -166,14 +166,15 @@ def bench_compaction(torch, steps=200, warmup=20):
     return out
 
 
-PROPAGATION_MODES = ("scatter", "gather", "pull", "auto")
+PROPAGATION_MODES = ("scatter", "gather", "pull", "pull2", "auto")
 PROPAGATION_RATES = (0.2, 1.0, 5.0, 20.0)
 
 
 def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rates=PROPAGATION_RATES):
     """Isolated spike propagation: 51,978 neurons, Poisson(1000) in-degree
-    (~52 M synapses), batch 64, Bernoulli spikes at 0.2, 1, 5 and 20 Hz.  Four forms: the event-driven scatter, the
-    row-wise gather, the pull over the spike history of the last L steps, and `auto`, which decides on the device,
+    (~52 M synapses), batch 64, Bernoulli spikes at 0.2, 1, 5 and 20 Hz.  Five forms: the event-driven scatter, the
+    row-wise gather, the pull over the spike history of the last L steps, the same pull for two arrival steps per
+    pass over the table (`pull2`, timed per arrival step), and `auto`, which decides on the device,
     step by step, between pushing a step's spikes as events and leaving them to the pull.  A pool of L spike
     patterns serves as the history (row k % L = the spikes of step k)."""
     from bmtk_amd import ops, synthetic
@@ -204,6 +205,7 @@ def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rate
         active = sum(int(c.item()) for _, c, _ in pool_ev) / len(pool_ev)
         hist = torch.stack(pool_bits)                              # spike bits of the last L steps
         syn = torch.zeros(4, ne, device="cuda")
+        syn2 = torch.zeros(2, 4, ne, device="cuda")
         auto = ops.AutoPropagator(t_src, t_tgt, hist, ring, n, n, batch)
         for mode in modes:
             def one(k):
@@ -215,6 +217,9 @@ def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rate
                     auto.step(k, ids, count)
                 elif mode == "gather":
                     ops.csr_propagate_gather(pool_bits[k % L], n, t_tgt, ring, n, batch, k)
+                elif mode == "pull2":                                  # two arrival steps per call, every other step
+                    if k % 2 == 0:
+                        ops.csr_propagate_pull2(hist, n, t_tgt, syn2, n, batch, k + L + 1)
                 else:
                     ops.csr_propagate_pull(hist, n, t_tgt, syn, n, batch, k + L)
             for k in range(warmup):
@@ -224,10 +229,13 @@ def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rate
             per = dev / steps
             alg = events * B_PER_EVENT
             traffic = profile_traffic("propagation_kernels_52k_batch64.txt", "hbm_bytes_per_launch_%s_%gHz" % (mode, rate))
-            entry = {"kernel": {"auto": "auto_push_kernel or pull_kernel, chosen on the device"}.get(mode, mode + "_kernel"),
+            entry = {"kernel": {"auto": "auto_push_kernel or pull_kernel, chosen on the device",
+                                "pull2": "pull2_kernel: the arrivals of two steps per launch, half a launch per step"}
+                               .get(mode, mode + "_kernel"),
                      "workload": "propagation N=51978 nnz=%d batch=64 rate=%gHz" % (t_src.nnz, rate),
                      "events_per_launch": events, "active_elements_per_launch": active,
-                     "synaptic_events_per_s": events / per, "us_per_launch": per * 1e6,
+                     "synaptic_events_per_s": events / per, "us_per_launch": per * 1e6 * (2 if mode == "pull2" else 1),
+                     "us_per_arrival_step": per * 1e6,
                      "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS,
                                   "unit": "GB/s", "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
                                   "hbm_frac": None if traffic is None else traffic / per / 1e9 / HBM_PEAK_GBS}}
@@ -577,10 +585,10 @@ def kernel_summary(kernels):
                          "frac": r.get("frac"), "traffic": r.get("traffic")}
         elif w.startswith("propagation"):
             rate = w.split("rate=")[1]
-            out.setdefault("propagation_us_per_launch", {}).setdefault(rate, {})[k["kernel"].split(" ")[0]] = \
-                round(k["us_per_launch"], 1)
+            out.setdefault("propagation_us_per_arrival_step", {}).setdefault(rate, {})[k["kernel"].split(" ")[0].rstrip(":")] = \
+                round(k["us_per_arrival_step"], 1)
             if k["kernel"].startswith(("pull", "auto")):
-                out.setdefault("propagation_frac", {}).setdefault(rate, {})[k["kernel"].split(" ")[0]] = \
+                out.setdefault("propagation_frac", {}).setdefault(rate, {})[k["kernel"].split(" ")[0].rstrip(":")] = \
                     {"frac": r.get("frac"), "hbm_frac": r.get("hbm_frac"), "events_per_s": k["synaptic_events_per_s"]}
         elif w.startswith("BPTT step"):
             out["bptt_step"] = {"forward_s": k["forward_s"], "backward_s": k["backward_s"],

@@ -60,7 +60,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 20  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 21  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -86,6 +86,8 @@ SIGNATURES = {
     "bmtk_csr_propagate_pull_workspace_bytes": (c_int64, [c_int32, c_int64]),
     "bmtk_csr_propagate_pull": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
                                           c_int64, c_int64, c_void_p, c_void_p]),
+    "bmtk_csr_propagate_pull2": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
+                                           c_int64, c_int64, c_void_p, c_void_p]),
     "bmtk_csr_pack": (c_int32, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "bmtk_csr_pack_wide": (c_int32, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p]),
     "bmtk_csr_segment_offsets": (c_int32, [c_int64, c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p,

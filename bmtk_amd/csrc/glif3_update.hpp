@@ -45,32 +45,6 @@ struct Glif3Prop {
             psc0[k] = p[(GLIF3_PSC0_0 + k) * stride];
         }
     }
-
-    // The same from a wavefront register that holds row k of the column in lane k (one load instruction fetched the
-    // whole column): every lane gets every entry, through scalar registers.
-    __device__ __forceinline__ void load_from_lanes(float column)
-    {
-        auto at = [&](int k) { return bcast_f(column, k); };
-        P33 = at(GLIF3_P33);
-        P30 = at(GLIF3_P30);
-        th = at(GLIF3_TH);
-        Ur = at(GLIF3_UR);
-        n_ref = (int)at(GLIF3_NREF);
-#pragma unroll
-        for (int a = 0; a < GLIF3_NASC; ++a) {
-            c[a] = at(GLIF3_C0 + a);
-            d[a] = at(GLIF3_D0 + a);
-            r[a] = at(GLIF3_R0 + a);
-            amp[a] = at(GLIF3_AMP0 + a);
-        }
-#pragma unroll
-        for (int k = 0; k < GLIF3_NREC; ++k) {
-            P11[k] = at(GLIF3_P11_0 + k);
-            P31[k] = at(GLIF3_P31_0 + k);
-            P32[k] = at(GLIF3_P32_0 + k);
-            psc0[k] = at(GLIF3_PSC0_0 + k);
-        }
-    }
 };
 
 // Advance one element by one step.  syn[r]: weight sum arriving on receptor r

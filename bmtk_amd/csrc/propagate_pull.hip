@@ -198,6 +198,127 @@ __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__r
     } while (b0.row < n_tgt);
 }
 
+// What arrives in TWO consecutive steps, t-1 and t, in one pass over the table.  Both sums only depend on the spikes
+// of steps up to t-1 (delays are at least one step), so a caller that advances two steps between calls needs the
+// table -- most of the bytes of a call at low rates -- half as often.  Per synapse two questions (did the source
+// fire in step t-1-delay, in step t-delay), two stages, two sets of sums; otherwise pull_kernel.  One workgroup of
+// 1024 threads per compute unit (its two sets of accumulators and stages take 80 KB of LDS).
+constexpr size_t kPull2AccBytes = 2 * kPullAccBytes;
+constexpr size_t kPull2LdsMax = 150u * 1024u;
+template <bool kWords64>
+__global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride, int L,
+                                                           int batch, const int32_t *__restrict__ indptr,
+                                                           const bmtk_synapse *__restrict__ packed,
+                                                           float *__restrict__ syn2, int64_t n_tgt, int64_t ne,
+                                                           int slot_now, const uint32_t *__restrict__ any_map, int n_w32)
+{
+    extern __shared__ unsigned long long pull_lds[];  // accumulators [wave][step][4][64], stages [wave][step][64], map
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    constexpr int kWaves = kPullBlock / kWave;
+    unsigned long long *acc = pull_lds + wave * (2 * GLIF3_NREC * kWave);
+    uint2 *stage = reinterpret_cast<uint2 *>(pull_lds + kWaves * 2 * GLIF3_NREC * kWave) + wave * 2 * kWave;
+    uint32_t *any_l = reinterpret_cast<uint32_t *>(pull_lds + kWaves * 2 * (GLIF3_NREC + 1) * kWave);
+    const unsigned lane = (unsigned)lane_id();
+    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
+    __syncthreads();
+    const int tile0 = kWords64 ? 0 : (int)blockIdx.y * kWave;
+    const int width = kWords64 ? kWave : min(kWave, batch - tile0);
+    const unsigned hstride = (unsigned)hist_stride;  // L * hist_stride * 8 < 2^32 bytes (checked by the caller)
+    const unsigned uL = (unsigned)L, uw32 = (unsigned)n_w32;
+    const unsigned now_b = (unsigned)slot_now, now_a = (unsigned)((slot_now + L - 1) % L);  // rows of steps t and t-1
+    const char *__restrict__ hist_bytes = reinterpret_cast<const char *>(hist);
+    auto fetch = [&](unsigned long long *dst, const PullBlock &blk) {
+        const bool some = blk.row < n_tgt && blk.base < blk.p1;
+        const char *__restrict__ src = reinterpret_cast<const char *>(packed) + (some ? (size_t)blk.base * 8u : (size_t)0);
+        const unsigned last = some ? (unsigned)(blk.p1 - blk.base) - 1u : 0u;
+#pragma unroll
+        for (int u = 0; u < kPullChunks; ++u)
+            dst[u] = __builtin_nontemporal_load(
+                reinterpret_cast<const unsigned long long *>(src + min(lane + u * kWave, last) * 8u));
+    };
+    PullCursor cursor;
+    cursor.start(indptr, n_tgt, (int64_t)blockIdx.x * kWaves + wave, (int64_t)gridDim.x * kWaves);
+    PullBlock b0 = cursor.next();
+    if (b0.row >= n_tgt) return;
+    unsigned long long d0[kPullChunks] = {0ull, 0ull, 0ull, 0ull}, d1[kPullChunks] = {0ull, 0ull, 0ull, 0ull};
+    fetch(d0, b0);
+    PullBlock b1 = cursor.next();
+    fetch(d1, b1);
+#pragma unroll
+    for (int r = 0; r < 2 * GLIF3_NREC; ++r) acc[r * kWave + lane] = 0ull;
+    int staged[2] = {0, 0};  // entries in the two stages (same in all lanes)
+    // the staged synapses of one arrival step: gather their trial masks, convert their weights, add
+    auto flush = [&](int k) {
+        if ((int)lane < staged[k]) {
+            const uint2 e = stage[k * kWave + lane];  // {source | receptor << 24 | delay << 26, weight}
+            const unsigned src = e.x & 0xFFFFFFu;
+            const unsigned back = (k ? now_b : now_a) - (e.x >> 26);  // history row of the emitting step
+            const unsigned row = min(back, back + uL);
+            unsigned long long mm;
+            if (kWords64)
+                mm = *reinterpret_cast<const unsigned long long *>(hist_bytes + (__umul24(row, hstride) + src) * 8u);
+            else
+                mm = source_mask(hist + (size_t)row * hstride, (int)src, batch, tile0, width);
+            unsigned long long *a = acc + (k * GLIF3_NREC + ((e.x >> 24) & 3u)) * kWave;
+            const unsigned long long w = to_fixed(__uint_as_float(e.y));
+            while (mm) {
+                const int b = __ffsll((long long)mm) - 1;
+                mm &= mm - 1ull;
+                atomicAdd(a + b, w);
+            }
+        }
+        staged[k] = 0;
+    };
+    auto turn = [&](PullBlock &cb, unsigned long long *cd) {
+        const unsigned left = cb.base < cb.p1 ? (unsigned)(cb.p1 - cb.base) : 0u;
+        // activity bits of the four chunks for both arrival steps (LDS reads, no branch between them): the map of a
+        // step is the row of its history slot; a synapse of delay d looks at step t-1-d and at step t-d
+        unsigned word_a[kPullChunks], word_b[kPullChunks];
+#pragma unroll
+        for (int u = 0; u < kPullChunks; ++u) {
+            const unsigned tdr = (unsigned)cd[u];
+            const unsigned back_b = now_b - (tdr >> 26), back_a = now_a - (tdr >> 26);
+            const unsigned at = (tdr & 0xFFFFFFu) >> 5;
+            word_b[u] = any_l[__umul24(min(back_b, back_b + uL), uw32) + at];
+            word_a[u] = any_l[__umul24(min(back_a, back_a + uL), uw32) + at];
+        }
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+#pragma unroll
+            for (int u = 0; u < kPullChunks; ++u) {
+                const unsigned tdr = (unsigned)cd[u];
+                const bool hit = lane + u * kWave < left && (((k ? word_b[u] : word_a[u]) >> (tdr & 31u)) & 1u);
+                const unsigned long long who = __ballot(hit);
+                const int n = __popcll(who);
+                if (n == 0) continue;
+                if (staged[k] + n > kWave) flush(k);
+                if (hit) stage[k * kWave + staged[k] + lane_prefix(who)] = make_uint2(tdr, (unsigned)(cd[u] >> 32));
+                staged[k] += n;
+            }
+        }
+        if (cb.last) {
+            flush(0);
+            flush(1);
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+#pragma unroll
+                for (int r = 0; r < GLIF3_NREC; ++r) {
+                    unsigned long long *cell = acc + (k * GLIF3_NREC + r) * kWave + lane;
+                    if ((int)lane < width)
+                        syn2[((int64_t)k * GLIF3_NREC + r) * ne + cb.row * batch + tile0 + lane] = from_fixed(*cell);
+                    *cell = 0ull;
+                }
+            }
+        }
+        cb = cursor.next();
+        fetch(cd, cb);
+    };
+    do {  // (one way out, after a whole round of the buffers: see pull_kernel)
+        turn(b0, d0);
+        turn(b1, d1);
+    } while (b0.row < n_tgt);
+}
+
 // bmtk_csr_propagate_auto, first launch: the spikes of step `step` as events, if they are few.  Every workgroup
 // reads the number of active elements and decides the same way; up to cnt_max the elements' rows are walked and
 // their weights pushed into the ring (fp32 atomics), above it nothing happens here and the step is left to the
@@ -390,5 +511,59 @@ extern "C" int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_a
         hipLaunchKernelGGL((pull_kernel<false, true>), grid, dim3(kPullBlock), lds, st, spike_hist, hist_stride, L, batch,
                            tgt_indptr, tgt_packed, cells, n_tgt, ne, slot_arrive, any_map, n_w32, (const int32_t *)ctrl);
     BMTK_CHECK_LAUNCH("csr_propagate_auto");
+    return BMTK_OK;
+}
+
+extern "C" int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src,
+                                        int32_t batch, const int32_t *indptr, const bmtk_synapse *packed, float *syn2,
+                                        int64_t n_tgt, int64_t t_arrive, void *workspace, void *stream)
+{
+    using namespace bmtk;
+    BMTK_REQUIRE(spike_hist && indptr && packed && syn2 && workspace, "csr_propagate_pull2: pointers must be non-null");
+    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && n_src > 0 && t_arrive >= 1, "csr_propagate_pull2: bad batch, sizes or step");
+    BMTK_REQUIRE(L > 1 && L <= 64, "csr_propagate_pull2: L must lie in 2..64");
+    BMTK_REQUIRE(hist_stride >= (n_src * (int64_t)batch + 63) / 64 + 1,
+                 "csr_propagate_pull2: hist_stride must hold ceil(n_src*batch/64)+1 words");
+    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31) && n_src < (1ll << 24), "csr_propagate_pull2: network too large");
+    BMTK_REQUIRE((int64_t)L * hist_stride < (1ll << 29) && hist_stride < (1ll << 24),
+                 "csr_propagate_pull2: spike history beyond 4 GiB");
+    const int n_w32 = (int)((n_src + 31) / 32);
+    const size_t lds = (size_t)L * n_w32 * 4 + kPull2AccBytes;
+    BMTK_REQUIRE(lds <= kPull2LdsMax, "csr_propagate_pull2: L * n_src too large for the activity map in LDS");
+    uint32_t *any_map = (uint32_t *)workspace;
+    const int64_t map_threads = (int64_t)L * n_w32 * 32;
+    hipLaunchKernelGGL(pull_anymap_kernel, dim3((unsigned)((map_threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, spike_hist, hist_stride, L, batch, n_src, n_w32, any_map);
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    static int cu_count[64];
+    int n_cu = (dev >= 0 && dev < 64) ? cu_count[dev] : 0;
+    if (n_cu <= 0) {
+        n_cu = 256;
+        (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (dev >= 0 && dev < 64) cu_count[dev] = n_cu;
+    }
+    const unsigned rows_per_block = kPullBlock / kWave;
+    const unsigned want = (unsigned)((n_tgt + rows_per_block - 1) / rows_per_block);
+    const dim3 grid(want < (unsigned)n_cu ? want : (unsigned)n_cu, (unsigned)((batch + kWave - 1) / kWave));
+    BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_pull2: batch too large");
+    static bool asked[2][64];
+    if (dev >= 0 && dev < 64 && !asked[batch == kWave][dev]) {
+        const hipError_t err = hipFuncSetAttribute(
+            batch == kWave ? reinterpret_cast<const void *>(pull2_kernel<true>) : reinterpret_cast<const void *>(pull2_kernel<false>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPull2LdsMax);
+        if (err != hipSuccess) {
+            set_error("csr_propagate_pull2: cannot reserve %zu bytes of LDS: %s", kPull2LdsMax, hipGetErrorString(err));
+            return BMTK_E_LAUNCH;
+        }
+        asked[batch == kWave][dev] = true;
+    }
+    if (batch == kWave)
+        hipLaunchKernelGGL(pull2_kernel<true>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
+                           batch, indptr, packed, syn2, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
+    else
+        hipLaunchKernelGGL(pull2_kernel<false>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
+                           batch, indptr, packed, syn2, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
+    BMTK_CHECK_LAUNCH("csr_propagate_pull2");
     return BMTK_OK;
 }

@@ -40,10 +40,7 @@ namespace bmtk {
 
 constexpr int kFuseBlock = 1024;
 constexpr int kFuseWaves = kFuseBlock / kWave;
-#ifndef FUSE_AHEAD
-#define FUSE_AHEAD 2
-#endif
-constexpr int kFuseAhead = FUSE_AHEAD;  // table blocks of 2 KB per wavefront, in flight or at hand (4 and 5: no faster)
+constexpr int kFuseAhead = 2;  // table blocks of 2 KB per wavefront, in flight or at hand (4 and 5: no faster)
 constexpr size_t kFuseLdsMax = 150u * 1024u;  // one workgroup per compute unit
 
 struct FusedLaunch {

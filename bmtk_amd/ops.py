@@ -382,6 +382,25 @@ def csr_propagate_pull(spike_hist, n_src, table, syn, n_tgt, batch, t_arrive):
                                            int(t_arrive), _p(ws), _stream()))
 
 
+def csr_propagate_pull2(spike_hist, n_src, table, syn2, n_tgt, batch, t_arrive):
+    """Everything arriving in steps ``t_arrive - 1`` and ``t_arrive`` in one pass over a target-major table, from
+    the spike bits of steps ``t_arrive - L .. t_arrive - 1`` (``spike_hist`` int64 [L, words+1], row k mod L = bits
+    of step k); overwrites ``syn2`` [2, 4, n_tgt*batch]."""
+    lib = _lib.load()
+    if table.n_rows != n_tgt or syn2.numel() != 2 * NREC * n_tgt * batch:
+        raise ValueError("target-major table must have one row per target and syn2 must be [2, 4, n_tgt*batch]")
+    L = spike_hist.shape[0]
+    if table.max_delay() >= L:
+        raise ValueError("spike history of {} steps is shorter than the largest delay".format(L))
+    ws = getattr(table, "_pull_ws", None)
+    need = lib.bmtk_csr_propagate_pull_workspace_bytes(L, n_src)
+    if ws is None or ws.numel() * 4 < need:
+        ws = table._pull_ws = torch.zeros(need // 4 + 1, dtype=torch.int32, device=syn2.device)
+    _lib.check(lib.bmtk_csr_propagate_pull2(_p(spike_hist, torch.int64), spike_hist.shape[1], L, n_src, batch,
+                                            _p(table.indptr), _p(table.packed()), _p(syn2, torch.float32), n_tgt,
+                                            int(t_arrive), _p(ws), _stream()))
+
+
 def csr_propagate_bwd(table, lam_ring, n, batch, step, gz=None, trials_per_lane=0):
     """Transposed propagation (adjoint of the delivery) through a source-major table of ``n`` rows:
     ``gz[j*batch+b] = sum_(j->i,w,d,r) w * lam_ring[(step+d) % L, r, i*batch+b]``.  ``trials_per_lane`` 0 lets the

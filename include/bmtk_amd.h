@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 20
+#define BMTK_AMD_ABI_VERSION 21
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -175,6 +175,17 @@ int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_active, int6
                             const int32_t *tgt_indptr, const bmtk_synapse *tgt_packed,
                             float *ring, int64_t n_tgt, int64_t step, int64_t scatter_max_active, void *workspace,
                             void *stream);
+
+/* The same for TWO consecutive arrival steps in one pass over the table: syn2[0][r][..] is what arrives in step
+ * t_arrive - 1, syn2[1][r][..] what arrives in step t_arrive ([2][4][n_tgt*batch], overwritten).  Both only depend
+ * on the spikes of steps up to t_arrive - 1 (delays are at least one step): spike_hist must hold the steps
+ * t_arrive - L .. t_arrive - 1 (row k mod L = step k).  A caller that advances two steps between calls -- sums of
+ * t-1 into the update of t, sums of t into the update of t+1 -- reads the table, most of a call's bytes at low
+ * rates, once per two steps (the batched simulation driver does the same inside its launches).  Workspace and
+ * limits as bmtk_csr_propagate_pull, except that the bit map may take up to 70 KB of LDS. */
+int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src, int32_t batch,
+                             const int32_t *indptr, const bmtk_synapse *packed, float *syn2, int64_t n_tgt,
+                             int64_t t_arrive, void *workspace, void *stream);
 
 /* Packed synapse format used by the fused simulation: one 8-byte record per
  * synapse, {uint32 tdr, float weight} with tdr = index | receptor << 24 |
@@ -321,8 +332,8 @@ typedef struct bmtk_glif3_sim {
      * table is read once per two steps.  The joint table's index field names a source of the joint space: neuron j is j,
      * input source k is fuse_in_base + k, fuse_in_base = ceil(n_neurons*batch/64)*64/batch.  work_bits is then the
      * joint history [hist_slots][fuse_hist_stride]: bit j*batch+b of row t % hist_slots = source j fired (or had an
-     * input event) in trial b of step t; the driver writes the input part of row t from in_ptr / in_events in the
-     * launch of step t.  Repeated ids of a step go through the ring as events (in_repeat_*, with inp_indptr /
+     * input event) in trial b of step t; a launch writes the input parts of the rows of its own two steps from in_ptr /
+     * in_events, for the launches after it.  Repeated ids of a step go through the ring as events (in_repeat_*, with inp_indptr /
      * inp_packed), as in the pull form.  fuse_any is the "some trial fired" map of the joint sources, one bit per
      * group of 2^fuse_shift sources and history row; a coarser map (larger shift) costs mask fetches for silent
      * sources but is what lets any number of sources fit the LDS: ring_slots * fuse_any_words * 4 bytes beside
