@@ -60,7 +60,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 21  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 22  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -98,6 +98,8 @@ SIGNATURES = {
                                     c_void_p, c_void_p, c_void_p, c_void_p]),
     "bmtk_glif3_simulate_fwd": (c_int32, [C.POINTER(Glif3Sim), c_int64, c_int64, c_void_p]),
     "bmtk_glif3_simulate_bwd": (c_int32, [C.POINTER(Glif3Bwd), c_int64, c_int64, c_void_p]),
+    "bmtk_glif3_step_bwd": (c_int32, [C.POINTER(Glif3Bwd), c_int64, c_int64, c_int32, c_void_p]),
+    "bmtk_csr_weight_grad": (c_int32, [C.POINTER(Glif3Bwd), c_int64, c_int64, c_void_p]),
     "bmtk_csr_propagate_bwd": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int32, c_int64, c_void_p,
                                          c_int32, c_void_p]),
     "bmtk_csr_propagate_bwd_blocked": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int32, c_int64,

@@ -785,22 +785,44 @@ int blocked_launch(const bmtk_glif3_bwd &a, const BwdStep &q, const BlockedPlan 
 
 }  // namespace
 
+namespace {
+
+// what every entry point that takes the whole bmtk_glif3_bwd requires of it
+int bwd_check(const bmtk_glif3_bwd *bwd, const char *who)
+{
+    BMTK_REQUIRE(bwd != nullptr, "%s: bwd is null", who);
+    const bmtk_glif3_bwd &a = *bwd;
+    BMTK_REQUIRE(a.n_neurons > 0 && a.batch > 0, "%s: n_neurons and batch must be positive", who);
+    const int64_t ne = a.n_neurons * (int64_t)a.batch;
+    BMTK_REQUIRE(ne < (1ll << 31) && a.n_neurons < (1ll << 24), "%s: network too large", who);
+    BMTK_REQUIRE(a.ring_slots > 1 && a.ring_slots <= 64, "%s: ring_slots must lie in 2..64", who);
+    BMTK_REQUIRE(a.h > 0.0f && a.dampening >= 0.0f, "%s: h must be positive, dampening non-negative", who);
+    BMTK_REQUIRE(a.prop && a.prop_stride > 0 && (a.class_id || a.prop_stride >= a.n_neurons),
+                 "%s: prop table missing or too small", who);
+    BMTK_REQUIRE(a.save_v && a.save_flags && a.spike_bits, "%s: the forward record is incomplete", who);
+    BMTK_REQUIRE(a.spike_bits_stride >= (ne + 63) / 64, "%s: spike_bits_stride too small", who);
+    BMTK_REQUIRE(a.lam_V && a.lam_asc && a.lam_y1 && a.lam_y2 && a.lam_ring && a.gz,
+                 "%s: adjoint state pointers must be non-null", who);
+    BMTK_REQUIRE(!(a.dl_dz && a.dl_dz_const), "%s: give dl_dz or dl_dz_const, not both", who);
+    const bool has_rec = a.rec_indptr != nullptr;
+    BMTK_REQUIRE(!has_rec || a.rec_packed, "%s: recurrent table needs rec_packed", who);
+    BMTK_REQUIRE(!a.d_rec_w || has_rec, "%s: d_rec_w without a recurrent table", who);
+    BMTK_REQUIRE(!a.d_blk_w || a.blk_count != 0, "%s: d_blk_w without the blocked table", who);
+    BMTK_REQUIRE(!a.d_inp_w || (a.in_ptr && a.in_events && a.inp_indptr && a.inp_packed),
+                 "%s: d_inp_w needs the input events and the input table", who);
+    return BMTK_OK;
+}
+
+}  // namespace
+
 extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_steps, void *stream)
 {
-    BMTK_REQUIRE(bwd != nullptr, "glif3_simulate_bwd: bwd is null");
+    {
+        const int rc = bwd_check(bwd, "glif3_simulate_bwd");
+        if (rc != BMTK_OK) return rc;
+    }
     const bmtk_glif3_bwd &a = *bwd;
-    BMTK_REQUIRE(a.n_neurons > 0 && a.batch > 0, "glif3_simulate_bwd: n_neurons and batch must be positive");
     const int64_t ne = a.n_neurons * (int64_t)a.batch;
-    BMTK_REQUIRE(ne < (1ll << 31) && a.n_neurons < (1ll << 24), "glif3_simulate_bwd: network too large");
-    BMTK_REQUIRE(a.ring_slots > 1 && a.ring_slots <= 64, "glif3_simulate_bwd: ring_slots must lie in 2..64");
-    BMTK_REQUIRE(a.h > 0.0f && a.dampening >= 0.0f, "glif3_simulate_bwd: h must be positive, dampening non-negative");
-    BMTK_REQUIRE(a.prop && a.prop_stride > 0 && (a.class_id || a.prop_stride >= a.n_neurons),
-                 "glif3_simulate_bwd: prop table missing or too small");
-    BMTK_REQUIRE(a.save_v && a.save_flags && a.spike_bits, "glif3_simulate_bwd: the forward record is incomplete");
-    BMTK_REQUIRE(a.spike_bits_stride >= (ne + 63) / 64, "glif3_simulate_bwd: spike_bits_stride too small");
-    BMTK_REQUIRE(a.lam_V && a.lam_asc && a.lam_y1 && a.lam_y2 && a.lam_ring && a.gz,
-                 "glif3_simulate_bwd: adjoint state pointers must be non-null");
-    BMTK_REQUIRE(!(a.dl_dz && a.dl_dz_const), "glif3_simulate_bwd: give dl_dz or dl_dz_const, not both");
     const bool blocked = a.blk_count != 0;
     BlockedPlan pl{};
     if (blocked) {
@@ -809,12 +831,7 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
         if (rc != BMTK_OK) return rc;
     }
     const bool has_rec = a.rec_indptr != nullptr;
-    BMTK_REQUIRE(!has_rec || a.rec_packed, "glif3_simulate_bwd: recurrent table needs rec_packed");
-    BMTK_REQUIRE(!a.d_rec_w || has_rec, "glif3_simulate_bwd: d_rec_w without a recurrent table");
-    BMTK_REQUIRE(!a.d_blk_w || blocked, "glif3_simulate_bwd: d_blk_w without the blocked table");
     const bool inp_grad = a.d_inp_w != nullptr;
-    BMTK_REQUIRE(!inp_grad || (a.in_ptr && a.in_events && a.inp_indptr && a.inp_packed),
-                 "glif3_simulate_bwd: d_inp_w needs the input events and the input table");
     BMTK_REQUIRE(step0 >= 0 && n_steps >= 0, "glif3_simulate_bwd: step0 and n_steps must be non-negative");
     hipStream_t st = (hipStream_t)stream;
     const unsigned rows_grid = (unsigned)((a.n_neurons + kBlock / kWave - 1) / (kBlock / kWave));
@@ -850,6 +867,38 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
         if (a.d_rec_w && !fused) hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
     }
     BMTK_CHECK_LAUNCH("glif3_simulate_bwd");
+    return BMTK_OK;
+}
+
+extern "C" int bmtk_glif3_step_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t k, int32_t gz_parts, void *stream)
+{
+    const int rc = bwd_check(bwd, "glif3_step_bwd");
+    if (rc != BMTK_OK) return rc;
+    BMTK_REQUIRE(step0 >= 0 && k >= 0, "glif3_step_bwd: step0 and k must be non-negative");
+    BMTK_REQUIRE(gz_parts == 1 || gz_parts == 8, "glif3_step_bwd: gz holds 1 sum or 8 partial sums per element");
+    const bmtk_glif3_bwd &a = *bwd;
+    const int64_t ne = a.n_neurons * (int64_t)a.batch;
+    BwdStep q{step0 + k, k, gz_parts};
+    hipLaunchKernelGGL(bwd_state_kernel, dim3((unsigned)((ne + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, a, q, 0);
+    BMTK_CHECK_LAUNCH("glif3_step_bwd");
+    return BMTK_OK;
+}
+
+extern "C" int bmtk_csr_weight_grad(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t k, void *stream)
+{
+    const int rc = bwd_check(bwd, "csr_weight_grad");
+    if (rc != BMTK_OK) return rc;
+    BMTK_REQUIRE(step0 >= 0 && k >= 0, "csr_weight_grad: step0 and k must be non-negative");
+    const bmtk_glif3_bwd &a = *bwd;
+    BMTK_REQUIRE(a.d_rec_w || a.d_inp_w, "csr_weight_grad: neither d_rec_w nor d_inp_w is given");
+    BwdStep q{step0 + k, k, 1};
+    if (a.d_rec_w)
+        hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3((unsigned)((a.n_neurons + kBlock / kWave - 1) / (kBlock / kWave))),
+                           dim3(kBlock), 0, (hipStream_t)stream, a, q);
+    if (a.d_inp_w)  // (bwd_state_kernel with nothing but gradient workgroups)
+        hipLaunchKernelGGL(bwd_state_kernel, dim3(kInpGradGrid), dim3(kBlock), 0, (hipStream_t)stream, a, q, kInpGradGrid);
+    BMTK_CHECK_LAUNCH("csr_weight_grad");
     return BMTK_OK;
 }
 

@@ -86,10 +86,7 @@ class Glif3Bptt:
             if t is not None:
                 t.zero_()
 
-    def backward(self, fwd, dl_dz_const=None, dl_dz=None):
-        """``fwd`` is what ``sim.run(n, save_state=True)`` returned.  Accumulates
-        into ``d_rec_w`` / ``d_inp_w`` (same order as ``sim.rec`` / ``sim.inp``).
-        Calls for consecutive chunks must come in reverse time order."""
+    def _struct(self, fwd, dl_dz_const, dl_dz, blocked):
         sim, saved, bits = self.sim, fwd["saved"], fwd["bits"]
         if saved is None or bits is None:
             raise ValueError("forward run was made without save_state=True or without spike bits")
@@ -101,7 +98,7 @@ class Glif3Bptt:
         a.spike_bits, a.spike_bits_stride = _p(bits, torch.int64), bits.shape[1]
         if sim.rec is not None:
             a.rec_indptr, a.rec_packed = _p(sim.rec.indptr), _p(sim.rec.packed())
-            if self.blk is None:
+            if not blocked:
                 a.d_rec_w = _p(self.d_rec_w)
             else:
                 a.blk_count, a.blk_indptr, a.blk_packed = self.n_blocks, _p(self.blk[0]), _p(self.blk[1])
@@ -114,7 +111,34 @@ class Glif3Bptt:
         a.dl_dz_const = _p(dl_dz_const, torch.float32, sim.ne, "dl_dz_const")
         a.lam_V, a.lam_asc, a.lam_y1, a.lam_y2 = (_p(x) for x in (self.lam_V, self.lam_asc, self.lam_y1, self.lam_y2))
         a.lam_ring, a.gz = _p(self.lam_ring), _p(self.gz)
-        _lib.check(self.lib.bmtk_glif3_simulate_bwd(C.byref(a), saved["step0"], n_steps, _stream()))
+        return a, saved["step0"], n_steps
+
+    def backward(self, fwd, dl_dz_const=None, dl_dz=None):
+        """``fwd`` is what ``sim.run(n, save_state=True)`` returned.  Accumulates
+        into ``d_rec_w`` / ``d_inp_w`` (same order as ``sim.rec`` / ``sim.inp``).
+        Calls for consecutive chunks must come in reverse time order."""
+        a, step0, n_steps = self._struct(fwd, dl_dz_const, dl_dz, self.blk is not None)
+        _lib.check(self.lib.bmtk_glif3_simulate_bwd(C.byref(a), step0, n_steps, _stream()))
         if self.blk is not None:  # the blocked kernel accumulates in its table's order: back to the order of sim.rec
             self.d_rec_w.index_add_(0, self.blk[2], self.d_blk_w)
             self.d_blk_w.zero_()
+
+    def backward_stepwise(self, fwd, dl_dz_const=None, dl_dz=None, between=None):
+        """The same pass as a loop over the three per-step entry points (transposed propagation through the
+        source-major table, state adjoint, weight gradients), calling ``between(k)`` after the state adjoint of
+        record row ``k`` -- the place for work of the caller's own on the adjoint state (clipping, a loss that
+        depends on it).  Several launches per step where ``backward`` has two: for training loops use ``backward``."""
+        from . import ops
+        sim = self.sim
+        a, step0, n_steps = self._struct(fwd, dl_dz_const, dl_dz, False)
+        gz = self.gz[:sim.ne]
+        for k in range(n_steps - 1, -1, -1):
+            if sim.rec is not None:
+                ops.csr_propagate_bwd(sim.rec, self.lam_ring, sim.n, sim.batch, step0 + k, gz=gz)
+            else:
+                gz.zero_()
+            _lib.check(self.lib.bmtk_glif3_step_bwd(C.byref(a), step0, k, 1, _stream()))
+            if self.d_rec_w is not None or self.d_inp_w is not None:
+                _lib.check(self.lib.bmtk_csr_weight_grad(C.byref(a), step0, k, _stream()))
+            if between is not None:
+                between(k)

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 21
+#define BMTK_AMD_ABI_VERSION 22
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -501,6 +501,20 @@ typedef struct bmtk_glif3_bwd {
 /* Differentiate steps step0+n_steps-1 down to step0 (three launches per step:
  * transposed propagation, state adjoint, weight gradients). */
 int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_steps, void *stream);
+
+/* One backward step in its three parts, for callers that put their own work between them (a loss that is computed
+ * step by step, truncation, clipping of the adjoint); no counterpart in the reference.  Both take the same struct
+ * as bmtk_glif3_simulate_bwd and differentiate step step0 + k, whose forward record is row k.
+ *  - bmtk_glif3_step_bwd: the state adjoint.  bwd->gz must hold the adjoint of the step's spikes that comes back
+ *    through the synapses, as bmtk_csr_propagate_bwd (gz_parts = 1) or bmtk_csr_propagate_bwd_blocked (gz_parts =
+ *    8 partial sums) leave it, or zeros; the loss derivative of the step is added to it.  Updates lam_V, lam_asc,
+ *    lam_y1, lam_y2 and writes slot (step0 + k) % ring_slots of lam_ring.
+ *  - bmtk_csr_weight_grad: d_rec_w += and d_inp_w += the step's contributions (whichever is given; d_blk_w is not
+ *    served).  Reads the slots of the steps ahead only, so it may run before or after the state adjoint of the
+ *    same step, but before that of step step0 + k - 1.
+ * One step of bmtk_glif3_simulate_bwd == bmtk_csr_propagate_bwd, bmtk_glif3_step_bwd, bmtk_csr_weight_grad. */
+int bmtk_glif3_step_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t k, int32_t gz_parts, void *stream);
+int bmtk_csr_weight_grad(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t k, void *stream);
 
 /* The transposed propagation of the backward pass on its own (the adjoint of the delivery; no counterpart in the
  * reference): through a packed SOURCE-major table of n_neurons rows,

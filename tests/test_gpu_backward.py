@@ -198,3 +198,54 @@ def test_state_adjoint_kernel_transposes_the_state_update():
     rhs = sum(float((jt_u[k].double().cpu().numpy().reshape(v[k].shape) * v[k].astype(np.float64)).sum()) for k in x0)
     assert abs(lhs) > 1.0
     assert abs(lhs - rhs) <= 1e-4 * abs(lhs), (lhs, rhs)
+
+
+@pytest.mark.parametrize("batch,seed", [(1, 2), (3, 4), (8, 8), (32, 9), (100, 12)])
+def test_backward_pass_in_its_three_parts_equals_the_fused_driver(batch, seed):
+    """``bmtk_csr_propagate_bwd`` + ``bmtk_glif3_step_bwd`` + ``bmtk_csr_weight_grad`` step by step ==
+    ``bmtk_glif3_simulate_bwd`` (pinned against autograd above): the adjoint state bit for bit (the same kernels
+    in the same order; the driver's skipped rows have a zero surrogate derivative), the gradients bit for bit where
+    the driver uses the same gradient kernels (more than 64 trials) and to 1e-6 of the largest entry otherwise (the
+    driver's gradient rides along with the transposed propagation there and adds a row's trials in another
+    order).  ``between`` sees every step once, last step first."""
+    cfg = _net(batch, seed)
+    n, T, h = cfg["n"], cfg["steps"], cfg["h"]
+    ne = n * batch
+    sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                         resident=False)
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    fwd = sim.run(T, save_state=True)
+    dl = torch.as_tensor(np.random.default_rng(seed).normal(size=(T, ne)).astype(np.float32), device="cuda")
+    whole = training.Glif3Bptt(sim, dampening=0.3, blocked=False)
+    whole.backward(fwd, dl_dz=dl)
+    parts = training.Glif3Bptt(sim, dampening=0.3, blocked=False)
+    seen = []
+    parts.backward_stepwise(fwd, dl_dz=dl, between=seen.append)
+    assert seen == list(range(T - 1, -1, -1))
+    for name in ("lam_V", "lam_asc", "lam_y1", "lam_y2", "lam_ring"):
+        assert torch.equal(getattr(parts, name), getattr(whole, name)), name
+    assert float(whole.lam_V.abs().max()) > 0 and float(whole.d_rec_w.abs().max()) > 0
+    for name in ("d_rec_w", "d_inp_w"):
+        got, want = getattr(parts, name), getattr(whole, name)
+        if batch > 64:
+            assert torch.equal(got, want), name
+        else:
+            assert float((got - want).abs().max()) <= 1e-6 * float(want.abs().max()), name
+
+
+def test_backward_parts_argument_errors():
+    cfg = _net(4, 6)
+    sim = Glif3Simulator(cfg["n"], cfg["par"], cfg["h"], batch=4, rec=cfg["rec_src"], ring_slots=cfg["L"],
+                         resident=False)
+    fwd = sim.run(5, save_state=True)
+    bptt = training.Glif3Bptt(sim, blocked=False)
+    a, step0, _ = bptt._struct(fwd, None, None, False)
+    import ctypes
+    from bmtk_amd import _lib
+    lib = _lib.load()
+    assert lib.bmtk_glif3_step_bwd(ctypes.byref(a), step0, 0, 3, None) != 0          # 1 or 8 partial sums
+    assert "partial sums" in lib.bmtk_amd_last_error().decode()
+    assert lib.bmtk_glif3_step_bwd(ctypes.byref(a), step0, -1, 1, None) != 0
+    a.d_rec_w = None
+    assert lib.bmtk_csr_weight_grad(ctypes.byref(a), step0, 0, None) != 0             # nothing to fill
+    assert "neither" in lib.bmtk_amd_last_error().decode()
