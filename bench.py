@@ -229,6 +229,8 @@ def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rate
             per = dev / steps
             alg = events * B_PER_EVENT
             traffic = profile_traffic("propagation_kernels_52k_batch64.txt", "hbm_bytes_per_launch_%s_%gHz" % (mode, rate))
+            if traffic is not None and mode == "pull2":
+                traffic /= 2                                            # per arrival step, like the time below
             entry = {"kernel": {"auto": "auto_push_kernel or pull_kernel, chosen on the device",
                                 "pull2": "pull2_kernel: the arrivals of two steps per launch, half a launch per step"}
                                .get(mode, mode + "_kernel"),
@@ -317,10 +319,11 @@ def bench_bptt(torch, steps=600):
         "roofline": {"bound": "hbm", "achieved": bwd_step * steps / t_b / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bwd_step * steps / t_b / 1e9 / HBM_PEAK_GBS, "what": "backward pass, HBM-compulsory bytes",
                      "algorithmic_bytes_per_step": bwd_step,
-                     "traffic": profile_traffic("backward_kernels_52k_batch32.txt", "hbm_bytes_per_backward_step")},
+                     "traffic": profile_traffic("training_step_kernels_52k_batch32.txt", "hbm_bytes_per_backward_step")},
         "roofline_forward": {"bound": "hbm", "achieved": fwd_step * steps / t_f / 1e9, "peak": HBM_PEAK_GBS,
                              "unit": "GB/s", "frac": fwd_step * steps / t_f / 1e9 / HBM_PEAK_GBS,
-                             "algorithmic_bytes_per_step": fwd_step}}
+                             "algorithmic_bytes_per_step": fwd_step,
+                             "traffic": profile_traffic("training_step_kernels_52k_batch32.txt", "hbm_bytes_per_forward_step")}}
     # the transposed propagation alone, every row active
     lam = torch.randn(L, 4, ne, device="cuda", generator=g)
     gz = torch.empty(8, ne, device="cuda")
@@ -338,7 +341,7 @@ def bench_bptt(torch, steps=600):
                              "frac": alg / per / 1e9 / HBM_PEAK_GBS,
                              "what": "HBM-compulsory bytes: table + adjoint ring + output once",
                              "algorithmic_bytes_per_launch": alg,
-                             "traffic": profile_traffic("backward_kernels_52k_batch32.txt", traffic_key),
+                             "traffic": profile_traffic("training_step_kernels_52k_batch32.txt", traffic_key),
                              "traffic_note": traffic_note}}
 
     entries = [step_entry]
@@ -619,6 +622,9 @@ def main():
     ap.add_argument("--propagation-modes", default=",".join(PROPAGATION_MODES),
                     help="delivery forms the propagation group times (profiler runs leave out 'auto', which launches "
                          "the scatter and gather kernels too and would be pooled with them)")
+    ap.add_argument("--propagation-rates", default=",".join("%g" % r for r in PROPAGATION_RATES),
+                    help="firing rates (Hz) the propagation group times (profiler runs take one at a time, so that a "
+                         "kernel's launches are not pooled over the rates)")
     ap.add_argument("--only-kernels", action="store_true",
                     help="run only the isolated-kernel measurements of --kernels (for profiler runs); prints a line "
                          "with just their entries")
@@ -646,10 +652,11 @@ def main():
         return
 
     modes = tuple(m for m in args.propagation_modes.split(",") if m)
+    rates = tuple(float(r) for r in args.propagation_rates.split(",") if r)
     if set(modes) - set(PROPAGATION_MODES):
         sys.exit("bench.py: --propagation-modes takes %s" % ", ".join(PROPAGATION_MODES))
     groups = {"state": bench_state_update, "compaction": bench_compaction,
-              "propagation": lambda t: bench_propagation(t, modes=modes), "bptt": bench_bptt,
+              "propagation": lambda t: bench_propagation(t, modes=modes, rates=rates), "bptt": bench_bptt,
               "small": bench_small_network, "batched_v1": bench_batched_v1, "lds": bench_lds}   # (the headline run reports "small" with its front-end entries)
     want = [g for g in args.kernels.split(",") if g]
     unknown = set(want) - set(groups)
