@@ -323,6 +323,11 @@ def bench_bptt(torch, steps=600):
         "roofline_forward": {"bound": "hbm", "achieved": fwd_step * steps / t_f / 1e9, "peak": HBM_PEAK_GBS,
                              "unit": "GB/s", "frac": fwd_step * steps / t_f / 1e9 / HBM_PEAK_GBS,
                              "algorithmic_bytes_per_step": fwd_step,
+                             "what": "the joint table once per step + state in and out + record out (the kernel reads "
+                                     "the table once per TWO steps, so its traffic is below this)",
+                             "frac_by_update_and_event_bytes":
+                                 (ne * B_PER_UPDATE_PLAIN + (events / steps + in_ev.numel() / (2 * steps) * (nnz_in / n_in)) * B_PER_EVENT)
+                                 * steps / t_f / 1e9 / HBM_PEAK_GBS,
                              "traffic": profile_traffic("training_step_kernels_52k_batch32.txt", "hbm_bytes_per_forward_step")}}
     # the transposed propagation alone, every row active
     lam = torch.randn(L, 4, ne, device="cuda", generator=g)
