@@ -157,3 +157,10 @@ def test_pull_equals_gather_at_in_degree_1000_batch_64():
     ops.csr_propagate_pull(hist, n, t_tgt, syn, n, batch, L)
     assert float(ring[0].abs().max()) > 10.0
     assert torch.equal(syn, ring[0])
+    # the two-step pull over the same history: arrivals of step L == the above, of step L-1 == the one-step pull's
+    before = torch.empty_like(syn)
+    ops.csr_propagate_pull(hist, n, t_tgt, before, n, batch, L - 1)
+    both = torch.full((2, 4, ne), -1.0, device="cuda")
+    ops.csr_propagate_pull2(hist, n, t_tgt, both, n, batch, L)
+    assert torch.equal(both[1], syn) and torch.equal(both[0], before)
+    assert not torch.equal(before, syn)
