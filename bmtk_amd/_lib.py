@@ -55,12 +55,12 @@ class Glif3Bwd(C.Structure):
         ("lam_V", c_void_p), ("lam_asc", c_void_p), ("lam_y1", c_void_p), ("lam_y2", c_void_p),
         ("lam_ring", c_void_p), ("gz", c_void_p),
         ("d_rec_w", c_void_p), ("d_inp_w", c_void_p),
-        ("blk_count", c_int32), ("reserved0", c_int32), ("blk_indptr", c_void_p), ("blk_packed", c_void_p),
+        ("blk_count", c_int32), ("gz_planes", c_int32), ("blk_indptr", c_void_p), ("blk_packed", c_void_p),
         ("d_blk_w", c_void_p),
     ]
 
 
-ABI_VERSION = 22  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 23  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {

@@ -214,6 +214,7 @@ __global__ __launch_bounds__(kBlock) void bwd_gather4_kernel(bmtk_glif3_bwd a, B
 // what bounds the rows of a sweep: 16 wavefronts x gpw row groups x 64/lp rows.  The eight XCDs each see every
 // row for their own ranges and write a partial sum of their own, gz[x][ne]; the state adjoint adds the eight.
 __device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves);
+__device__ __forceinline__ void bwd_inp_grad2_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves);
 constexpr int kBlkThreads = 1024;
 constexpr int kBlkWaves = kBlkThreads / kWave;
 constexpr int kBlkMaxGroups = 8;  // row groups per wavefront and sweep: one byte of trial masks each in a 64-bit register
@@ -489,6 +490,317 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_gl
     if (do_inp) bwd_inp_grad_waves(a, q, (int)blockIdx.x * kBlkWaves + wave, (int)gridDim.x * kBlkWaves);
 }
 
+// TWO steps, t = q.t and t-1, in one pass over the blocked table (batches above 16: lp >= 8).  gz of step t reads
+// the adjoint slots t+1 .. t+L-1, gz of step t-1 the slots t .. t+L-2, and slot t only depends on what the state
+// adjoint of step t+1 left behind (it is psc0 times the adjoint of y1 BEFORE step t is undone): both sums can be taken
+// before the state adjoint of step t runs.  Per synapse the record, its weight, the trip round the row's lanes, the
+// row's bounds and the loop around them are paid once for two steps; the two adjoint rows (same target and
+// receptor, neighbouring slots) are fetched side by side.  The weight gradient rides along for both steps with ONE
+// read-modify-write per record.  Partial sums: gz[x] for step t, gz[8 + x] for step t-1.  Everything else as in
+// bwd_gather_blocked_kernel, except that a row's two partial sums take 32 bytes of LDS per lane (half as many rows
+// per sweep) and that eight records are worked off as two fours (their sixteen adjoint rows would not fit the
+// registers at once).
+template <bool kGrad, bool kNe24>
+__global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked2_kernel(bmtk_glif3_bwd a, BwdStep q, int lp, int rows_cu,
+                                                                          int sweeps, int gpw, int use_order, int do_inp)
+{
+    extern __shared__ float4 blk_acc[];  // [kBlkWaves][gpw][2][kWave], then the row order (uint16 per place)
+    constexpr int kF = kBlkInFlight, kH = kGrad ? kBlkInFlight / 2 : kBlkInFlight;
+    const int batch = a.batch;
+    const int64_t n = a.n_neurons, ne = n * batch;
+    const int L = a.ring_slots;
+    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    const int x = blockIdx.x & 7;
+    const int P = a.blk_count >> 3;
+    const int per = kWave / lp;
+    const int grp = lane / lp, b4 = (lane - grp * lp) * 4;
+    const bool lane_on = b4 < batch;
+    const unsigned long long grp_lanes = (lp == kWave ? ~0ull : ((1ull << lp) - 1ull)) << (grp * lp);
+    const int64_t row_lo = (int64_t)(blockIdx.x >> 3) * rows_cu;
+    const int64_t row_hi = row_lo + rows_cu < n ? row_lo + rows_cu : n;
+    const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.blk_packed);
+    const char *__restrict__ ring = reinterpret_cast<const char *>(a.lam_ring);
+    const unsigned lane_off = (unsigned)b4 * 4u;
+    const unsigned q_lo = (unsigned)(q.t % L) * 4u, q_wrap = q_lo - 4u * (unsigned)L;
+    const unsigned ne32 = (unsigned)ne, batch32 = (unsigned)batch;
+    // from a synapse's cell for step t to its cell for step t-1: one slot down, or L-1 slots up from slot 0 (bytes)
+    const unsigned slot_down = 0u - 16u * ne32, slot_up = 16u * ne32 * (unsigned)(L - 1);
+    auto cell_offs = [&](unsigned tdr, unsigned &off_t, unsigned &off_p) {
+        const unsigned dq = tdr >> 24;
+        const unsigned plane = min(dq + q_lo, dq + q_wrap);  // (slot of step t + delay) * 4 + receptor
+        const unsigned elem = mad_u24(tdr, batch32, kNe24 ? mul_u24(plane, ne32) : plane * ne32);
+        off_t = (elem << 2) + lane_off;
+        off_p = off_t + (plane < 4u ? slot_up : slot_down);
+    };
+    float4 *acc = blk_acc + (size_t)wave * gpw * 2 * kWave + lane;
+    const uint64_t *__restrict__ bits_t = a.spike_bits + q.row * a.spike_bits_stride;
+    const uint64_t *__restrict__ bits_p = a.spike_bits + (q.row - 1) * a.spike_bits_stride;
+    uint16_t *order = reinterpret_cast<uint16_t *>(blk_acc + (size_t)kBlkWaves * gpw * 2 * kWave);
+    const int places = sweeps * kBlkWaves * gpw * per;
+    if (kGrad && use_order) {  // rows whose source fired in one of the two steps first (see bwd_gather_blocked_kernel)
+        __shared__ unsigned scan_l[2][kBlkWaves];
+        unsigned fm = 0u, n_mine = 0u;
+        for (int i = 0; (int)threadIdx.x + i * kBlkThreads < rows_cu; ++i) {
+            const int64_t j = row_lo + threadIdx.x + i * kBlkThreads;
+            if (j < row_hi && (trial_mask(bits_t, j, batch, 0, batch) | trial_mask(bits_p, j, batch, 0, batch)) != 0ull)
+                fm |= 1u << i;
+            ++n_mine;
+        }
+        const unsigned c1 = (unsigned)__popc(fm), c0 = n_mine - c1;
+        const unsigned in1 = wave_inclusive_scan(c1), in0 = wave_inclusive_scan(c0);
+        if (lane == kWave - 1) {
+            scan_l[0][wave] = in0;
+            scan_l[1][wave] = in1;
+        }
+        __syncthreads();
+        unsigned base0 = 0u, base1 = 0u, total1 = 0u;
+#pragma unroll
+        for (int w = 0; w < kBlkWaves; ++w) {
+            if (w < wave) {
+                base0 += scan_l[0][w];
+                base1 += scan_l[1][w];
+            }
+            total1 += scan_l[1][w];
+        }
+        unsigned at1 = base1 + in1 - c1, at0 = total1 + base0 + in0 - c0;
+        for (unsigned i = 0; i < n_mine; ++i) {
+            const unsigned local = threadIdx.x + i * kBlkThreads;
+            if ((fm >> i) & 1u)
+                order[at1++] = (uint16_t)local;
+            else
+                order[at0++] = (uint16_t)local;
+        }
+        for (int i = rows_cu + (int)threadIdx.x; i < places; i += kBlkThreads) order[i] = 0xFFFFu;
+        __syncthreads();
+    }
+    auto row_of = [&](int sw, int k) -> int64_t {
+        const int place = ((sw * gpw + k) * kBlkWaves + wave) * per + grp;
+        if (kGrad && use_order) {
+            const unsigned local = order[place];
+            return local == 0xFFFFu ? row_hi : row_lo + local;
+        }
+        return place < rows_cu ? row_lo + place : row_hi;
+    };
+    // trials of this lane with a non-zero surrogate derivative in the step of record row `rec_row`
+    auto active_trials = [&](int64_t rec_row, int64_t j) -> unsigned {
+        if (!a.save_flags) return 0xFu;
+        const int64_t e = j * batch + b4;
+        const uint32_t f4 = *reinterpret_cast<const uint32_t *>(a.save_flags + rec_row * ne + e);
+        const float4 v4 = *reinterpret_cast<const float4 *>(a.save_v + rec_row * ne + e);
+        const int64_t col = a.class_id ? (int64_t)a.class_id[j] : j;
+        const float th = a.prop[GLIF3_TH * a.prop_stride + col];
+        const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+        unsigned act = 0u;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (((f4 >> (8 * c)) & BMTK_F_INTEGRATING) && fabsf((v[c] - th) / th) < 1.0f) act |= 1u << c;
+        return act;
+    };
+    for (int sw = 0; sw < sweeps; ++sw) {
+        // per row group one byte in each word: bits 0-3 the lane's trials with a non-zero surrogate derivative in
+        // the step, bits 4-7 those in which the source fired (kGrad); masks_t for step t, masks_p for step t-1
+        unsigned long long masks_t = 0ull, masks_p = 0ull;
+        for (int k = 0; k < gpw; ++k) {
+            const int64_t j = row_of(sw, k);
+            unsigned at = 0u, ap = 0u, mt = 0u, mp = 0u;
+            if (j < row_hi && lane_on) {
+                at = active_trials(q.row, j);
+                ap = active_trials(q.row - 1, j);
+                if (kGrad) {
+                    mt = (unsigned)(trial_mask(bits_t, j, batch, 0, batch) >> b4) & 0xFu;
+                    mp = (unsigned)(trial_mask(bits_p, j, batch, 0, batch) >> b4) & 0xFu;
+                }
+            }
+            masks_t |= (unsigned long long)(at | (mt << 4)) << (8 * k);
+            masks_p |= (unsigned long long)(ap | (mp << 4)) << (8 * k);
+            acc[(2 * k) * kWave] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            acc[(2 * k + 1) * kWave] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+        const unsigned long long masks_any = masks_t | masks_p;
+        auto row_range = [&](int ph, int k, int &p, int &p1) {
+            p = p1 = 0;
+            if (ph >= P) return;
+            const bool want = ((masks_any >> (8 * k)) & 0xFFull) != 0ull;
+            const int64_t j = row_of(sw, k);
+            if ((__ballot(want) & grp_lanes) != 0ull && j < row_hi) {
+                const int32_t *__restrict__ ip = a.blk_indptr + (int64_t)(x * P + ph) * n + j;
+                p = ip[0];
+                p1 = ip[1];
+            }
+        };
+        int p_next, p1_next;
+        row_range(0, 0, p_next, p1_next);
+        for (int ph = 0; ph < P; ++ph) {
+            for (int k = 0; k < gpw; ++k) {
+                int p = p_next;
+                const int p1 = p1_next;
+                row_range(k + 1 < gpw ? ph : ph + 1, k + 1 < gpw ? k + 1 : 0, p_next, p1_next);
+                if (__ballot(p < p1) == 0ull) continue;
+                const unsigned mine_t = (unsigned)(masks_t >> (8 * k + 4)) & 0xFu, mine_p = (unsigned)(masks_p >> (8 * k + 4)) & 0xFu;
+                const int p1_lane = ((masks_any >> (8 * k)) & 0xFFull) != 0ull ? p1 : 0;
+                const bool row_fired = kGrad && (__ballot((mine_t | mine_p) != 0u) & grp_lanes) != 0ull;
+                const int in_row = lane - grp * lp;
+                const int c8 = in_row & 7, first = grp * lp;
+                float4 s_t = make_float4(0.0f, 0.0f, 0.0f, 0.0f), s_p = s_t;
+                struct Shared {
+                    uint2 r[kF / 8];
+                };
+                auto fetch = [&](int ahead) {
+                    Shared f;
+#pragma unroll
+                    for (int i = 0; i < kF / 8; ++i) f.r[i] = rows[p + ahead + 8 * i + c8];
+                    return f;
+                };
+                auto record = [&](const Shared &have, int u) {
+                    return make_uint2((unsigned)__shfl((int)have.r[u / 8].x, first + (u & 7), kWave),
+                                      (unsigned)__shfl((int)have.r[u / 8].y, first + (u & 7), kWave));
+                };
+                Shared cur = fetch(0), nxt = cur;
+                auto work = [&](const Shared &have, Shared &ahead) {
+                    float keep = 0.0f;
+                    const bool grad_now = kGrad && __ballot(row_fired && p < p1) != 0ull;
+#pragma unroll
+                    for (int h = 0; h < kF / kH; ++h) {
+                        float4 vt[kH], vp[kH];
+                        float w[kH];
+#pragma unroll
+                        for (int u = 0; u < kH; ++u) {
+                            const uint2 sy = record(have, h * kH + u);
+                            const bool valid = p + h * kH + u < p1_lane;
+                            // (lanes past their row's end take record 0 with weight 0: one select, then the same
+                            // arithmetic and the same two loads for every lane -- nothing for the compiler to branch on)
+                            unsigned off_t, off_p;
+                            cell_offs(valid ? sy.x : 0u, off_t, off_p);
+                            w[u] = valid ? __uint_as_float(sy.y) : 0.0f;
+                            vt[u] = *reinterpret_cast<const float4 *>(ring + off_t);
+                            vp[u] = *reinterpret_cast<const float4 *>(ring + off_p);
+                        }
+                        if (h == 0) ahead = fetch(kF);
+#pragma unroll
+                        for (int u = 0; u < kH; ++u) {
+                            s_t.x = fmaf(w[u], vt[u].x, s_t.x);
+                            s_t.y = fmaf(w[u], vt[u].y, s_t.y);
+                            s_t.z = fmaf(w[u], vt[u].z, s_t.z);
+                            s_t.w = fmaf(w[u], vt[u].w, s_t.w);
+                            s_p.x = fmaf(w[u], vp[u].x, s_p.x);
+                            s_p.y = fmaf(w[u], vp[u].y, s_p.y);
+                            s_p.z = fmaf(w[u], vp[u].z, s_p.z);
+                            s_p.w = fmaf(w[u], vp[u].w, s_p.w);
+                        }
+                        if (grad_now) {
+                            // gradient of a record: over the row's lanes, the adjoint entries of the trials in which
+                            // the source fired, of step t and of step t-1 (see bwd_gather_blocked_kernel)
+#pragma unroll
+                            for (int u = 0; u < kH; ++u) {
+                                float g = ((mine_t & 1u) ? vt[u].x : 0.0f) + ((mine_t & 2u) ? vt[u].y : 0.0f) +
+                                          ((mine_t & 4u) ? vt[u].z : 0.0f) + ((mine_t & 8u) ? vt[u].w : 0.0f);
+                                g += ((mine_p & 1u) ? vp[u].x : 0.0f) + ((mine_p & 2u) ? vp[u].y : 0.0f) +
+                                     ((mine_p & 4u) ? vp[u].z : 0.0f) + ((mine_p & 8u) ? vp[u].w : 0.0f);
+                                g += dpp_move<0xB1>(g);
+                                g += dpp_move<0x4E>(g);
+                                g += dpp_move<0x141>(g);
+                                if (lp > 8) g += dpp_move<0x140>(g);
+                                keep = in_row == h * kH + u ? g : keep;
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);  // the second four after the first: registers for one four only
+                    }
+                    if (grad_now && row_fired && in_row < kF && p + in_row < p1) a.d_blk_w[p + in_row] += keep;
+                    p = min(p + kF, p1);  // (a lane whose segment has ended stays at its end: BMTK_BLOCKED_PAD)
+                };
+                while (true) {
+                    work(cur, nxt);
+                    if (__ballot(p < p1) == 0ull) break;
+                    work(nxt, cur);
+                    if (__ballot(p < p1) == 0ull) break;
+                }
+                float4 t = acc[(2 * k) * kWave];
+                t.x += s_t.x;
+                t.y += s_t.y;
+                t.z += s_t.z;
+                t.w += s_t.w;
+                acc[(2 * k) * kWave] = t;
+                t = acc[(2 * k + 1) * kWave];
+                t.x += s_p.x;
+                t.y += s_p.y;
+                t.z += s_p.z;
+                t.w += s_p.w;
+                acc[(2 * k + 1) * kWave] = t;
+            }
+        }
+        for (int k = 0; k < gpw; ++k) {
+            const int64_t j = row_of(sw, k);
+            if (j < row_hi && lane_on) {
+                const unsigned at = (unsigned)(masks_t >> (8 * k)) & 0xFu, ap = (unsigned)(masks_p >> (8 * k)) & 0xFu;
+                float4 t = acc[(2 * k) * kWave];
+                *reinterpret_cast<float4 *>(a.gz + (int64_t)x * ne + j * batch + b4) =
+                    make_float4((at & 1u) ? t.x : 0.0f, (at & 2u) ? t.y : 0.0f, (at & 4u) ? t.z : 0.0f, (at & 8u) ? t.w : 0.0f);
+                t = acc[(2 * k + 1) * kWave];
+                *reinterpret_cast<float4 *>(a.gz + (int64_t)(8 + x) * ne + j * batch + b4) =
+                    make_float4((ap & 1u) ? t.x : 0.0f, (ap & 2u) ? t.y : 0.0f, (ap & 4u) ? t.z : 0.0f, (ap & 8u) ? t.w : 0.0f);
+            }
+        }
+    }
+    // the input-weight gradients of both steps, in the kernel's tail
+    if (do_inp) bwd_inp_grad2_waves(a, q, (int)blockIdx.x * kBlkWaves + wave, (int)gridDim.x * kBlkWaves);
+}
+
+// One step of the state adjoint on registers: the adjoint of the state after the step comes in, that of the state
+// before it goes out.  sg = surrogate derivative times the adjoint of the step's spike (only read where the
+// element was integrating).
+__device__ __forceinline__ void state_adjoint_step(float &lV, float (&lA)[GLIF3_NASC], float (&l1)[GLIF3_NREC],
+                                                   float (&l2)[GLIF3_NREC], const Glif3Prop &p, float h, uint8_t f, float sg)
+{
+    // y1' = P11*y1 + psc0*s ; y2' = P21*y1 + P11*y2
+    float n1[GLIF3_NREC], n2[GLIF3_NREC];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) {
+        n1[k] = p.P11[k] * l1[k] + (h * p.P11[k]) * l2[k];
+        n2[k] = p.P11[k] * l2[k];
+    }
+    float nV, nA[GLIF3_NASC];
+    if (f & BMTK_F_INTEGRATING) {
+        const float lU = lV + sg;
+        nV = p.P33 * lU;
+        const float lS = p.P30 * lU;
+#pragma unroll
+        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = p.c[k] * lS + p.d[k] * lA[k];
+#pragma unroll
+        for (int k = 0; k < GLIF3_NREC; ++k) {
+            n1[k] += p.P31[k] * lU;
+            n2[k] += p.P32[k] * lU;
+        }
+    } else if (f & BMTK_F_RESET) {
+        nV = 0.0f;
+#pragma unroll
+        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = p.r[k] * lA[k];
+    } else {
+        nV = lV;
+#pragma unroll
+        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = lA[k];
+    }
+    lV = nV;
+#pragma unroll
+    for (int k = 0; k < GLIF3_NASC; ++k) lA[k] = nA[k];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) {
+        l1[k] = n1[k];
+        l2[k] = n2[k];
+    }
+}
+
+// surrogate derivative times the adjoint of the spike of element e in the step of record row `row`: what comes back
+// through the synapses (`parts` partial sums from plane `first` of gz on) plus the loss derivative
+__device__ __forceinline__ float spike_adjoint(const bmtk_glif3_bwd &a, const Glif3Prop &p, int64_t row, int64_t e, int64_t ne,
+                                               int first, int parts)
+{
+    float g = a.gz[(int64_t)first * ne + e];
+    for (int x = 1; x < parts; ++x) g += a.gz[(int64_t)(first + x) * ne + e];
+    if (a.dl_dz) g += a.dl_dz[row * ne + e];
+    if (a.dl_dz_const) g += a.dl_dz_const[e];
+    return surrogate(a.save_v[row * ne + e], p.th, a.dampening) * g;
+}
+
 // state adjoint of one step, one thread per element; writes the adjoint of
 // this step's arrivals into ring slot t
 __device__ __forceinline__ void bwd_state_block(const bmtk_glif3_bwd &a, const BwdStep &q, int64_t block)
@@ -510,48 +822,81 @@ __device__ __forceinline__ void bwd_state_block(const bmtk_glif3_bwd &a, const B
         l1[k] = a.lam_y1[k * ne + e];
         l2[k] = a.lam_y2[k * ne + e];
     }
-    // y1' = P11*y1 + psc0*s ; y2' = P21*y1 + P11*y2
     float *slot = a.lam_ring + (int64_t)(q.t % a.ring_slots) * GLIF3_NREC * ne + e;
-    float n1[GLIF3_NREC], n2[GLIF3_NREC];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) slot[k * ne] = p.psc0[k] * l1[k];
+    const float sg = (f & BMTK_F_INTEGRATING) ? spike_adjoint(a, p, q.row, e, ne, 0, q.parts) : 0.0f;
+    state_adjoint_step(lV, lA, l1, l2, p, a.h, f, sg);
+    a.lam_V[e] = lV;
+#pragma unroll
+    for (int k = 0; k < GLIF3_NASC; ++k) a.lam_asc[k * ne + e] = lA[k];
 #pragma unroll
     for (int k = 0; k < GLIF3_NREC; ++k) {
-        slot[k * ne] = p.psc0[k] * l1[k];
-        n1[k] = p.P11[k] * l1[k] + (a.h * p.P11[k]) * l2[k];
-        n2[k] = p.P11[k] * l2[k];
+        a.lam_y1[k * ne + e] = l1[k];
+        a.lam_y2[k * ne + e] = l2[k];
     }
-    float nV, nA[GLIF3_NASC];
-    if (f & BMTK_F_INTEGRATING) {
-        float g = a.gz[e];
-        for (int x = 1; x < q.parts; ++x) g += a.gz[(int64_t)x * ne + e];
-        if (a.dl_dz) g += a.dl_dz[q.row * ne + e];
-        if (a.dl_dz_const) g += a.dl_dz_const[e];
-        const float lU = lV + surrogate(a.save_v[q.row * ne + e], p.th, a.dampening) * g;
-        nV = p.P33 * lU;
-        const float lS = p.P30 * lU;
+}
+
+// The state adjoints of steps t = q.t and t-1 in one launch, the adjoint state in registers in between: the partial
+// sums of step t are planes 0-7 of gz, those of step t-1 planes 8-15 (bwd_gather_blocked2_kernel).  Ring slots
+// follow the rule of that kernel: slot s holds psc0 times the adjoint of y1 before step s is undone, so this launch
+// writes slot t-1 between its two steps and, with write_after, slot t-2 from what it leaves (for the pair of steps
+// that follows); slot t was written by the launch before, or by bwd_seed_slot_kernel at the start of a call.
+__global__ __launch_bounds__(kBlock) void bwd_state2_kernel(bmtk_glif3_bwd a, BwdStep q, int write_after)
+{
+    const int64_t ne = a.n_neurons * (int64_t)a.batch;
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= ne) return;
+    const int64_t n = a.batch == 1 ? e : (int64_t)((uint32_t)e / (uint32_t)a.batch);
+    const int64_t col = a.class_id ? (int64_t)a.class_id[n] : n;
+    Glif3Prop p;
+    p.load(a.prop, a.prop_stride, col);
+    const int L = a.ring_slots;
+    float lV = a.lam_V[e];
+    float lA[GLIF3_NASC], l1[GLIF3_NREC], l2[GLIF3_NREC];
 #pragma unroll
-        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = p.c[k] * lS + p.d[k] * lA[k];
-#pragma unroll
-        for (int k = 0; k < GLIF3_NREC; ++k) {
-            n1[k] += p.P31[k] * lU;
-            n2[k] += p.P32[k] * lU;
-        }
-    } else if (f & BMTK_F_RESET) {
-        nV = 0.0f;
-#pragma unroll
-        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = p.r[k] * lA[k];
-    } else {
-        nV = lV;
-#pragma unroll
-        for (int k = 0; k < GLIF3_NASC; ++k) nA[k] = lA[k];
-    }
-    a.lam_V[e] = nV;
-#pragma unroll
-    for (int k = 0; k < GLIF3_NASC; ++k) a.lam_asc[k * ne + e] = nA[k];
+    for (int k = 0; k < GLIF3_NASC; ++k) lA[k] = a.lam_asc[k * ne + e];
 #pragma unroll
     for (int k = 0; k < GLIF3_NREC; ++k) {
-        a.lam_y1[k * ne + e] = n1[k];
-        a.lam_y2[k * ne + e] = n2[k];
+        l1[k] = a.lam_y1[k * ne + e];
+        l2[k] = a.lam_y2[k * ne + e];
     }
+    const uint8_t f_t = a.save_flags[q.row * ne + e], f_p = a.save_flags[(q.row - 1) * ne + e];
+    const float sg_t = (f_t & BMTK_F_INTEGRATING) ? spike_adjoint(a, p, q.row, e, ne, 0, 8) : 0.0f;
+    const float sg_p = (f_p & BMTK_F_INTEGRATING) ? spike_adjoint(a, p, q.row - 1, e, ne, 8, 8) : 0.0f;
+    state_adjoint_step(lV, lA, l1, l2, p, a.h, f_t, sg_t);
+    float *slot = a.lam_ring + (int64_t)((q.t - 1) % L) * GLIF3_NREC * ne + e;
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) slot[k * ne] = p.psc0[k] * l1[k];
+    state_adjoint_step(lV, lA, l1, l2, p, a.h, f_p, sg_p);
+    if (write_after) {
+        slot = a.lam_ring + (int64_t)((q.t + L - 2) % L) * GLIF3_NREC * ne + e;
+#pragma unroll
+        for (int k = 0; k < GLIF3_NREC; ++k) slot[k * ne] = p.psc0[k] * l1[k];
+    }
+    a.lam_V[e] = lV;
+#pragma unroll
+    for (int k = 0; k < GLIF3_NASC; ++k) a.lam_asc[k * ne + e] = lA[k];
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k) {
+        a.lam_y1[k * ne + e] = l1[k];
+        a.lam_y2[k * ne + e] = l2[k];
+    }
+}
+
+// ring slot `slot` = psc0 times the present adjoint of y1: what the state adjoint of the step the slot belongs to
+// would write first, done ahead for the two-step form, whose transposed propagation reads it before that
+__global__ __launch_bounds__(kBlock) void bwd_seed_slot_kernel(bmtk_glif3_bwd a, int slot)
+{
+    const int64_t ne = a.n_neurons * (int64_t)a.batch;
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= ne) return;
+    const int64_t n = a.batch == 1 ? e : (int64_t)((uint32_t)e / (uint32_t)a.batch);
+    const int64_t col = a.class_id ? (int64_t)a.class_id[n] : n;
+#pragma unroll
+    for (int k = 0; k < GLIF3_NREC; ++k)
+        a.lam_ring[((int64_t)slot * GLIF3_NREC + k) * ne + e] =
+            a.prop[(GLIF3_PSC0_0 + k) * a.prop_stride + col] * a.lam_y1[k * ne + e];
 }
 
 // d_rec_w[p] += sum over trials b in which source j spiked in step t of
@@ -603,52 +948,115 @@ __device__ __forceinline__ void bwd_inp_grad_block(const bmtk_glif3_bwd &a, cons
 {
     bwd_inp_grad_waves(a, q, block * (kBlock / kWave) + threadIdx.x / kWave, n_blocks * (kBlock / kWave));
 }
-__device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves)
+// source of an input event
+__device__ __forceinline__ int event_source(int ev, int batch)
+{
+    return batch == 1 ? ev : (int)((uint32_t)ev / (uint32_t)batch);
+}
+
+// d_inp_w of source j's row += the adjoint cells of the trials of two runs of events: [k, k_end) of a step whose
+// adjoint slots start at slot0, and [m, m_end) of the step before it (slots start one lower); either may be empty
+__device__ __forceinline__ void inp_grad_row(const bmtk_glif3_bwd &a, int j, int slot0, int64_t k, int64_t k_end,
+                                             int slot0_before, int64_t m, int64_t m_end)
 {
     const int batch = a.batch;
     const int64_t ne = a.n_neurons * (int64_t)batch;
     const int L = a.ring_slots;
-    const int slot0 = (int)(q.t % L);
-    const int64_t k0 = a.in_ptr[q.t], k1 = a.in_ptr[q.t + 1];
     const uint2 *__restrict__ rows = reinterpret_cast<const uint2 *>(a.inp_packed);
-    for (int64_t k = k0 + wave; k < k1; k += n_waves) {
-        const int ev = a.in_events[k];
-        const int j = batch == 1 ? ev : (int)((uint32_t)ev / (uint32_t)batch);
-        if (k > k0 && (batch == 1 ? a.in_events[k - 1] : (int)((uint32_t)a.in_events[k - 1] / (uint32_t)batch)) == j)
-            continue;  // not the first event of its source's run
-        int64_t k_end = k + 1;
-        while (k_end < k1 && (batch == 1 ? a.in_events[k_end] : (int)((uint32_t)a.in_events[k_end] / (uint32_t)batch)) == j)
-            ++k_end;
-        const int p0 = a.inp_indptr[j], p1 = a.inp_indptr[j + 1];
-        // four synapses per lane at a time: their records, then their adjoint cells, travel together
-        constexpr int kUnroll = 4;
-        for (int base = p0 + lane_id(); base < p1; base += kUnroll * kWave) {
-            uint2 sy[kUnroll];
-            float old[kUnroll], acc[kUnroll];
+    const int p0 = a.inp_indptr[j], p1 = a.inp_indptr[j + 1];
+    // four synapses per lane at a time: their records, then their adjoint cells, travel together
+    constexpr int kUnroll = 4;
+    for (int base = p0 + lane_id(); base < p1; base += kUnroll * kWave) {
+        uint2 sy[kUnroll];
+        float old[kUnroll], acc[kUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int p = base + u * kWave;
-                if (p < p1) {
-                    sy[u] = rows[p];
-                    old[u] = a.d_inp_w[p];
-                }
+        for (int u = 0; u < kUnroll; ++u) {
+            const int p = base + u * kWave;
+            if (p < p1) {
+                sy[u] = rows[p];
+                old[u] = a.d_inp_w[p];
             }
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                acc[u] = 0.0f;
-                if (base + u * kWave < p1) {
-                    int slot = slot0 + (int)(sy[u].x >> 26);
-                    slot = slot >= L ? slot - L : slot;
-                    const int r = (sy[u].x >> 24) & 3;
-                    const int64_t i = sy[u].x & 0xFFFFFFu;
-                    const float *cell = a.lam_ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch;
-                    for (int64_t kk = k; kk < k_end; ++kk) acc[u] += cell[a.in_events[kk] - j * batch];
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
-                if (base + u * kWave < p1) a.d_inp_w[base + u * kWave] = old[u] + acc[u];
         }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            acc[u] = 0.0f;
+            if (base + u * kWave < p1) {
+                const int d = (int)(sy[u].x >> 26), r = (sy[u].x >> 24) & 3;
+                const int64_t i = sy[u].x & 0xFFFFFFu;
+                int slot = slot0 + d;
+                slot = slot >= L ? slot - L : slot;
+                const float *cell = a.lam_ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch;
+                for (int64_t kk = k; kk < k_end; ++kk) acc[u] += cell[a.in_events[kk] - j * batch];
+                if (m < m_end) {
+                    slot = slot0_before + d;
+                    slot = slot >= L ? slot - L : slot;
+                    cell = a.lam_ring + (int64_t)(slot * GLIF3_NREC + r) * ne + i * batch;
+                    for (int64_t kk = m; kk < m_end; ++kk) acc[u] += cell[a.in_events[kk] - j * batch];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            if (base + u * kWave < p1) a.d_inp_w[base + u * kWave] = old[u] + acc[u];
+    }
+}
+
+__device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves)
+{
+    const int batch = a.batch;
+    const int slot0 = (int)(q.t % a.ring_slots);
+    const int64_t k0 = a.in_ptr[q.t], k1 = a.in_ptr[q.t + 1];
+    for (int64_t k = k0 + wave; k < k1; k += n_waves) {
+        const int j = event_source(a.in_events[k], batch);
+        if (k > k0 && event_source(a.in_events[k - 1], batch) == j) continue;  // not the first event of its source's run
+        int64_t k_end = k + 1;
+        while (k_end < k1 && event_source(a.in_events[k_end], batch) == j) ++k_end;
+        inp_grad_row(a, j, slot0, k, k_end, 0, 0, 0);
+    }
+}
+
+// first event of [lo, hi) (ascending in source*batch+trial) whose source is at least j
+__device__ __forceinline__ int64_t first_event_of(const int32_t *__restrict__ events, int64_t lo, int64_t hi, int j, int batch)
+{
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (event_source(events[mid], batch) < j)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+// The same for steps t = q.t and t-1 in ONE launch.  Two wavefronts must never update one source's row at a time, so
+// a source with events in both steps belongs to the wavefront that holds the first event of its run in step t,
+// which looks its run of step t-1 up (the events of a step are sorted) and adds both with one read-modify-write;
+// runs of step t-1 whose source has no event in step t are taken by the holder of their first event.
+__device__ __forceinline__ void bwd_inp_grad2_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves)
+{
+    const int batch = a.batch;
+    const int L = a.ring_slots;
+    const int slot_t = (int)(q.t % L), slot_p = (int)((q.t - 1) % L);
+    const int64_t k0 = a.in_ptr[q.t], k1 = a.in_ptr[q.t + 1];
+    const int64_t m0 = a.in_ptr[q.t - 1], m1 = k0;  // (in_ptr[t-1] .. in_ptr[t]: the events of step t-1)
+    for (int64_t k = k0 + wave; k < k1; k += n_waves) {
+        const int j = event_source(a.in_events[k], batch);
+        if (k > k0 && event_source(a.in_events[k - 1], batch) == j) continue;
+        int64_t k_end = k + 1;
+        while (k_end < k1 && event_source(a.in_events[k_end], batch) == j) ++k_end;
+        const int64_t m = first_event_of(a.in_events, m0, m1, j, batch);
+        int64_t m_end = m;
+        while (m_end < m1 && event_source(a.in_events[m_end], batch) == j) ++m_end;
+        inp_grad_row(a, j, slot_t, k, k_end, slot_p, m, m_end);
+    }
+    for (int64_t m = m0 + wave; m < m1; m += n_waves) {
+        const int j = event_source(a.in_events[m], batch);
+        if (m > m0 && event_source(a.in_events[m - 1], batch) == j) continue;
+        const int64_t k = first_event_of(a.in_events, k0, k1, j, batch);
+        if (k < k1 && event_source(a.in_events[k], batch) == j) continue;  // the source's run of step t takes it along
+        int64_t m_end = m + 1;
+        while (m_end < m1 && event_source(a.in_events[m_end], batch) == j) ++m_end;
+        inp_grad_row(a, j, slot_p, m, m_end, 0, 0, 0);
     }
 }
 
@@ -706,6 +1114,9 @@ struct BlockedPlan {
     unsigned grid;
     int lp, rows_cu, sweeps, gpw, use_order;
     size_t lds;
+    // the two-step kernel: twice the LDS per row, hence half as many row groups per wavefront and sweep
+    int sweeps2, gpw2, use_order2;
+    size_t lds2;
 };
 constexpr size_t kBlkLdsMax = 160u * 1024u - 256u;  // a compute unit's LDS less the kernel's static part
 
@@ -737,6 +1148,13 @@ int blocked_plan(const bmtk_glif3_bwd &a, BlockedPlan &pl)
     const size_t order_bytes = (size_t)pl.sweeps * kBlkWaves * pl.gpw * per * sizeof(uint16_t);
     pl.use_order = (pl.lds + order_bytes <= kBlkLdsMax && rows_cu <= 16 * kBlkThreads && rows_cu < 0xFFFF) ? 1 : 0;
     if (pl.use_order) pl.lds += order_bytes;
+    const int64_t cap2 = (int64_t)kBlkWaves * (kBlkMaxGroups / 2) * per;
+    pl.sweeps2 = (int)((rows_cu + cap2 - 1) / cap2);
+    pl.gpw2 = (int)((rows_cu + (int64_t)pl.sweeps2 * kBlkWaves * per - 1) / ((int64_t)pl.sweeps2 * kBlkWaves * per));
+    pl.lds2 = (size_t)kBlkWaves * pl.gpw2 * 2 * kWave * sizeof(float4);
+    const size_t order_bytes2 = (size_t)pl.sweeps2 * kBlkWaves * pl.gpw2 * per * sizeof(uint16_t);
+    pl.use_order2 = (pl.lds2 + order_bytes2 <= kBlkLdsMax && rows_cu <= 16 * kBlkThreads && rows_cu < 0xFFFF) ? 1 : 0;
+    if (pl.use_order2) pl.lds2 += order_bytes2;
     static bool asked[8][64];
     const void *variants[8];
     for (int g = 0; g < 8; ++g) variants[g] = blocked_variant(g & 4, g & 2, g & 1);
@@ -749,6 +1167,21 @@ int blocked_plan(const bmtk_glif3_bwd &a, BlockedPlan &pl)
             return BMTK_E_LAUNCH;
         }
         asked[g][dev] = true;
+    }
+    static bool asked2[64];
+    if (dev >= 0 && dev < 64 && !asked2[dev]) {
+        const void *pair[4] = {reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<true, true>),
+                               reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<true, false>),
+                               reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<false, true>),
+                               reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<false, false>)};
+        for (int g = 0; g < 4; ++g) {
+            const hipError_t err = hipFuncSetAttribute(pair[g], hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlkLdsMax);
+            if (err != hipSuccess) {
+                set_error("transposed propagation: cannot reserve LDS: %s", hipGetErrorString(err));
+                return BMTK_E_LAUNCH;
+            }
+        }
+        asked2[dev] = true;
     }
     return BMTK_OK;
 }
@@ -778,6 +1211,27 @@ int blocked_launch(const bmtk_glif3_bwd &a, const BwdStep &q, const BlockedPlan 
                                            params, pl.lds, st);
     if (err != hipSuccess) {
         set_error("transposed propagation: launch failed: %s", hipGetErrorString(err));
+        return BMTK_E_LAUNCH;
+    }
+    return BMTK_OK;
+}
+
+// the two-step kernel for steps q.t and q.t - 1
+int blocked2_launch(const bmtk_glif3_bwd &a, const BwdStep &q, const BlockedPlan &pl, bool grad, bool inp_grad, hipStream_t st)
+{
+    const bool ne24 = a.n_neurons * (int64_t)a.batch < (1ll << 24);
+    bmtk_glif3_bwd args = a;
+    BwdStep step = q;
+    int lp = pl.lp, rows_cu = pl.rows_cu, sweeps = pl.sweeps2, gpw = pl.gpw2, use_order = pl.use_order2;
+    int do_inp = inp_grad ? 1 : 0;
+    void *params[] = {&args, &step, &lp, &rows_cu, &sweeps, &gpw, &use_order, &do_inp};
+    const void *fn = grad ? (ne24 ? reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<true, true>)
+                                  : reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<true, false>))
+                          : (ne24 ? reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<false, true>)
+                                  : reinterpret_cast<const void *>(bwd_gather_blocked2_kernel<false, false>));
+    const hipError_t err = hipLaunchKernel(fn, dim3(pl.grid), dim3(kBlkThreads), params, pl.lds2, st);
+    if (err != hipSuccess) {
+        set_error("transposed propagation (two steps): launch failed: %s", hipGetErrorString(err));
         return BMTK_E_LAUNCH;
     }
     return BMTK_OK;
@@ -839,7 +1293,20 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
     const unsigned elem_grid = (unsigned)((ne + kBlock - 1) / kBlock);
     int bp = 1;  // trial-tile width: the batch rounded up to a power of two, at most one wavefront
     while (bp < a.batch && bp < kWave) bp <<= 1;
-    for (int64_t k = n_steps - 1; k >= 0; --k) {
+    int64_t k_top = n_steps - 1;
+    // Two steps per pass over the blocked table where gz has room for both steps' partial sums and a lane holds
+    // whole adjoint rows of eight lanes (batches above 16): pairs (k, k-1) from the top, a step left over at the
+    // end goes the one-step way.
+    if (blocked && a.gz_planes >= 16 && pl.lp >= 8 && n_steps >= 2) {
+        hipLaunchKernelGGL(bwd_seed_slot_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, (int)((step0 + k_top) % a.ring_slots));
+        for (; k_top >= 1; k_top -= 2) {
+            BwdStep q{step0 + k_top, k_top, 8};
+            const int rc = blocked2_launch(a, q, pl, a.d_blk_w != nullptr, inp_grad, st);
+            if (rc != BMTK_OK) return rc;
+            hipLaunchKernelGGL(bwd_state2_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q, k_top - 1 > 0 ? 1 : 0);
+        }
+    }
+    for (int64_t k = k_top; k >= 0; --k) {
         BwdStep q{step0 + k, k, blocked ? 8 : 1};
         // The recurrent weight gradient of step t reads the adjoint slots t+1 .. t+L-1, which the state adjoint of
         // this step (it writes slot t) leaves alone: it can ride along with the transposed propagation, which

@@ -50,10 +50,11 @@ class Glif3Bptt:
     # adjoint rings above this size use the table regrouped by target range (the ring no longer fits the L2s)
     BLOCKED_MIN_RING_BYTES = 32 << 20
 
-    def __init__(self, sim, dampening=0.3, blocked=None, n_blocks=None):
+    def __init__(self, sim, dampening=0.3, blocked=None, n_blocks=None, two_steps=True):
         """``blocked``: use the recurrent table regrouped by target range for the transposed propagation (None:
         when the adjoint ring exceeds ``BLOCKED_MIN_RING_BYTES`` and the batch allows it); ``n_blocks``: number of
-        target ranges, a multiple of 8 (None: ``ops.blocked_table_blocks``)."""
+        target ranges, a multiple of 8 (None: ``ops.blocked_table_blocks``); ``two_steps``: let the blocked form take
+        two steps per pass over its table (batches above 16; ``gz`` then holds the partial sums of both)."""
         if sim.res_span or sim.delay_offset:
             raise ValueError("the backward pass needs a simulator built with resident=False and delay_offset 0")
         self.sim, self.dampening = sim, float(dampening)
@@ -78,7 +79,9 @@ class Glif3Bptt:
                 raise ValueError("n_blocks must be a multiple of 8")
             self.blk = sim.rec.blocked(sim.n, self.n_blocks)
             self.d_blk_w = torch.zeros(sim.rec.nnz, device=dev)
-        self.gz = torch.zeros(8 * ne if blocked else ne, device=dev)
+        # the blocked form takes two steps per pass over its table when gz has room for both steps' partial sums
+        self.gz_planes = (16 if two_steps else 8) if blocked else 1
+        self.gz = torch.zeros(self.gz_planes * ne, device=dev)
         self.d_inp_w = torch.zeros(sim.inp.nnz, device=dev) if sim.inp is not None and sim.in_ptr is not None else None
 
     def zero(self):
@@ -102,6 +105,7 @@ class Glif3Bptt:
                 a.d_rec_w = _p(self.d_rec_w)
             else:
                 a.blk_count, a.blk_indptr, a.blk_packed = self.n_blocks, _p(self.blk[0]), _p(self.blk[1])
+                a.gz_planes = self.gz_planes
                 a.d_blk_w = _p(self.d_blk_w)
         if self.d_inp_w is not None:
             a.in_ptr, a.in_events = _p(sim.in_ptr), _p(sim.in_events)

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 22
+#define BMTK_AMD_ABI_VERSION 23
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -478,7 +478,7 @@ typedef struct bmtk_glif3_bwd {
     /* adjoint state, in/out (zero before the last step of the whole run) */
     float *lam_V, *lam_asc, *lam_y1, *lam_y2; /* [ne], [2][ne], [4][ne], [4][ne] */
     float *lam_ring;               /* [L][4][ne]: adjoint of the arrivals of the steps still ahead */
-    float *gz;                     /* [ne] scratch; [8][ne] when the blocked table is given */
+    float *gz;                     /* [ne] scratch; [8][ne] when the blocked table is given, [16][ne] with gz_planes 16 */
     /* outputs */
     float *d_rec_w;                /* [rec nnz] or NULL */
     float *d_inp_w;                /* [inp nnz] or NULL */
@@ -491,7 +491,9 @@ typedef struct bmtk_glif3_bwd {
      * the records in that order FOLLOWED BY BMTK_BLOCKED_PAD more records of any content (the kernel reads up to
      * that many records past a row's end and ignores them).  Needs a lam_ring below 4 GB. */
     int32_t blk_count;             /* 0 = no blocked table */
-    int32_t reserved0;
+    int32_t gz_planes;             /* planes of n_neurons*batch floats gz holds: 0 = 8.  With 16 or more and a batch above
+                                      16 the blocked form takes TWO steps per pass over its table (a step's eight partial
+                                      sums in planes 0-7, those of the step before it in planes 8-15) */
     const int32_t *blk_indptr;
     const bmtk_synapse *blk_packed;
     float *d_blk_w;                /* [rec nnz] recurrent weight gradient in the order of blk_packed, accumulated,

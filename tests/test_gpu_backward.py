@@ -249,3 +249,35 @@ def test_backward_parts_argument_errors():
     a.d_rec_w = None
     assert lib.bmtk_csr_weight_grad(ctypes.byref(a), step0, 0, None) != 0             # nothing to fill
     assert "neither" in lib.bmtk_amd_last_error().decode()
+
+
+@pytest.mark.parametrize("batch,seed,n_blocks,steps", [(32, 9, 16, 70), (64, 3, 8, 69), (20, 5, 8, 33), (32, 11, 8, 3),
+                                                        (32, 12, 8, 4)])
+def test_two_steps_per_pass_of_the_blocked_form_equal_one(batch, seed, n_blocks, steps):
+    """The blocked transposed propagation taking two steps per pass over its table (``gz_planes`` 16, batches above
+    16) against the same form step by step: every sum is added in the same order, so the adjoint state and the
+    adjoint ring agree BIT FOR BIT after an even and an odd number of steps, in one call and in chunks; the weight
+    gradients add the two steps' contributions in another order (1e-6 of the largest entry)."""
+    cfg = _net(batch, seed, steps=steps)
+    n, T, h = cfg["n"], cfg["steps"], cfg["h"]
+    ne = n * batch
+    sim = Glif3Simulator(n, cfg["par"], h, batch=batch, rec=cfg["rec_src"], inp=cfg["inp_src"], ring_slots=cfg["L"],
+                         resident=False)
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    cut = max(1, T // 3)
+    chunks = [sim.run(cut, save_state=True), sim.run(T - cut, save_state=True)]
+    rng = np.random.default_rng(seed)
+    dl = [torch.as_tensor(rng.normal(size=(c["bits"].shape[0], ne)).astype(np.float32), device="cuda") for c in chunks]
+    one = training.Glif3Bptt(sim, dampening=0.3, blocked=True, n_blocks=n_blocks, two_steps=False)
+    two = training.Glif3Bptt(sim, dampening=0.3, blocked=True, n_blocks=n_blocks, two_steps=True)
+    assert one.gz_planes == 8 and two.gz_planes == 16
+    for b in (one, two):
+        for c, d in zip(reversed(chunks), reversed(dl)):       # chunks in reverse time order
+            b.backward(c, dl_dz=d)
+    for name in ("lam_V", "lam_asc", "lam_y1", "lam_y2", "lam_ring"):
+        assert torch.equal(getattr(one, name), getattr(two, name)), name
+    assert float(one.lam_V.abs().max()) > 0
+    for name in ("d_rec_w", "d_inp_w"):
+        got, want = getattr(two, name), getattr(one, name)
+        assert float(want.abs().max()) > 0 or steps < 30        # (a few steps from rest: nothing has fired yet)
+        assert float((got - want).abs().max()) <= 1e-6 * float(want.abs().max()), name

@@ -164,3 +164,32 @@ def test_pull_equals_gather_at_in_degree_1000_batch_64():
     ops.csr_propagate_pull2(hist, n, t_tgt, both, n, batch, L)
     assert torch.equal(both[1], syn) and torch.equal(both[0], before)
     assert not torch.equal(before, syn)
+
+
+def test_two_steps_per_pass_at_the_training_size_equal_one():
+    """51,978 x batch 32, 24 ranges: five and then four steps of a real forward run differentiated through the
+    two-step form of the blocked kernel (four sweeps of four row groups) and through the one-step form: adjoint
+    state and ring bit for bit, gradients to 1e-6 of the largest."""
+    n, batch, L = N52K, 32, 6
+    rng = np.random.default_rng(6)
+    par = synthetic.random_cells(rng, n)
+    _, by_src, _ = synthetic.device_network(n, 1000, "poisson", seed=2, max_delay=L - 1, w_scale=0.2)
+    inp = synthetic.device_input_table(17400, n, 8_000_000, seed=4, w_scale=2.0)
+    in_ptr, in_ev = ops.poisson_events(17400, 5.0, 1.0, 64, batch=batch, seed=5)
+    sim = Glif3Simulator(n, par, 1.0, batch=batch, rec=by_src, inp=inp, resident=False, ring_slots=L)
+    sim.set_input_events(in_ptr, in_ev)
+    sim.run(40)
+    chunks = [sim.run(4, save_state=True), sim.run(5, save_state=True)]
+    g = torch.Generator(device="cuda").manual_seed(2)
+    dl = torch.randn(n * batch, device="cuda", generator=g) * 1e-3
+    one = training.Glif3Bptt(sim, dampening=0.3, blocked=True, n_blocks=24, two_steps=False)
+    two = training.Glif3Bptt(sim, dampening=0.3, blocked=True, n_blocks=24, two_steps=True)
+    for b in (one, two):
+        for c in reversed(chunks):
+            b.backward(c, dl_dz_const=dl)
+    for name in ("lam_V", "lam_asc", "lam_y1", "lam_y2", "lam_ring"):
+        assert torch.equal(getattr(one, name), getattr(two, name)), name
+    assert float(one.lam_V.abs().max()) > 0 and float(one.d_rec_w.abs().max()) > 0
+    for name in ("d_rec_w", "d_inp_w"):
+        got, want = getattr(two, name), getattr(one, name)
+        assert float((got - want).abs().max()) <= 1e-6 * float(want.abs().max()), name
