@@ -305,9 +305,9 @@ def bench_bptt(torch, steps=600):
     # in and out, the record (potential and flags) out, the neuron's propagator column once per neuron
     fwd_step = (nnz + nnz_in) * 8 + ne * (12 * 8 + 5) + n * 29 * 4
     step_entry = {
-        "kernel": "%s (forward), bwd_gather_blocked_kernel + bwd_state_kernel + bwd_inp_grad_kernel (backward; the "
-                  "recurrent weight gradient rides in bwd_gather_blocked_kernel)" %
-                  ("sim_fused_kernel: pull and update in one launch per step" if sim.fuse_table is not None
+        "kernel": "%s (forward), bwd_gather_blocked2_kernel + bwd_state2_kernel (backward, two steps per launch; both "
+                  "weight gradients ride in the former)" %
+                  ("sim_fused_kernel: pull and update fused, two steps per launch" if sim.fuse_table is not None
                    else "sim_step_kernel + pull_kernel"),
         "blocked_table_ranges": bptt.n_blocks if bptt.blk is not None else 0,
         "workload": "BPTT step N=51978 nnz=%d inputs=17400 batch=32 steps=%d" % (nnz, steps),

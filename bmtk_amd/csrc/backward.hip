@@ -498,14 +498,13 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked_kernel(bmtk_gl
 // receptor, neighbouring slots) are fetched side by side.  The weight gradient rides along for both steps with ONE
 // read-modify-write per record.  Partial sums: gz[x] for step t, gz[8 + x] for step t-1.  Everything else as in
 // bwd_gather_blocked_kernel, except that a row's two partial sums take 32 bytes of LDS per lane (half as many rows
-// per sweep) and that eight records are worked off as two fours (their sixteen adjoint rows would not fit the
-// registers at once).
+// per sweep).
 template <bool kGrad, bool kNe24>
 __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked2_kernel(bmtk_glif3_bwd a, BwdStep q, int lp, int rows_cu,
                                                                           int sweeps, int gpw, int use_order, int do_inp)
 {
     extern __shared__ float4 blk_acc[];  // [kBlkWaves][gpw][2][kWave], then the row order (uint16 per place)
-    constexpr int kF = kBlkInFlight, kH = kGrad ? kBlkInFlight / 2 : kBlkInFlight;
+    constexpr int kF = kBlkInFlight;
     const int batch = a.batch;
     const int64_t n = a.n_neurons, ne = n * batch;
     const int L = a.ring_slots;
@@ -659,51 +658,48 @@ __global__ __launch_bounds__(kBlkThreads) void bwd_gather_blocked2_kernel(bmtk_g
                 auto work = [&](const Shared &have, Shared &ahead) {
                     float keep = 0.0f;
                     const bool grad_now = kGrad && __ballot(row_fired && p < p1) != 0ull;
+                    float4 vt[kF], vp[kF];
+                    float w[kF];
 #pragma unroll
-                    for (int h = 0; h < kF / kH; ++h) {
-                        float4 vt[kH], vp[kH];
-                        float w[kH];
+                    for (int u = 0; u < kF; ++u) {
+                        const uint2 sy = record(have, u);
+                        const bool valid = p + u < p1_lane;
+                        // (lanes past their row's end take record 0 with weight 0: one select, then the same
+                        // arithmetic and the same two loads for every lane.  With the select on the address instead,
+                        // the compiler branched around the loads and waited for each of them.)
+                        unsigned off_t, off_p;
+                        cell_offs(valid ? sy.x : 0u, off_t, off_p);
+                        w[u] = valid ? __uint_as_float(sy.y) : 0.0f;
+                        vt[u] = *reinterpret_cast<const float4 *>(ring + off_t);
+                        vp[u] = *reinterpret_cast<const float4 *>(ring + off_p);
+                    }
+                    ahead = fetch(kF);
 #pragma unroll
-                        for (int u = 0; u < kH; ++u) {
-                            const uint2 sy = record(have, h * kH + u);
-                            const bool valid = p + h * kH + u < p1_lane;
-                            // (lanes past their row's end take record 0 with weight 0: one select, then the same
-                            // arithmetic and the same two loads for every lane -- nothing for the compiler to branch on)
-                            unsigned off_t, off_p;
-                            cell_offs(valid ? sy.x : 0u, off_t, off_p);
-                            w[u] = valid ? __uint_as_float(sy.y) : 0.0f;
-                            vt[u] = *reinterpret_cast<const float4 *>(ring + off_t);
-                            vp[u] = *reinterpret_cast<const float4 *>(ring + off_p);
+                    for (int u = 0; u < kF; ++u) {
+                        s_t.x = fmaf(w[u], vt[u].x, s_t.x);
+                        s_t.y = fmaf(w[u], vt[u].y, s_t.y);
+                        s_t.z = fmaf(w[u], vt[u].z, s_t.z);
+                        s_t.w = fmaf(w[u], vt[u].w, s_t.w);
+                        s_p.x = fmaf(w[u], vp[u].x, s_p.x);
+                        s_p.y = fmaf(w[u], vp[u].y, s_p.y);
+                        s_p.z = fmaf(w[u], vp[u].z, s_p.z);
+                        s_p.w = fmaf(w[u], vp[u].w, s_p.w);
+                    }
+                    if (grad_now) {
+                        // gradient of a record: over the row's lanes, the adjoint entries of the trials in which the
+                        // source fired, of step t and of step t-1 (see bwd_gather_blocked_kernel)
+#pragma unroll
+                        for (int u = 0; u < kF; ++u) {
+                            float g = ((mine_t & 1u) ? vt[u].x : 0.0f) + ((mine_t & 2u) ? vt[u].y : 0.0f) +
+                                      ((mine_t & 4u) ? vt[u].z : 0.0f) + ((mine_t & 8u) ? vt[u].w : 0.0f);
+                            g += ((mine_p & 1u) ? vp[u].x : 0.0f) + ((mine_p & 2u) ? vp[u].y : 0.0f) +
+                                 ((mine_p & 4u) ? vp[u].z : 0.0f) + ((mine_p & 8u) ? vp[u].w : 0.0f);
+                            g += dpp_move<0xB1>(g);
+                            g += dpp_move<0x4E>(g);
+                            g += dpp_move<0x141>(g);
+                            if (lp > 8) g += dpp_move<0x140>(g);
+                            keep = in_row == u ? g : keep;
                         }
-                        if (h == 0) ahead = fetch(kF);
-#pragma unroll
-                        for (int u = 0; u < kH; ++u) {
-                            s_t.x = fmaf(w[u], vt[u].x, s_t.x);
-                            s_t.y = fmaf(w[u], vt[u].y, s_t.y);
-                            s_t.z = fmaf(w[u], vt[u].z, s_t.z);
-                            s_t.w = fmaf(w[u], vt[u].w, s_t.w);
-                            s_p.x = fmaf(w[u], vp[u].x, s_p.x);
-                            s_p.y = fmaf(w[u], vp[u].y, s_p.y);
-                            s_p.z = fmaf(w[u], vp[u].z, s_p.z);
-                            s_p.w = fmaf(w[u], vp[u].w, s_p.w);
-                        }
-                        if (grad_now) {
-                            // gradient of a record: over the row's lanes, the adjoint entries of the trials in which
-                            // the source fired, of step t and of step t-1 (see bwd_gather_blocked_kernel)
-#pragma unroll
-                            for (int u = 0; u < kH; ++u) {
-                                float g = ((mine_t & 1u) ? vt[u].x : 0.0f) + ((mine_t & 2u) ? vt[u].y : 0.0f) +
-                                          ((mine_t & 4u) ? vt[u].z : 0.0f) + ((mine_t & 8u) ? vt[u].w : 0.0f);
-                                g += ((mine_p & 1u) ? vp[u].x : 0.0f) + ((mine_p & 2u) ? vp[u].y : 0.0f) +
-                                     ((mine_p & 4u) ? vp[u].z : 0.0f) + ((mine_p & 8u) ? vp[u].w : 0.0f);
-                                g += dpp_move<0xB1>(g);
-                                g += dpp_move<0x4E>(g);
-                                g += dpp_move<0x141>(g);
-                                if (lp > 8) g += dpp_move<0x140>(g);
-                                keep = in_row == h * kH + u ? g : keep;
-                            }
-                        }
-                        __builtin_amdgcn_sched_barrier(0);  // the second four after the first: registers for one four only
                     }
                     if (grad_now && row_fired && in_row < kF && p + in_row < p1) a.d_blk_w[p + in_row] += keep;
                     p = min(p + kF, p1);  // (a lane whose segment has ended stays at its end: BMTK_BLOCKED_PAD)
@@ -1015,17 +1011,25 @@ __device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, cons
     }
 }
 
-// first event of [lo, hi) (ascending in source*batch+trial) whose source is at least j
+// first event of [lo, hi) (ascending in source*batch+trial) whose source is at least j; called by a whole wavefront
+// with the same arguments in every lane: 64 probes a round instead of one, two rounds for a step's few thousand
+// events where a binary search is a chain of twelve dependent loads
 __device__ __forceinline__ int64_t first_event_of(const int32_t *__restrict__ events, int64_t lo, int64_t hi, int j, int batch)
 {
-    while (lo < hi) {
-        const int64_t mid = (lo + hi) >> 1;
-        if (event_source(events[mid], batch) < j)
-            lo = mid + 1;
-        else
-            hi = mid;
+    const int lane = lane_id();
+    while (hi - lo > kWave) {
+        const int64_t stride = (hi - lo + kWave - 1) / kWave;
+        const int64_t at = lo + lane * stride;
+        const bool below = at < hi && event_source(events[at], batch) < j;  // ascending: the lanes below j are a prefix
+        const int c = __popcll(__ballot(below));
+        if (c == 0) return lo;
+        const int64_t upto = lo + c * stride;
+        lo = lo + (c - 1) * stride + 1;
+        hi = upto < hi ? upto : hi;
     }
-    return lo;
+    const int64_t at = lo + lane;
+    const unsigned long long at_least = __ballot(at < hi && event_source(events[at], batch) >= j);
+    return at_least ? lo + (__ffsll((long long)at_least) - 1) : hi;
 }
 
 // The same for steps t = q.t and t-1 in ONE launch.  Two wavefronts must never update one source's row at a time, so
