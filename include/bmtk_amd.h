@@ -500,8 +500,10 @@ typedef struct bmtk_glif3_bwd {
                                       or NULL (then d_rec_w, if given, is filled through rec_indptr / rec_packed) */
 } bmtk_glif3_bwd;
 
-/* Differentiate steps step0+n_steps-1 down to step0 (three launches per step:
- * transposed propagation, state adjoint, weight gradients). */
+/* Differentiate steps step0+n_steps-1 down to step0.  Per step: the transposed propagation (the weight gradients
+ * ride in it where a wavefront holds whole adjoint rows), the state adjoint, and for batches above 64 a launch for
+ * the recurrent weight gradient; with the blocked table, gz_planes >= 16 and a batch above 16, two launches per TWO
+ * steps.  Whatever the form, lam_V .. lam_ring leave as a step-by-step evaluation would leave them. */
 int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0, int64_t n_steps, void *stream);
 
 /* One backward step in its three parts, for callers that put their own work between them (a loss that is computed
