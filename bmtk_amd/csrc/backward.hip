@@ -1307,6 +1307,11 @@ extern "C" int bmtk_glif3_simulate_bwd(const bmtk_glif3_bwd *bwd, int64_t step0,
             BwdStep q{step0 + k_top, k_top, 8};
             const int rc = blocked2_launch(a, q, pl, a.d_blk_w != nullptr, inp_grad, st);
             if (rc != BMTK_OK) return rc;
+            if (a.d_rec_w && !a.d_blk_w) {  // (before the state adjoint, which overwrites a slot step t-1's gradient reads)
+                const BwdStep before{q.t - 1, q.row - 1, 8};
+                hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, q);
+                hipLaunchKernelGGL(bwd_rec_grad_kernel, dim3(rows_grid), dim3(kBlock), 0, st, a, before);
+            }
             hipLaunchKernelGGL(bwd_state2_kernel, dim3(elem_grid), dim3(kBlock), 0, st, a, q, k_top - 1 > 0 ? 1 : 0);
         }
     }

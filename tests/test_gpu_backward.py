@@ -281,3 +281,31 @@ def test_two_steps_per_pass_of_the_blocked_form_equal_one(batch, seed, n_blocks,
         got, want = getattr(two, name), getattr(one, name)
         assert float(want.abs().max()) > 0 or steps < 30        # (a few steps from rest: nothing has fired yet)
         assert float((got - want).abs().max()) <= 1e-6 * float(want.abs().max()), name
+
+
+def test_blocked_form_with_the_gradient_in_source_major_order():
+    """A caller of the C interface may give the blocked table for the transposed propagation and still ask for the
+    recurrent gradient in the order of the source-major table (``d_rec_w`` without ``d_blk_w``): a launch of its
+    own per step, which in the two-step form must come before the state adjoint.  Equal to the gradient that rides
+    along, brought back through the sort permutation (1e-6 of the largest: other order of additions)."""
+    import ctypes
+    from bmtk_amd import _lib
+    cfg = _net(32, 14, steps=41)
+    n, T = cfg["n"], cfg["steps"]
+    sim = Glif3Simulator(n, cfg["par"], cfg["h"], batch=32, rec=cfg["rec_src"], inp=cfg["inp_src"],
+                         ring_slots=cfg["L"], resident=False)
+    sim.set_input_events(cfg["in_ptr"], cfg["in_events"])
+    fwd = sim.run(T, save_state=True)
+    dl = torch.as_tensor(np.random.default_rng(1).normal(size=(T, n * 32)).astype(np.float32), device="cuda")
+    want = training.Glif3Bptt(sim, dampening=0.3, blocked=True, n_blocks=8)
+    want.backward(fwd, dl_dz=dl)
+    assert float(want.d_rec_w.abs().max()) > 0
+    for two_steps in (True, False):
+        b = training.Glif3Bptt(sim, dampening=0.3, blocked=True, n_blocks=8, two_steps=two_steps)
+        a, step0, n_steps = b._struct(fwd, None, dl, True)
+        a.d_blk_w = None
+        a.d_rec_w = b.d_rec_w.data_ptr()
+        _lib.check(_lib.load().bmtk_glif3_simulate_bwd(ctypes.byref(a), step0, n_steps, None))
+        torch.cuda.synchronize()
+        assert float((b.d_rec_w - want.d_rec_w).abs().max()) <= 1e-6 * float(want.d_rec_w.abs().max()), two_steps
+        assert torch.equal(b.lam_V, want.lam_V) and torch.equal(b.lam_ring, want.lam_ring)
