@@ -630,6 +630,9 @@ def main():
     ap.add_argument("--propagation-rates", default=",".join("%g" % r for r in PROPAGATION_RATES),
                     help="firing rates (Hz) the propagation group times (profiler runs take one at a time, so that a "
                          "kernel's launches are not pooled over the rates)")
+    ap.add_argument("--kernels-in-line", action="store_true",
+                    help="put the full isolated-kernel entries into the result line (default: a short kernel_summary "
+                         "in the line, the full entries as a JSON line on stderr)")
     ap.add_argument("--only-kernels", action="store_true",
                     help="run only the isolated-kernel measurements of --kernels (for profiler runs); prints a line "
                          "with just their entries")
@@ -748,7 +751,12 @@ def main():
     if args.cpu_steps > 0:
         line["cpu_baseline"] = cpu_baseline(torch, sim, par, class_id, settled, max(CPU_MIN_STEPS, args.cpu_steps))
     if kernels is not None:
-        line["kernels"] = kernels
+        # The full entries are long (every form and rate): they go to stderr as a JSON line of their own unless asked
+        # for in the result line, which stays short enough to be kept whole by whatever records it.
+        if args.kernels_in_line:
+            line["kernels"] = kernels
+        else:
+            print(json.dumps({"kernels": kernels}), file=sys.stderr, flush=True)
     print(json.dumps(line))
 
 
