@@ -88,8 +88,6 @@ __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__r
     uint2 *stage = reinterpret_cast<uint2 *>(pull_lds + (kPullBlock / kWave) * GLIF3_NREC * kWave) + wave * kWave;
     uint32_t *any_l = reinterpret_cast<uint32_t *>(pull_lds + (kPullBlock / kWave) * (GLIF3_NREC + 1) * kWave);
     const unsigned lane = (unsigned)lane_id();
-    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
-    __syncthreads();
     const int tile0 = kWords64 ? 0 : (int)blockIdx.y * kWave;
     const int width = kWords64 ? kWave : min(kWave, batch - tile0);
     const unsigned hstride = (unsigned)hist_stride;  // L * hist_stride * 8 < 2^32 bytes (checked by the caller)
@@ -116,7 +114,6 @@ __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__r
     // Three table blocks per wavefront: the one at hand and the two after it, whose loads stay in flight during
     // the whole turn (a buffer is refilled, with the block three ahead, as soon as its turn is over).
     PullBlock b0 = cursor.next();
-    if (b0.row >= n_tgt) return;
     unsigned long long d0[kPullChunks] = {0ull, 0ull, 0ull, 0ull}, d1[kPullChunks] = {0ull, 0ull, 0ull, 0ull},
                        d2[kPullChunks] = {0ull, 0ull, 0ull, 0ull};
     fetch(d0, b0);
@@ -124,6 +121,10 @@ __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__r
     fetch(d1, b1);
     PullBlock b2 = cursor.next();
     fetch(d2, b2);
+    // the activity map comes into LDS while the first table blocks are on their way
+    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
+    __syncthreads();
+    if (b0.row >= n_tgt) return;
 #pragma unroll
     for (int r = 0; r < GLIF3_NREC; ++r) acc[r][lane] = 0ull;
     int staged = 0;  // entries in the stage (same in all lanes)
@@ -219,8 +220,6 @@ __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__res
     uint2 *stage = reinterpret_cast<uint2 *>(pull_lds + kWaves * 2 * GLIF3_NREC * kWave) + wave * 2 * kWave;
     uint32_t *any_l = reinterpret_cast<uint32_t *>(pull_lds + kWaves * 2 * (GLIF3_NREC + 1) * kWave);
     const unsigned lane = (unsigned)lane_id();
-    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
-    __syncthreads();
     const int tile0 = kWords64 ? 0 : (int)blockIdx.y * kWave;
     const int width = kWords64 ? kWave : min(kWave, batch - tile0);
     const unsigned hstride = (unsigned)hist_stride;  // L * hist_stride * 8 < 2^32 bytes (checked by the caller)
@@ -239,11 +238,14 @@ __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__res
     PullCursor cursor;
     cursor.start(indptr, n_tgt, (int64_t)blockIdx.x * kWaves + wave, (int64_t)gridDim.x * kWaves);
     PullBlock b0 = cursor.next();
-    if (b0.row >= n_tgt) return;
     unsigned long long d0[kPullChunks] = {0ull, 0ull, 0ull, 0ull}, d1[kPullChunks] = {0ull, 0ull, 0ull, 0ull};
     fetch(d0, b0);
     PullBlock b1 = cursor.next();
     fetch(d1, b1);
+    // the activity map comes into LDS while the first table blocks are on their way
+    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
+    __syncthreads();
+    if (b0.row >= n_tgt) return;
 #pragma unroll
     for (int r = 0; r < 2 * GLIF3_NREC; ++r) acc[r * kWave + lane] = 0ull;
     int staged[2] = {0, 0};  // entries in the two stages (same in all lanes)
