@@ -590,7 +590,10 @@ def kernel_summary(kernels):
         if w.startswith("state update"):
             name = "state_update_class_table" if "class table" in w else "state_update_per_neuron_parameters"
             out[name] = {"us_per_launch": k["us_per_launch"], "neuron_updates_per_s": k["neuron_updates_per_s"],
-                         "frac": r.get("frac"), "traffic": r.get("traffic")}
+                         "frac": r.get("frac"), "traffic": r.get("traffic"),
+                         # measured HBM bytes (profile) / this run's launch time / peak
+                         "hbm_frac": None if not r.get("traffic") else
+                         r["traffic"] / (k["us_per_launch"] * 1e-6) / 1e9 / HBM_PEAK_GBS}
         elif w.startswith("propagation"):
             rate = w.split("rate=")[1]
             out.setdefault("propagation_us_per_arrival_step", {}).setdefault(rate, {})[k["kernel"].split(" ")[0].rstrip(":")] = \
