@@ -463,8 +463,10 @@ class AutoPropagator:
 
     ``hist`` is the caller's spike history, int64 [L, words+1]: before ``step(k, ...)`` row k % L must hold the
     spike bits of step k.  After the call ring slot (k + 1) % L holds everything that arrives in step k + 1; the
-    caller consumes and clears it before the next call.  Default threshold: 2,000 active elements per 52 M synapses
-    of table, the measured break-even on one MI355X."""
+    caller consumes and clears it before the next call.  Default threshold: where pushing costs what a pass costs
+    on one MI355X -- an active element's row goes out at 2e10 events/s, a pass streams the packed table at 5 TB/s
+    after 20 us of launches and set-up -- i.e. 0.032 n_src + 4e5 n_src / nnz active elements (2,000 at 52 k sources
+    with 52 M synapses, where it was measured)."""
 
     def __init__(self, table_src, table_tgt, hist, ring, n_src, n_tgt, batch, scatter_max_active=None):
         self.lib = _lib.load()
@@ -476,7 +478,7 @@ class AutoPropagator:
         self.src, self.tgt, self.hist, self.ring = table_src, table_tgt, hist, ring
         self.L, self.n_src, self.n_tgt, self.batch = L, n_src, n_tgt, batch
         if scatter_max_active is None:
-            scatter_max_active = max(1, int(2000 * table_tgt.nnz / 52e6))
+            scatter_max_active = max(1, int(0.032 * n_src + 4e5 * n_src / max(1, table_tgt.nnz)))
         self.scatter_max_active = int(scatter_max_active)
         need = self.lib.bmtk_csr_propagate_auto_workspace_bytes(L, n_src)
         self.workspace = torch.zeros(need // 4 + 1, dtype=torch.int32, device=ring.device)

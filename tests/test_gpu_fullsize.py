@@ -349,3 +349,38 @@ def test_fused_batched_driver_at_120k_neurons_batch_16():
         got = sim.state.to_numpy()
         for k in ("V", "asc", "y1", "y2", "ref"):
             np.testing.assert_array_equal(got[k], st[k], err_msg="%s shift %d" % (k, shift))
+
+
+def test_device_side_switch_at_52k_neurons_batch_64():
+    """``bmtk_csr_propagate_auto`` at 51,978 x batch 64 (in-degree ~120, quarter-pA weights) over 14 steps whose
+    activity goes 0.2 Hz -> 20 Hz -> 0.2 Hz: with the default threshold the quiet steps are pushed as events (665
+    active elements) and the busy ones pulled (66,000), so that arrival slots hold pushed weights when the pull adds
+    its sums and pulled steps reach into stretches that were pushed.  After every call the arrival slot == the slot
+    the deterministic row-wise gather fills (itself == the fp32 oracle above), bit for bit."""
+    n, batch, L, T = N52K, 64, 6, 14
+    t_tgt, t_src, _ = _network(n, 120, seed=21)
+    ne = n * batch
+    g = torch.Generator(device="cuda").manual_seed(5)
+    rates = [0.2, 0.2, 20.0, 0.2, 20.0, 20.0, 0.2, 0.2, 0.2, 5.0, 0.2, 20.0, 0.2, 0.2]
+    words = ops.n_words(ne)
+    hist = torch.zeros(L, words + 1, dtype=torch.int64, device="cuda")
+    ring_a = torch.zeros(L, 4, ne, device="cuda")
+    ring_g = torch.zeros(L, 4, ne, device="cuda")
+    comp = ops.SpikeCompactor(ne)
+    auto = ops.AutoPropagator(t_src, t_tgt, hist, ring_a, n, n, batch)
+    pulled = []
+    for k in range(T):
+        z = (torch.rand(ne, device="cuda", generator=g) < rates[k] * 1e-3)
+        bits = torch.zeros(words + 1, dtype=torch.int64, device="cuda")
+        bits[:-1] = (z.view(-1, 64).to(torch.int64) << torch.arange(64, device="cuda")).sum(1)
+        hist[k % L] = bits
+        ids, cnt = comp(z.to(torch.uint8))
+        ops.csr_propagate_gather(bits, n, t_tgt, ring_g, n, batch, k)
+        auto.step(k, ids, cnt)
+        pulled.append(bool(auto.pulled_steps()[k % L]))
+        slot = (k + 1) % L
+        assert torch.equal(ring_a[slot], ring_g[slot]), k
+        ring_a[slot].zero_()        # the consumer's part: the slot is read and cleared before the next call
+        ring_g[slot].zero_()
+    assert pulled == [r >= 5.0 for r in rates]
+    assert float(ring_g.abs().max()) > 0
