@@ -6,6 +6,7 @@ tables, validates everything a kernel will index with on the host, and drives
 ``bmtk_glif3_simulate_fwd``.
 """
 import ctypes as C
+import math
 
 import numpy as np
 import torch
@@ -17,6 +18,16 @@ from .ops import Glif3State, SpikeCompactor, SynapseTable, _dev, _p, _stream, gl
 
 PULL_MAP_BYTES = 40 * 1024      # activity map of bmtk_csr_propagate_pull: what is left of 80 KB beside its accumulators
 PULL_MIN_DENSITY = 0.06         # synaptic events per synapse and step from which "auto" pulls instead of pushing
+                                # (the unfused pull form: batches other than 8, 16, 32, 64)
+# What a step of a batched run costs on one MI355X, in picoseconds, fitted to runs of 51,978 neurons x 60 M synapses at
+# batches 8, 16, 32 and 0 - 3.2 Hz and of 230,924 neurons x 77 M synapses at batch 8: the fused pull form streams the
+# joint table once per two steps (per synapse, divided by how full a row's blocks of 256 are) and adds a little per
+# synaptic event; the event-driven form pays per element for its update (less with a class table) and an atomic per event.
+FUSE_PS_PER_SYNAPSE = 1.35
+FUSE_PS_PER_EVENT = 6.0
+PUSH_PS_PER_ELEMENT = 55.0
+PUSH_PS_PER_ELEMENT_CLASS_TABLE = 27.0
+PUSH_PS_PER_EVENT = 48.0
 FUSE_LDS_BYTES = 150 * 1024     # LDS of one workgroup of the fused batched driver (kFuseLdsMax of csrc/simulate_fused.hip)
 FUSE_WAVES = 16                 # wavefronts of one of its workgroups (kFuseWaves)
 FUSE_BATCHES = (8, 16, 32, 64)  # lane = trial, whole bytes of spike bits per neuron
@@ -50,6 +61,21 @@ def resident_span(ne, batch, ring_slots, n_cu, single=True):
     return span
 
 
+def fused_pays(n_neurons, batch, n_synapses, class_table, rate_hz, h_ms=1.0):
+    """Whether the fused pull form of the batched driver is expected to take less time per step than pushing the
+    spikes as events, for a network of ``n_neurons`` with ``n_synapses`` recurrent and input synapses at ``batch``
+    trials and a mean rate of ``rate_hz``."""
+    if n_synapses <= 0:
+        return False
+    events = n_synapses * batch * float(rate_hz) * 1e-3 * h_ms
+    row = n_synapses / float(n_neurons)
+    blocks_full = row / (256.0 * math.ceil(row / 256.0))
+    fused = FUSE_PS_PER_SYNAPSE * n_synapses / blocks_full + FUSE_PS_PER_EVENT * events
+    push = ((PUSH_PS_PER_ELEMENT_CLASS_TABLE if class_table else PUSH_PS_PER_ELEMENT) * n_neurons * batch
+            + PUSH_PS_PER_EVENT * events)
+    return fused < push
+
+
 class Glif3Simulator:
     """A population of GLIF3 neurons with recurrent and external synapses.
 
@@ -74,12 +100,15 @@ class Glif3Simulator:
                 carries batch * rate * h events per step, and on one MI355X the pass is the cheaper of the two from
                 about 0.06 events per synapse and step (measured: 51,978 neurons x 32 trials at 3.2 Hz pull 168 us
                 against 340 pushed; 230,924 neurons x 8 and x 16 at 2.8 Hz pushed 132 / 237 us against 321 / 358
-                pulled).  Default 3 Hz: batches from 20 at 1 ms steps.
+                pulled).  Default 3 Hz: batches from 20 at 1 ms steps.  That mark decides the unfused ``pull``;
+                ``fused`` is decided by ``fused_pays``, which compares the fitted cost of a step in either form.
     fused       launch-per-step mode, batch 8, 16, 32 or 64, delay_offset 0: one launch per step in which a
                 wavefront sums what arrives at a neuron -- over recurrent and input synapses, from a joint
                 target-major table and a joint history of spike and input-event bits -- and advances the neuron's
-                trials, lane = trial; no arrival sum passes through device memory.  "auto": whenever ``pull``
-                "auto" would pull and the batch is one of those; takes any number of sources (above what the activity map in
+                trials, lane = trial; no arrival sum passes through device memory.  "auto": when ``fused_pays``
+                says a step costs less this way than pushed as events (the update's share grows with the batch,
+                the table pass does not: 51,978 neurons x 60 M synapses from batch 16 on at any rate, at batch 8
+                from about 3.3 Hz); takes any number of sources (above what the activity map in
                 LDS holds, one bit of the map stands for 2, 4, ... sources).  False: the pull form as separate
                 launches (below).  ``ring`` then holds only the few input ids repeated within a step.
     pull        launch-per-step mode only: sum the recurrent arrivals of a step in one pass over a target-major
@@ -240,7 +269,9 @@ class Glif3Simulator:
         if pull is True and not can_pull:
             raise ValueError("the pull form needs a recurrent table, launch-per-step mode, delay_offset 0 and "
                              "ring_slots * n_neurons / 8 bytes of LDS (at most 40 KB)")
-        if can_fuse and fused and (fused is True or pull is True or dense):
+        n_syn = sum(t.nnz for t in (self.rec, self.inp) if t is not None)
+        if can_fuse and fused and (fused is True or pull is True or
+                                   fused_pays(self.n, self.batch, n_syn, self.class_id is not None, expected_rate_hz, self.h)):
             tables = [t for t in (self.rec, self.inp) if t is not None]
             if all(fixed_point_ok(t) for t in tables):
                 self._setup_fused()
