@@ -47,6 +47,32 @@ struct Glif3Prop {
     }
 };
 
+// A class table small enough for LDS is copied there as it lies in device memory, [quantity][class], sixteen bytes
+// per lane and load, four loads asked for before the first is stored; ``prop`` must be 16-byte aligned.  Threads of
+// one wavefront then read a quantity of their own classes: two lanes meet in a bank only when their classes differ
+// by a multiple of the bank count, with this layout as with a transposed one.  The caller synchronises.
+template <int kThreads>
+__device__ __forceinline__ void stage_class_table(float *__restrict__ lds, const float *__restrict__ prop, int n_words)
+{
+    const int n4 = n_words >> 2;
+    const float4 *src = reinterpret_cast<const float4 *>(prop);
+    float4 *dst = reinterpret_cast<float4 *>(lds);
+    for (int base = 0; base < n4; base += 4 * kThreads) {
+        float4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = base + j * kThreads + (int)threadIdx.x;
+            v[j] = src[i < n4 ? i : 0];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = base + j * kThreads + (int)threadIdx.x;
+            if (i < n4) dst[i] = v[j];
+        }
+    }
+    for (int i = (n4 << 2) + (int)threadIdx.x; i < n_words; i += kThreads) lds[i] = prop[i];
+}
+
 // Advance one element by one step.  syn[r]: weight sum arriving on receptor r
 // in this step; I: external current.  Returns true on a spike and then sets
 // *frac to the fraction of the step at which U crossed threshold.

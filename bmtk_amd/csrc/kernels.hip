@@ -113,18 +113,21 @@ struct StepArgs {
     float *frac;
 };
 
-// kLdsTable: the propagators come from a class table small enough for LDS; the workgroup stages it once,
-// transposed to [class][quantity], and every thread reads its class's 29 values from there.  Read from device
-// memory instead, those 29 scattered loads per thread, not the state traffic, set the pace (4.3 TB/s of
-// algorithmic traffic against 6.1 with one parameter column per neuron).
+// kLdsTable: the propagators come from a class table small enough for LDS; the workgroup copies it there once
+// and every thread reads its class's 29 values from there.  Read from device memory instead, those 29 scattered
+// loads per thread, not the state traffic, set the pace (4.3 TB/s of algorithmic traffic against 6.1 with one
+// parameter column per neuron).  At N = 2^20 with 111 classes, on two machines: 18.3 / 18.5 us with four tiles
+// per workgroup, 18.1 / 19.5 with two, 24.4 with one; transposing the table on its way into LDS (an integer
+// division per word, one word per load) took 19.8 / 20.2 with four tiles.  By measured bytes the launch then moves
+// 5.95 TB/s where the form with a column per neuron moved 6.15 TB/s on the same machine.
 constexpr int kStepTiles = 4;
 
 template <bool kLdsTable>
 __global__ __launch_bounds__(kBlock) void glif3_step_kernel(StepArgs a)
 {
-    extern __shared__ float step_table[];  // [columns][GLIF3_NPROP] when kLdsTable
+    extern __shared__ __align__(16) float step_table[];  // [GLIF3_NPROP][columns] when kLdsTable
     // with the table in LDS a workgroup takes kStepTiles tiles of 256 elements, so that staging the table is
-    // shared by 1024 elements.  The state of all tiles is asked for first, before the table is staged: the loads
+    // shared by several tiles.  The state of all tiles is asked for first, before the table is staged: the loads
     // of the tiles travel together, and the staging runs while they are on their way.
     constexpr int kTiles = kLdsTable ? kStepTiles : 1;
     Glif3Elem s[kTiles];
@@ -145,11 +148,7 @@ __global__ __launch_bounds__(kBlock) void glif3_step_kernel(StepArgs a)
         }
     }
     if (kLdsTable) {
-        const int n_cols = (int)a.stride;
-        for (int i = threadIdx.x; i < n_cols * GLIF3_NPROP; i += kBlock) {
-            const int k = i / n_cols, c = i - k * n_cols;
-            step_table[c * GLIF3_NPROP + k] = a.prop[i];
-        }
+        stage_class_table<kBlock>(step_table, a.prop, (int)a.stride * GLIF3_NPROP);
         __syncthreads();
     }
 #pragma unroll
@@ -158,7 +157,7 @@ __global__ __launch_bounds__(kBlock) void glif3_step_kernel(StepArgs a)
         if (e[t] < a.ne) {
             Glif3Prop p;
             if (kLdsTable)
-                p.load(step_table + col[t] * GLIF3_NPROP, 1, 0);
+                p.load(step_table, a.stride, col[t]);
             else
                 p.load(a.prop, a.stride, col[t]);
             float frac = 0.0f;
@@ -431,9 +430,10 @@ int bmtk_glif3_step_fwd(int64_t n_neurons, int32_t batch, float *V, float *asc, 
     BMTK_REQUIRE(ne < (1ll << 31), "glif3_step_fwd: n_neurons*batch must stay below 2^31");
     StepArgs a{ne, batch, V, asc, y1, y2, ref, prop, prop_stride, class_id, h, syn, clear_syn, i_ext, z, zbits, frac};
     const unsigned grid = (unsigned)((ne + kBlock - 1) / kBlock);
-    // a class table of up to 48 KB (423 classes) is staged in LDS by every workgroup
+    // a class table of up to 48 KB (423 classes) is staged in LDS by every workgroup (sixteen bytes per load: a
+    // table that is not 16-byte aligned is read through the caches instead)
     const size_t table_bytes = (size_t)prop_stride * GLIF3_NPROP * sizeof(float);
-    if (class_id && table_bytes <= 48u * 1024u)
+    if (class_id && table_bytes <= 48u * 1024u && ((uintptr_t)prop & 15u) == 0)
         hipLaunchKernelGGL(glif3_step_kernel<true>, dim3((grid + kStepTiles - 1) / kStepTiles), dim3(kBlock), table_bytes,
                            (hipStream_t)stream, a);
     else

@@ -49,7 +49,7 @@ struct SimLaunch {
 
 __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, SimLaunch q)
 {
-    extern __shared__ float table[];  // [class][GLIF3_NPROP] when q.lds_table
+    extern __shared__ __align__(16) float table[];  // [GLIF3_NPROP][class] when q.lds_table
     const int batch = s.batch;
     const int64_t ne = s.n_neurons * (int64_t)batch;
     const int64_t words = (ne + 63) >> 6;
@@ -108,54 +108,64 @@ __global__ __launch_bounds__(kSimBlock) void sim_step_kernel(bmtk_glif3_sim s, S
     }
 
     // ---- update (or, in the closing launch, fold only) ----
+    // What an element reads from device memory -- its state, slot t-1 of the ring with the pulled sums, its current,
+    // its class -- is asked for first; the class table is copied into LDS while those loads are on their way.
     const int n_cols = (int)s.prop_stride;
-    if (q.lds_table) {
-        for (int i = threadIdx.x; i < n_cols * GLIF3_NPROP; i += kSimBlock) {
-            const int k = i / n_cols, c = i - k * n_cols;
-            table[c * GLIF3_NPROP + k] = s.prop[i];
-        }
-        __syncthreads();
-    }
     const int64_t e = (int64_t)(bid - q.n_input - q.n_deliver) * kSimBlock + threadIdx.x;
     bool spike = false;
     float frac = 0.0f;
-    if (e < ne) {
+    const bool live = e < ne;
+    float *prev = s.ring + (int64_t)((q.t + L - 1) % L) * GLIF3_NREC * ne + (live ? e : 0);
+    int64_t col = 0;
+    float arrived[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float I = 0.0f;
+    Glif3Elem st;
+    if (live) {
         const int64_t n = batch == 1 ? e : (int64_t)((uint32_t)e / (uint32_t)batch);
-        const int64_t col = s.class_id ? (int64_t)s.class_id[n] : n;
-        float *prev = s.ring + (int64_t)((q.t + L - 1) % L) * GLIF3_NREC * ne + e;
+        col = s.class_id ? (int64_t)s.class_id[n] : n;
+        if (q.fold_prev) {
+#pragma unroll
+            for (int k = 0; k < GLIF3_NREC; ++k) {
+                float a = prev[k * ne];
+                if (q.pull) a = a + s.pull_syn[k * ne + e];
+                if (q.pull_inp) a = a + s.pull_inp_syn[k * ne + e];
+                arrived[k] = a;
+            }
+        }
+        if (q.do_update) {
+            glif3_load(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
+            I = s.i_ext ? s.i_ext[e] : 0.0f;
+        }
+    }
+    if (q.lds_table) {
+        stage_class_table<kSimBlock>(table, s.prop, n_cols * GLIF3_NPROP);
+        __syncthreads();
+    }
+    if (live) {
         if (!q.do_update) {
             if (q.fold_prev) {
 #pragma unroll
                 for (int k = 0; k < GLIF3_NREC; ++k) {
-                    const float psc0 = q.lds_table ? table[col * GLIF3_NPROP + GLIF3_PSC0_0 + k]
+                    const float psc0 = q.lds_table ? table[(GLIF3_PSC0_0 + k) * n_cols + col]
                                                    : s.prop[(GLIF3_PSC0_0 + k) * s.prop_stride + col];
-                    float a = prev[k * ne];
-                    if (q.pull) a = a + s.pull_syn[k * ne + e];
-                    if (q.pull_inp) a = a + s.pull_inp_syn[k * ne + e];
                     prev[k * ne] = 0.0f;
-                    s.y1[k * ne + e] = s.y1[k * ne + e] + a * psc0;
+                    s.y1[k * ne + e] = s.y1[k * ne + e] + arrived[k] * psc0;
                 }
             }
         } else {
             Glif3Prop p;
             if (q.lds_table)
-                p.load(table + col * GLIF3_NPROP, 1, 0);
+                p.load(table, n_cols, col);
             else
                 p.load(s.prop, s.prop_stride, col);
-            Glif3Elem st;
-            glif3_load(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
             if (q.fold_prev) {
 #pragma unroll
                 for (int k = 0; k < GLIF3_NREC; ++k) {
-                    float a = prev[k * ne];
-                    if (q.pull) a = a + s.pull_syn[k * ne + e];
-                    if (q.pull_inp) a = a + s.pull_inp_syn[k * ne + e];
                     prev[k * ne] = 0.0f;
-                    st.y1[k] = st.y1[k] + a * p.psc0[k];
+                    st.y1[k] = st.y1[k] + arrived[k] * p.psc0[k];
                 }
             }
             const float zero[GLIF3_NREC] = {0.0f, 0.0f, 0.0f, 0.0f};
-            const float I = s.i_ext ? s.i_ext[e] : 0.0f;
             const int ref_before = st.ref;
             spike = glif3_update(st, p, s.h, zero, I, &frac);
             glif3_store(st, s.V, s.asc, s.y1, s.y2, s.ref, ne, e);
@@ -359,7 +369,7 @@ extern "C" int bmtk_glif3_simulate_fwd(const bmtk_glif3_sim *sim, int64_t step0,
     const bool repeats = pull_inp && s.in_repeat_ptr != nullptr;
     const int n_input = has_inp ? (!pull_inp ? 64 : (repeats ? 4 : 0)) : 0;
     const size_t table_bytes = (size_t)s.prop_stride * GLIF3_NPROP * sizeof(float);
-    q.lds_table = (s.class_id && table_bytes <= (size_t)kLdsTableBytes) ? 1 : 0;
+    q.lds_table = (s.class_id && table_bytes <= (size_t)kLdsTableBytes && ((uintptr_t)s.prop & 15u) == 0) ? 1 : 0;
     const size_t lds = q.lds_table ? table_bytes : 0;
     for (int64_t k = 0; k <= n_steps; ++k) {
         const bool closing = k == n_steps;

@@ -101,6 +101,44 @@ def test_step_without_inputs_and_outputs():
         np.testing.assert_array_equal(got[k], cpu[k])
 
 
+@pytest.mark.parametrize("classes", [1, 3, 7, 111, 423, 500])
+def test_class_table_in_any_size_and_alignment_equals_one_column_per_neuron(classes):
+    """The class table is copied into LDS sixteen bytes at a time when it is 16-byte aligned and at most 48 KB
+    (423 classes), and read through the caches otherwise: word counts that are no multiple of four (3 x 29, 7 x 29),
+    the largest staged table, a larger one and a table that starts 4 bytes past an aligned address must all give,
+    bit for bit, what one parameter column per neuron gives (the form the oracle test above covers)."""
+    rng = np.random.default_rng(23 + classes)
+    n, batch, h = 3000, 2, 1.0
+    par = synthetic.random_cells(rng, classes)
+    class_id = rng.integers(0, classes, n).astype(np.int32)
+    class_id[:min(classes, n)] = np.arange(min(classes, n))   # every class occurs
+    p32 = orc.precompute(par, h).astype(np.float32)
+    st0 = synthetic.random_state(rng, par, n, batch, class_id)
+    table = to_dev(p32)
+    shifted = torch.empty(p32.size + 1, device="cuda")[1:].view(p32.shape)
+    shifted.copy_(table)
+    assert table.data_ptr() % 16 == 0 and shifted.data_ptr() % 16 == 4
+    forms = {"per neuron": (to_dev(np.ascontiguousarray(p32[:, class_id])), None),
+             "table": (table, to_dev(class_id)), "table off alignment": (shifted, to_dev(class_id))}
+    got = {}
+    for name, (prop, cid) in forms.items():
+        st = ops.Glif3State.from_numpy(st0)
+        zb = torch.zeros(ops.n_words(n * batch) + 1, dtype=torch.int64, device="cuda")
+        spikes = 0
+        r = np.random.default_rng(5)
+        for t in range(60):
+            syn = to_dev((r.lognormal(0, 1, (4, n * batch)) * (r.random((4, n * batch)) < 0.05) * 30).astype(np.float32))
+            cur = to_dev(r.normal(100, 50, n * batch).astype(np.float32))
+            ops.glif3_step_fwd(st, prop, h, batch=batch, class_id=cid, syn=syn, i_ext=cur, zbits=zb)
+            spikes += int(ops.unpack_bits(zb, n * batch).sum())
+        got[name] = (st.to_numpy(), spikes)
+    assert got["per neuron"][1] > 0
+    for name in ("table", "table off alignment"):
+        assert got[name][1] == got["per neuron"][1]
+        for k, v in got["per neuron"][0].items():
+            np.testing.assert_array_equal(got[name][0][k], v, err_msg="%s %s" % (name, k))
+
+
 def test_step_argument_errors():
     from bmtk_amd._lib import BmtkAmdError
     st = ops.Glif3State.zeros(10)
