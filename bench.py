@@ -407,7 +407,8 @@ def bench_lds(torch, clock_ghz=2.4):
     """What the LDS and the path between workgroups cost (the figures the resident kernels' design quotes):
     additions into a 92 KB LDS array in five forms with 64, 8 and 1 active lanes per wavefront, in clocks per
     wavefront instruction on a compute unit at a nominal 2.4 GHz, and the time a word takes from one workgroup to
-    another through device memory, on one XCD and across two."""
+    another through device memory, on one XCD and across two; and the rate of scattered fp32 atomic additions into
+    device memory, anywhere and with every XCD confined to an eighth of the region."""
     from bmtk_amd import _lib
     from bmtk_amd.ops import _p, _stream
     lib = _lib.load()
@@ -438,6 +439,23 @@ def bench_lds(torch, clock_ghz=2.4):
         x = xcc.cpu().tolist()
         entries.append({"kernel": "hop_kernel", "workload": "word passed between two workgroups through device memory, " + what,
                         "xcd_of_each": x[:2], "gave_up": bool(x[2]), "us_per_hop": best / hop_rounds / 2 * 1e6})
+    # scattered fp32 atomic additions into device memory: what holds the event-driven propagation forms
+    per_thread, blocks = 64, 8192
+    for mb in (4, 53, 400):
+        cells = torch.zeros(mb * (1 << 20) // 32 * 8, device="cuda")
+        for own in (0, 1):
+            best = None
+            for _ in range(3):
+                cells.zero_()
+                _, dev = time_region(torch, lambda: _lib.check(lib.bmtk_microbench_atomics(
+                    _p(cells), cells.numel(), per_thread, blocks, own, _stream())))
+                best = dev if best is None else min(best, dev)
+            total = blocks * 256 * per_thread
+            entries.append({"kernel": "atomic_add_kernel",
+                            "workload": "fp32 atomic additions to random cells of %d MB, %s" % (
+                                mb, "each workgroup within its XCD's eighth" if own else "anywhere"),
+                            "atomics_per_s": total / best, "none_lost": float(cells.double().sum().item()) == float(total)})
+        del cells
     return entries
 
 

@@ -60,7 +60,7 @@ class Glif3Bwd(C.Structure):
     ]
 
 
-ABI_VERSION = 23  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
+ABI_VERSION = 24  # BMTK_AMD_ABI_VERSION of include/bmtk_amd.h that the mirrors above were written for
 
 # name -> (restype, argtypes); every symbol include/bmtk_amd.h declares
 SIGNATURES = {
@@ -106,6 +106,7 @@ SIGNATURES = {
                                                  c_void_p, c_void_p]),
     "bmtk_csr_propagate_bwd_blocked_plan": (c_int32, [c_int64, c_int32, c_void_p]),
     "bmtk_microbench_lds": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "bmtk_microbench_atomics": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "bmtk_microbench_hop": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_int32, C.c_uint32, c_void_p]),
     "bmtk_spike_counts": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
 }

@@ -1,6 +1,7 @@
-// Two small measurements the design of the simulation kernels rests on, kept in the library so that they can be
-// repeated (bench.py --kernels lds): what an addition into LDS costs in its different forms, and how long a word
-// takes from one workgroup to another through device memory.
+// Three small measurements the design of the simulation kernels rests on, kept in the library so that they can be
+// repeated (bench.py --kernels lds): what an addition into LDS costs in its different forms, how long a word
+// takes from one workgroup to another through device memory, and how many scattered fp32 atomic additions into
+// device memory the chip works off per second.
 #include "common.hpp"
 
 namespace bmtk {
@@ -80,9 +81,35 @@ __global__ void hop_kernel(unsigned *flag, unsigned *xcc, int a, int b, int roun
     }
 }
 
+// Every thread adds 1 to `per_thread` pseudo-random cells of a region of device memory with the global fp32 atomic
+// (what the event-driven propagation does per synaptic event).  own_eighth: a workgroup's cells all lie in the eighth
+// of the region that belongs to the XCD it runs on (read from the hardware register), so that no cache line is
+// ever touched from two XCDs.
+__global__ __launch_bounds__(kBlock) void atomic_add_kernel(float *cells, unsigned n_cells, int per_thread, int own_eighth)
+{
+    const unsigned part = n_cells >> 3;
+    const unsigned base = own_eighth ? (xcc_id() & 7u) * part : 0u, range = own_eighth ? part : n_cells;
+    unsigned x = (blockIdx.x * kBlock + threadIdx.x) * 2654435761u + 12345u;
+    for (int k = 0; k < per_thread; ++k) {
+        x = x * 1664525u + 1013904223u;
+        atomicAdd(cells + base + (x >> 8) % range, 1.0f);
+    }
+}
+
 }  // namespace bmtk
 
 using namespace bmtk;
+
+extern "C" int bmtk_microbench_atomics(float *cells, int64_t n_cells, int32_t per_thread, int32_t n_blocks,
+                                       int32_t own_eighth, void *stream)
+{
+    BMTK_REQUIRE(cells && n_cells >= 8 && n_cells < (1ll << 32) && per_thread >= 1 && n_blocks >= 1,
+                 "microbench_atomics: cells non-null, 8 <= n_cells < 2^32, per_thread and n_blocks positive");
+    hipLaunchKernelGGL(atomic_add_kernel, dim3((unsigned)n_blocks), dim3(kBlock), 0, (hipStream_t)stream, cells,
+                       (unsigned)n_cells, per_thread, own_eighth);
+    BMTK_CHECK_LAUNCH("microbench_atomics");
+    return BMTK_OK;
+}
 
 extern "C" int bmtk_microbench_lds(int32_t op, int32_t active_lanes, int32_t rounds, int32_t n_blocks, float *out,
                                    void *stream)

@@ -49,7 +49,7 @@ extern "C" {
 
 /* Bumped whenever a struct layout or a signature below changes; bmtk_amd_abi_version() returns the value the
  * library was built with. */
-#define BMTK_AMD_ABI_VERSION 23
+#define BMTK_AMD_ABI_VERSION 24
 int bmtk_amd_abi_version(void);
 const char *bmtk_amd_last_error(void);
 /* sizeof(bmtk_glif3_sim) as the library was compiled, for bindings that mirror the struct */
@@ -552,7 +552,7 @@ int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_step
                       void *stream);
 
 /* ---------------------------------------------------------------------------
- * Two measurements the kernels' design rests on, kept in the library so that they can be repeated
+ * Three measurements the kernels' design rests on, kept in the library so that they can be repeated
  * (bench.py --kernels lds).  No counterpart in the reference.
  *
  * bmtk_microbench_lds: n_blocks workgroups of 1024 threads; in each of `rounds` rounds, `active_lanes` lanes of every
@@ -563,7 +563,13 @@ int bmtk_spike_counts(const uint64_t *spike_bits, int64_t stride, int64_t n_step
  * bmtk_microbench_hop: workgroups block_a and block_b (0..15; workgroups go round the XCDs, so 0 and 8 share one, 0
  * and 1 do not) pass a counter back and forth `rounds` times through two words of `flags` (at least 512 bytes,
  * zeroed by the caller) with relaxed agent-scope loads and stores; time / rounds = two hops.  xcc (3 words, zeroed
- * by the caller): the XCD each ran on, and 1 in xcc[2] if a wait ran out after spin_limit polls (both then leave). */
+ * by the caller): the XCD each ran on, and 1 in xcc[2] if a wait ran out after spin_limit polls (both then leave).
+ * bmtk_microbench_atomics: n_blocks workgroups of 256 threads; every thread adds 1 to per_thread pseudo-random cells
+ * of `cells` (n_cells floats, zeroed by the caller) with the global fp32 atomic; own_eighth != 0: a workgroup only adds
+ * into the eighth of the region that belongs to the XCD it runs on.  The caller times the launch; the cells then sum
+ * to n_blocks * 256 * per_thread. */
+int bmtk_microbench_atomics(float *cells, int64_t n_cells, int32_t per_thread, int32_t n_blocks, int32_t own_eighth,
+                            void *stream);
 int bmtk_microbench_lds(int32_t op, int32_t active_lanes, int32_t rounds, int32_t n_blocks, float *out, void *stream);
 int bmtk_microbench_hop(uint32_t *flags, uint32_t *xcc, int32_t block_a, int32_t block_b, int32_t rounds,
                         uint32_t spin_limit, void *stream);
