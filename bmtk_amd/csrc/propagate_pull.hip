@@ -44,6 +44,27 @@ __global__ __launch_bounds__(kBlock) void pull_anymap_kernel(const uint64_t *__r
         any_map[(int64_t)slot * n_w32 + (j >> 5)] = (uint32_t)(m >> (lane_id() & 32));
 }
 
+// The same facts source-major for up to 8 history rows: any_rel[j] bit d = source j fired in at least one trial in
+// the step held by history row (slot_now - d) mod L, d = 0 .. L-1.  One byte answers every question a synapse of
+// that source can ask, whatever its delay and for both arrival steps of pull2_kernel, from an address that is the
+// source itself.
+__global__ __launch_bounds__(kBlock) void pull_anyrel_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride,
+                                                             int L, int batch, int64_t n_src, int slot_now,
+                                                             uint8_t *__restrict__ any_rel)
+{
+    const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (j >= n_src) return;
+    unsigned m = 0u;
+    for (int d = 0; d < L; ++d) {
+        const uint64_t *row = hist + (int64_t)((slot_now + L - d) % L) * hist_stride;
+        bool any = false;
+        for (int t0 = 0; t0 < batch && !any; t0 += kWave)
+            any = source_mask(row, (int)j, batch, t0, min(kWave, batch - t0)) != 0ull;
+        m |= (any ? 1u : 0u) << d;
+    }
+    any_rel[j] = (uint8_t)m;
+}
+
 constexpr int kPullBlock = 1024;  // 16 wavefronts share one staged activity map
 // per wavefront: 4 x 64 accumulators of 8 bytes and a stage of 64 entries of 8 bytes
 constexpr size_t kPullAccBytes = (size_t)(kPullBlock / kWave) * (GLIF3_NREC + 1) * kWave * sizeof(unsigned long long);
@@ -206,7 +227,9 @@ __global__ __launch_bounds__(kPullBlock, 8) void pull_kernel(const uint64_t *__r
 // 1024 threads per compute unit (its two sets of accumulators and stages take 80 KB of LDS).
 constexpr size_t kPull2AccBytes = 2 * kPullAccBytes;
 constexpr size_t kPull2LdsMax = 150u * 1024u;
-template <bool kWords64>
+// kByteMap: L <= 8 and one byte per source fits the LDS: the activity map is pull_anyrel_kernel's, one LDS read and
+// two shifts per synapse answer both questions (with the bit map: two reads at computed rows).
+template <bool kWords64, bool kByteMap>
 __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride, int L,
                                                            int batch, const int32_t *__restrict__ indptr,
                                                            const bmtk_synapse *__restrict__ packed,
@@ -242,10 +265,18 @@ __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__res
     fetch(d0, b0);
     PullBlock b1 = cursor.next();
     fetch(d1, b1);
-    // the activity map comes into LDS while the first table blocks are on their way
-    for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
+    // the activity map comes into LDS while the first table blocks are on their way (n_w32 counts the byte map's
+    // 16-byte pieces when kByteMap)
+    if (kByteMap) {
+        const uint4 *src16 = reinterpret_cast<const uint4 *>(any_map);
+        uint4 *dst16 = reinterpret_cast<uint4 *>(any_l);
+        for (int i = threadIdx.x; i < n_w32; i += kPullBlock) dst16[i] = src16[i];
+    } else {
+        for (int i = threadIdx.x; i < L * n_w32; i += kPullBlock) any_l[i] = any_map[i];
+    }
     __syncthreads();
     if (b0.row >= n_tgt) return;
+    const uint8_t *any_b = reinterpret_cast<const uint8_t *>(any_l);
 #pragma unroll
     for (int r = 0; r < 2 * GLIF3_NREC; ++r) acc[r * kWave + lane] = 0ull;
     int staged[2] = {0, 0};  // entries in the two stages (same in all lanes)
@@ -275,21 +306,29 @@ __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__res
         const unsigned left = cb.base < cb.p1 ? (unsigned)(cb.p1 - cb.base) : 0u;
         // activity bits of the four chunks for both arrival steps (LDS reads, no branch between them): the map of a
         // step is the row of its history slot; a synapse of delay d looks at step t-1-d and at step t-d
+        // (byte map: bit d of a source's byte = fired d steps before the step whose row is now_b, which holds step
+        // t - L; a synapse of delay d asks for bit d on behalf of step t and bit d + 1, bit L being bit 0, for t - 1)
         unsigned word_a[kPullChunks], word_b[kPullChunks];
 #pragma unroll
         for (int u = 0; u < kPullChunks; ++u) {
             const unsigned tdr = (unsigned)cd[u];
-            const unsigned back_b = now_b - (tdr >> 26), back_a = now_a - (tdr >> 26);
-            const unsigned at = (tdr & 0xFFFFFFu) >> 5;
-            word_b[u] = any_l[__umul24(min(back_b, back_b + uL), uw32) + at];
-            word_a[u] = any_l[__umul24(min(back_a, back_a + uL), uw32) + at];
+            if (kByteMap) {
+                const unsigned m = any_b[tdr & 0xFFFFFFu];
+                word_b[u] = (m | (m << uL)) >> (tdr >> 26);
+                word_a[u] = word_b[u] >> 1;
+            } else {
+                const unsigned back_b = now_b - (tdr >> 26), back_a = now_a - (tdr >> 26);
+                const unsigned at = (tdr & 0xFFFFFFu) >> 5;
+                word_b[u] = any_l[__umul24(min(back_b, back_b + uL), uw32) + at] >> (tdr & 31u);
+                word_a[u] = any_l[__umul24(min(back_a, back_a + uL), uw32) + at] >> (tdr & 31u);
+            }
         }
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
 #pragma unroll
             for (int u = 0; u < kPullChunks; ++u) {
                 const unsigned tdr = (unsigned)cd[u];
-                const bool hit = lane + u * kWave < left && (((k ? word_b[u] : word_a[u]) >> (tdr & 31u)) & 1u);
+                const bool hit = lane + u * kWave < left && ((k ? word_b[u] : word_a[u]) & 1u);
                 const unsigned long long who = __ballot(hit);
                 const int n = __popcll(who);
                 if (n == 0) continue;
@@ -369,7 +408,9 @@ __global__ __launch_bounds__(kBlock) void auto_anymap_kernel(const uint64_t *__r
 extern "C" int64_t bmtk_csr_propagate_pull_workspace_bytes(int32_t L, int64_t n_src)
 {
     if (L <= 0 || n_src <= 0) return 0;
-    return (int64_t)L * ((n_src + 31) / 32) * 4;
+    // one bit per (row, source), or one byte per source (the two-step form with up to 8 rows): the larger of the two
+    const int64_t bits = (int64_t)L * ((n_src + 31) / 32) * 4, bytes = (n_src + 15) / 16 * 16;
+    return bits > bytes ? bits : bytes;
 }
 
 extern "C" int bmtk_csr_propagate_pull(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src,
@@ -529,13 +570,23 @@ extern "C" int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist
     BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31) && n_src < (1ll << 24), "csr_propagate_pull2: network too large");
     BMTK_REQUIRE((int64_t)L * hist_stride < (1ll << 29) && hist_stride < (1ll << 24),
                  "csr_propagate_pull2: spike history beyond 4 GiB");
-    const int n_w32 = (int)((n_src + 31) / 32);
-    const size_t lds = (size_t)L * n_w32 * 4 + kPull2AccBytes;
+    // the activity map: one byte per source when the history has at most 8 rows and the bytes fit the LDS (the
+    // kernel then asks one question per synapse instead of two), else one bit per row and source
+    const int n_16 = (int)((n_src + 15) / 16);
+    const bool byte_map = L <= 8 && (size_t)n_16 * 16 + kPull2AccBytes <= kPull2LdsMax;
+    const int n_w32 = byte_map ? n_16 : (int)((n_src + 31) / 32);
+    const size_t lds = (byte_map ? (size_t)n_16 * 16 : (size_t)L * n_w32 * 4) + kPull2AccBytes;
     BMTK_REQUIRE(lds <= kPull2LdsMax, "csr_propagate_pull2: L * n_src too large for the activity map in LDS");
     uint32_t *any_map = (uint32_t *)workspace;
-    const int64_t map_threads = (int64_t)L * n_w32 * 32;
-    hipLaunchKernelGGL(pull_anymap_kernel, dim3((unsigned)((map_threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       (hipStream_t)stream, spike_hist, hist_stride, L, batch, n_src, n_w32, any_map);
+    if (byte_map) {
+        hipLaunchKernelGGL(pull_anyrel_kernel, dim3((unsigned)((n_src + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           (hipStream_t)stream, spike_hist, hist_stride, L, batch, n_src, (int)(t_arrive % L),
+                           (uint8_t *)workspace);
+    } else {
+        const int64_t map_threads = (int64_t)L * n_w32 * 32;
+        hipLaunchKernelGGL(pull_anymap_kernel, dim3((unsigned)((map_threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           (hipStream_t)stream, spike_hist, hist_stride, L, batch, n_src, n_w32, any_map);
+    }
     int dev = 0;
     (void)hipGetDevice(&dev);
     static int cu_count[64];
@@ -549,23 +600,30 @@ extern "C" int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist
     const unsigned want = (unsigned)((n_tgt + rows_per_block - 1) / rows_per_block);
     const dim3 grid(want < (unsigned)n_cu ? want : (unsigned)n_cu, (unsigned)((batch + kWave - 1) / kWave));
     BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_pull2: batch too large");
-    static bool asked[2][64];
-    if (dev >= 0 && dev < 64 && !asked[batch == kWave][dev]) {
-        const hipError_t err = hipFuncSetAttribute(
-            batch == kWave ? reinterpret_cast<const void *>(pull2_kernel<true>) : reinterpret_cast<const void *>(pull2_kernel<false>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPull2LdsMax);
+    const void *const kernels[2][2] = {
+        {reinterpret_cast<const void *>(pull2_kernel<false, false>), reinterpret_cast<const void *>(pull2_kernel<false, true>)},
+        {reinterpret_cast<const void *>(pull2_kernel<true, false>), reinterpret_cast<const void *>(pull2_kernel<true, true>)}};
+    const void *kernel = kernels[batch == kWave][byte_map];
+    static bool asked[2][2][64];
+    if (dev >= 0 && dev < 64 && !asked[batch == kWave][byte_map][dev]) {
+        const hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPull2LdsMax);
         if (err != hipSuccess) {
             set_error("csr_propagate_pull2: cannot reserve %zu bytes of LDS: %s", kPull2LdsMax, hipGetErrorString(err));
             return BMTK_E_LAUNCH;
         }
-        asked[batch == kWave][dev] = true;
+        asked[batch == kWave][byte_map][dev] = true;
     }
-    if (batch == kWave)
-        hipLaunchKernelGGL(pull2_kernel<true>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
-                           batch, indptr, packed, syn2, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
-    else
-        hipLaunchKernelGGL(pull2_kernel<false>, grid, dim3(kPullBlock), lds, (hipStream_t)stream, spike_hist, hist_stride, L,
-                           batch, indptr, packed, syn2, n_tgt, n_tgt * (int64_t)batch, (int)(t_arrive % L), any_map, n_w32);
+    int64_t ne = n_tgt * (int64_t)batch;
+    int slot_now = (int)(t_arrive % L), n_map = n_w32;
+    const uint32_t *map_arg = any_map;
+    int64_t stride_arg = hist_stride;
+    int32_t L_arg = L, batch_arg = batch;
+    void *args[] = {&spike_hist, &stride_arg, &L_arg, &batch_arg, &indptr, &packed, &syn2, &n_tgt, &ne, &slot_now, &map_arg, &n_map};
+    const hipError_t err = hipLaunchKernel(kernel, grid, dim3(kPullBlock), args, lds, (hipStream_t)stream);
+    if (err != hipSuccess) {
+        set_error("csr_propagate_pull2: launch failed: %s", hipGetErrorString(err));
+        return BMTK_E_LAUNCH;
+    }
     BMTK_CHECK_LAUNCH("csr_propagate_pull2");
     return BMTK_OK;
 }

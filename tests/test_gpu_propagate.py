@@ -194,23 +194,26 @@ def test_pull_matches_oracle(batch, p):
     assert np.abs(want).max() > 0
 
 
-@pytest.mark.parametrize("batch,p,n_src", [(1, 0.3, 211), (5, 0.2, 211), (32, 0.05, 1500), (64, 0.01, 211),
-                                            (64, 0.3, 211), (100, 0.1, 97), (130, 0.05, 211)])
-def test_two_step_pull_equals_two_pulls(batch, p, n_src):
+@pytest.mark.parametrize("batch,p,n_src,L", [(1, 0.3, 211, 6), (5, 0.2, 211, 6), (32, 0.05, 1500, 6), (64, 0.01, 211, 6),
+                                              (64, 0.3, 211, 6), (100, 0.1, 97, 6), (130, 0.05, 211, 6),
+                                              (64, 0.05, 211, 2), (32, 0.05, 400, 8), (64, 0.05, 211, 9), (5, 0.2, 300, 14)])
+def test_two_step_pull_equals_two_pulls(batch, p, n_src, L):
     """``csr_propagate_pull2`` (the arrivals of steps tau-1 and tau in one pass over the table) == two calls of
     ``csr_propagate_pull`` over the same spike history, bit for bit: both add the same Q31.32 weights, whose sum
-    does not depend on the order.  (The one-step form is pinned against the oracle above.)"""
-    rng = np.random.default_rng(70 + batch)
-    n_tgt, L = 190, 6
-    src, tgt, w, d, r = _edges(rng, n_src, n_tgt, 15000)
+    does not depend on the order.  (The one-step form is pinned against the oracle above.)  Histories of up to 8
+    rows take the form with one byte of activity per source, longer ones the form with one bit per row and
+    source; delays run up to L - 1 steps, the longest a history of L rows serves."""
+    rng = np.random.default_rng(70 + batch + L)
+    n_tgt = 190
+    src, tgt, w, d, r = _edges(rng, n_src, n_tgt, 15000, max_delay=L - 1)
     table = ops.SynapseTable.from_numpy(net.coo_to_csr(src, tgt, w, d, r, n_rows=n_tgt, major="target"))
     words = ops.n_words(n_src * batch)
     hist = torch.zeros(L, words + 1, dtype=torch.int64, device="cuda")
     one = torch.full((2, 4, n_tgt * batch), 7.0, device="cuda")
     two = torch.full((2, 4, n_tgt * batch), -3.0, device="cuda")      # must be overwritten, not accumulated
-    for tau in range(1, 15):
+    for tau in range(1, 2 * L + 4):
         hist[(tau - 1) % L] = to_dev(bits_of((rng.random(n_src * batch) < p).astype(np.uint8)))
-        if tau < L:                                                    # both steps need their L-1 steps of history
+        if tau <= L:                                                   # both steps need their L-1 steps of history
             continue
         # the row of step tau-1 is never read by the pull of step tau-1: delays are at least one step
         ops.csr_propagate_pull(hist, n_src, table, one[0], n_tgt, batch, tau - 1)
