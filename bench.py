@@ -166,16 +166,17 @@ def bench_compaction(torch, steps=200, warmup=20):
     return out
 
 
-PROPAGATION_MODES = ("scatter", "gather", "pull", "pull2", "auto")
+PROPAGATION_MODES = ("scatter", "gather", "pull", "pull2", "auto", "auto2")
 PROPAGATION_RATES = (0.2, 1.0, 5.0, 20.0)
 
 
 def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rates=PROPAGATION_RATES):
     """Isolated spike propagation: 51,978 neurons, Poisson(1000) in-degree
-    (~52 M synapses), batch 64, Bernoulli spikes at 0.2, 1, 5 and 20 Hz.  Five forms: the event-driven scatter, the
+    (~52 M synapses), batch 64, Bernoulli spikes at 0.2, 1, 5 and 20 Hz.  Six forms: the event-driven scatter, the
     row-wise gather, the pull over the spike history of the last L steps, the same pull for two arrival steps per
-    pass over the table (`pull2`, timed per arrival step), and `auto`, which decides on the device,
-    step by step, between pushing a step's spikes as events and leaving them to the pull.  A pool of L spike
+    pass over the table (`pull2`, timed per arrival step), `auto`, which decides on the device,
+    step by step, between pushing a step's spikes as events and leaving them to the pull, and `auto2`, the same
+    switch called every second step with the two-step pull behind it (timed per arrival step).  A pool of L spike
     patterns serves as the history (row k % L = the spikes of step k)."""
     from bmtk_amd import ops, synthetic
     n, batch, L = 51978, 64, 6
@@ -207,6 +208,7 @@ def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rate
         syn = torch.zeros(4, ne, device="cuda")
         syn2 = torch.zeros(2, 4, ne, device="cuda")
         auto = ops.AutoPropagator(t_src, t_tgt, hist, ring, n, n, batch)
+        auto2 = ops.AutoPropagator2(t_src, t_tgt, hist, ring, n, n, batch)
         for mode in modes:
             def one(k):
                 if mode == "scatter":
@@ -220,6 +222,9 @@ def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rate
                 elif mode == "pull2":                                  # two arrival steps per call, every other step
                     if k % 2 == 0:
                         ops.csr_propagate_pull2(hist, n, t_tgt, syn2, n, batch, k + L + 1)
+                elif mode == "auto2":                                  # likewise: the two-step form of the switch
+                    if k % 2 == 1:
+                        auto2.step2(k, pool_ev[(k - 1) % L][0], pool_ev[(k - 1) % L][1], pool_ev[k % L][0], pool_ev[k % L][1])
                 else:
                     ops.csr_propagate_pull(hist, n, t_tgt, syn, n, batch, k + L)
             for k in range(warmup):
@@ -229,21 +234,24 @@ def bench_propagation(torch, steps=200, warmup=20, modes=PROPAGATION_MODES, rate
             per = dev / steps
             alg = events * B_PER_EVENT
             traffic = profile_traffic("propagation_kernels_52k_batch64.txt", "hbm_bytes_per_launch_%s_%gHz" % (mode, rate))
-            if traffic is not None and mode == "pull2":
+            two = mode in ("pull2", "auto2")
+            if traffic is not None and two:
                 traffic /= 2                                            # per arrival step, like the time below
             entry = {"kernel": {"auto": "auto_push_kernel or pull_kernel, chosen on the device",
+                                "auto2": "auto2: auto_push_kernel or pull2_kernel, chosen on the device for each of the two steps of a call",
                                 "pull2": "pull2_kernel: the arrivals of two steps per launch, half a launch per step"}
                                .get(mode, mode + "_kernel"),
                      "workload": "propagation N=51978 nnz=%d batch=64 rate=%gHz" % (t_src.nnz, rate),
                      "events_per_launch": events, "active_elements_per_launch": active,
-                     "synaptic_events_per_s": events / per, "us_per_launch": per * 1e6 * (2 if mode == "pull2" else 1),
+                     "synaptic_events_per_s": events / per, "us_per_launch": per * 1e6 * (2 if two else 1),
                      "us_per_arrival_step": per * 1e6,
                      "roofline": {"bound": "hbm", "achieved": alg / per / 1e9, "peak": HBM_PEAK_GBS,
                                   "unit": "GB/s", "frac": alg / per / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
                                   "hbm_frac": None if traffic is None else traffic / per / 1e9 / HBM_PEAK_GBS}}
-            if mode == "auto":
-                entry["pulled"] = bool(auto.pulled_steps().any())
-                entry["scatter_max_active"] = auto.scatter_max_active
+            if mode in ("auto", "auto2"):
+                which = auto if mode == "auto" else auto2
+                entry["pulled"] = bool(which.pulled_steps().any())
+                entry["scatter_max_active"] = which.scatter_max_active
             out.append(entry)
     return out
 

@@ -83,6 +83,9 @@ SIGNATURES = {
     "bmtk_csr_propagate_auto_workspace_bytes": (c_int64, [c_int32, c_int64]),
     "bmtk_csr_propagate_auto": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int64, c_int32] +
                                 [c_void_p] * 7 + [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "bmtk_csr_propagate_auto2_workspace_bytes": (c_int64, [c_int32, c_int64]),
+    "bmtk_csr_propagate_auto2": (c_int32, [c_void_p] * 4 + [c_int64, c_void_p, c_int64, c_int32, c_int64, c_int32] +
+                                 [c_void_p] * 7 + [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "bmtk_csr_propagate_pull_workspace_bytes": (c_int64, [c_int32, c_int64]),
     "bmtk_csr_propagate_pull": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
                                           c_int64, c_int64, c_void_p, c_void_p]),

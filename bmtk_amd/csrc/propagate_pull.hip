@@ -48,15 +48,20 @@ __global__ __launch_bounds__(kBlock) void pull_anymap_kernel(const uint64_t *__r
 // the step held by history row (slot_now - d) mod L, d = 0 .. L-1.  One byte answers every question a synapse of
 // that source can ask, whatever its delay and for both arrival steps of pull2_kernel, from an address that is the
 // source itself.
+// `pulled` (bmtk_csr_propagate_auto2), when not null: one word per history row, zero for rows whose spikes were
+// pushed into the ring as events when they occurred -- the pull must not see those.
 __global__ __launch_bounds__(kBlock) void pull_anyrel_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride,
                                                              int L, int batch, int64_t n_src, int slot_now,
-                                                             uint8_t *__restrict__ any_rel)
+                                                             uint8_t *__restrict__ any_rel,
+                                                             const int32_t *__restrict__ pulled)
 {
     const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (j >= n_src) return;
     unsigned m = 0u;
     for (int d = 0; d < L; ++d) {
-        const uint64_t *row = hist + (int64_t)((slot_now + L - d) % L) * hist_stride;
+        const int r = (slot_now + L - d) % L;
+        if (pulled && !pulled[r]) continue;
+        const uint64_t *row = hist + (int64_t)r * hist_stride;
         bool any = false;
         for (int t0 = 0; t0 < batch && !any; t0 += kWave)
             any = source_mask(row, (int)j, batch, t0, min(kWave, batch - t0)) != 0ull;
@@ -229,14 +234,27 @@ constexpr size_t kPull2AccBytes = 2 * kPullAccBytes;
 constexpr size_t kPull2LdsMax = 150u * 1024u;
 // kByteMap: L <= 8 and one byte per source fits the LDS: the activity map is pull_anyrel_kernel's, one LDS read and
 // two shifts per synapse answer both questions (with the bit map: two reads at computed rows).
-template <bool kWords64, bool kByteMap>
+// out_a, out_b: [4][ne] each, the sums of steps t-1 and t.  kAuto (bmtk_csr_propagate_auto2): they are the two
+// steps' ring slots, `ctrl` says which history rows are left to this kernel (with none it returns at once) and
+// which of the two slots already hold what pushed spikes sent there (the sums are then added to the cells).
+template <bool kWords64, bool kByteMap, bool kAuto>
 __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__restrict__ hist, int64_t hist_stride, int L,
                                                            int batch, const int32_t *__restrict__ indptr,
                                                            const bmtk_synapse *__restrict__ packed,
-                                                           float *__restrict__ syn2, int64_t n_tgt, int64_t ne,
-                                                           int slot_now, const uint32_t *__restrict__ any_map, int n_w32)
+                                                           float *__restrict__ out_a, float *__restrict__ out_b,
+                                                           int64_t n_tgt, int64_t ne, int slot_now,
+                                                           const uint32_t *__restrict__ any_map, int n_w32,
+                                                           const int32_t *__restrict__ ctrl)
 {
     extern __shared__ unsigned long long pull_lds[];  // accumulators [wave][step][4][64], stages [wave][step][64], map
+    bool add_a = false, add_b = false;
+    if (kAuto) {
+        int pulled = 0;
+        for (int r = 0; r < L; ++r) pulled |= ctrl[r];
+        if (!pulled) return;
+        add_a = ctrl[kAutoRows + (slot_now + L - 1) % L] != 0;
+        add_b = ctrl[kAutoRows + slot_now] != 0;
+    }
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     constexpr int kWaves = kPullBlock / kWave;
     unsigned long long *acc = pull_lds + wave * (2 * GLIF3_NREC * kWave);
@@ -345,8 +363,14 @@ __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__res
 #pragma unroll
                 for (int r = 0; r < GLIF3_NREC; ++r) {
                     unsigned long long *cell = acc + (k * GLIF3_NREC + r) * kWave + lane;
-                    if ((int)lane < width)
-                        syn2[((int64_t)k * GLIF3_NREC + r) * ne + cb.row * batch + tile0 + lane] = from_fixed(*cell);
+                    if ((int)lane < width) {
+                        float *out = (k ? out_b : out_a) + (int64_t)r * ne + cb.row * batch + tile0 + lane;
+                        const float sum = from_fixed(*cell);
+                        if (kAuto && (k ? add_b : add_a))
+                            *out += sum;
+                        else
+                            *out = sum;
+                    }
                     *cell = 0ull;
                 }
             }
@@ -365,17 +389,20 @@ __global__ __launch_bounds__(kPullBlock) void pull2_kernel(const uint64_t *__res
 // their weights pushed into the ring (fp32 atomics), above it nothing happens here and the step is left to the
 // pull kernel.  One thread records the decision: ctrl[row] = 1 when the history row of the step is to be pulled,
 // and which ring slots hold pushed arrivals (the slot of the step itself, consumed by now, holds none).
+// consumed: how many ring slots the caller has read and cleared since the launch before this one, counted back from
+// slot0 (1 in the one-step form: the step's own slot; in the two-step form 2 for the first of a call's two steps --
+// its own slot and the one before -- and 0 for the second, whose own slot this call is about to complete).
 __global__ __launch_bounds__(kBlock) void auto_push_kernel(const int32_t *__restrict__ active,
                                                            const int32_t *__restrict__ n_active, int batch, Table t,
                                                            float *__restrict__ ring, int L, int64_t ne, int slot0,
-                                                           int cnt_max, int32_t *__restrict__ ctrl)
+                                                           int cnt_max, int32_t *__restrict__ ctrl, int consumed)
 {
     const int n_waves = gridDim.x * (kBlock / kWave);
     const int cnt = *n_active;
     const bool push = cnt <= cnt_max;
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         ctrl[slot0] = push ? 0 : 1;
-        ctrl[kAutoRows + slot0] = 0;
+        for (int c = 0; c < consumed; ++c) ctrl[kAutoRows + (slot0 + L - c) % L] = 0;
         if (push && cnt > 0)
             for (int d = 1; d < L; ++d) ctrl[kAutoRows + (slot0 + d) % L] = 1;
     }
@@ -513,7 +540,7 @@ extern "C" int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_a
         const unsigned grid = (unsigned)((waves + kBlock / kWave - 1) / (kBlock / kWave));
         Table t{src_indptr, src_indices, src_weights, src_delays, src_receptors};
         hipLaunchKernelGGL(auto_push_kernel, dim3(grid), dim3(kBlock), 0, st, active, n_active, batch, t, ring, L, ne, slot0,
-                           (int)scatter_max_active, ctrl);
+                           (int)scatter_max_active, ctrl, 1);
     }
     hipLaunchKernelGGL(auto_anymap_kernel, dim3((unsigned)(((int64_t)n_w32 * 32 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
                        spike_hist + (int64_t)slot0 * hist_stride, batch, n_src, n_w32, any_map + (size_t)slot0 * n_w32,
@@ -557,6 +584,97 @@ extern "C" int bmtk_csr_propagate_auto(const int32_t *active, const int32_t *n_a
     return BMTK_OK;
 }
 
+extern "C" int64_t bmtk_csr_propagate_auto2_workspace_bytes(int32_t L, int64_t n_src)
+{
+    if (L <= 0 || n_src <= 0) return 0;
+    return 2 * bmtk::kAutoRows * 4 + (n_src + 15) / 16 * 16;  // the record of pushed steps, then one byte per source
+}
+
+extern "C" int bmtk_csr_propagate_auto2(const int32_t *active_a, const int32_t *n_active_a, const int32_t *active_b,
+                                        const int32_t *n_active_b, int64_t max_active, const uint64_t *spike_hist,
+                                        int64_t hist_stride, int32_t L, int64_t n_src, int32_t batch,
+                                        const int32_t *src_indptr, const int32_t *src_indices, const float *src_weights,
+                                        const uint8_t *src_delays, const uint8_t *src_receptors,
+                                        const int32_t *tgt_indptr, const bmtk_synapse *tgt_packed, float *ring,
+                                        int64_t n_tgt, int64_t step, int64_t scatter_max_active, void *workspace,
+                                        void *stream)
+{
+    using namespace bmtk;
+    BMTK_REQUIRE(active_a && n_active_a && active_b && n_active_b && spike_hist && ring && workspace,
+                 "csr_propagate_auto2: pointers must be non-null");
+    BMTK_REQUIRE(src_indptr && src_indices && src_weights && src_delays && src_receptors && tgt_indptr && tgt_packed,
+                 "csr_propagate_auto2: both forms of the table are needed");
+    BMTK_REQUIRE(batch > 0 && n_tgt > 0 && n_src > 0 && step >= 1, "csr_propagate_auto2: bad batch, sizes or step");
+    BMTK_REQUIRE(L > 1 && L <= 8, "csr_propagate_auto2: L must lie in 2..8 (longer histories: bmtk_csr_propagate_auto)");
+    BMTK_REQUIRE(hist_stride >= (n_src * (int64_t)batch + 63) / 64 + 1,
+                 "csr_propagate_auto2: hist_stride must hold ceil(n_src*batch/64)+1 words");
+    BMTK_REQUIRE(n_tgt * (int64_t)batch < (1ll << 31) && n_src < (1ll << 24), "csr_propagate_auto2: network too large");
+    BMTK_REQUIRE((int64_t)L * hist_stride < (1ll << 29) && hist_stride < (1ll << 24),
+                 "csr_propagate_auto2: spike history beyond 4 GiB");
+    BMTK_REQUIRE(scatter_max_active >= 0 && scatter_max_active < (1ll << 31) && max_active >= 0,
+                 "csr_propagate_auto2: bad threshold or bound");
+    const int n_16 = (int)((n_src + 15) / 16);
+    const size_t lds = (size_t)n_16 * 16 + kPull2AccBytes;
+    BMTK_REQUIRE(lds <= kPull2LdsMax, "csr_propagate_auto2: n_src too large for the activity map in LDS");
+    hipStream_t st = (hipStream_t)stream;
+    int32_t *ctrl = (int32_t *)workspace;
+    uint8_t *any_rel = (uint8_t *)(ctrl + 2 * kAutoRows);
+    int64_t ne = n_tgt * (int64_t)batch;
+    {   // the two new steps' spikes as events where they are few (each launch records its decision)
+        const int64_t bound = max_active < scatter_max_active ? max_active : scatter_max_active;
+        const int64_t waves = bound < 1 ? 1 : (bound < 8192 ? bound : 8192);
+        const unsigned grid = (unsigned)((waves + kBlock / kWave - 1) / (kBlock / kWave));
+        Table t{src_indptr, src_indices, src_weights, src_delays, src_receptors};
+        hipLaunchKernelGGL(auto_push_kernel, dim3(grid), dim3(kBlock), 0, st, active_a, n_active_a, batch, t, ring, L, ne,
+                           (int)((step - 1) % L), (int)scatter_max_active, ctrl, 2);
+        hipLaunchKernelGGL(auto_push_kernel, dim3(grid), dim3(kBlock), 0, st, active_b, n_active_b, batch, t, ring, L, ne,
+                           (int)(step % L), (int)scatter_max_active, ctrl, 0);
+    }
+    int slot_now = (int)((step + 1) % L);  // the row the spikes of step + 1 will take: it holds step + 1 - L
+    hipLaunchKernelGGL(pull_anyrel_kernel, dim3((unsigned)((n_src + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, spike_hist,
+                       hist_stride, L, batch, n_src, slot_now, any_rel, (const int32_t *)ctrl);
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    static int cu_count[64];
+    int n_cu = (dev >= 0 && dev < 64) ? cu_count[dev] : 0;
+    if (n_cu <= 0) {
+        n_cu = 256;
+        (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        if (dev >= 0 && dev < 64) cu_count[dev] = n_cu;
+    }
+    const unsigned rows_per_block = kPullBlock / kWave;
+    const unsigned want = (unsigned)((n_tgt + rows_per_block - 1) / rows_per_block);
+    const dim3 grid(want < (unsigned)n_cu ? want : (unsigned)n_cu, (unsigned)((batch + kWave - 1) / kWave));
+    BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_auto2: batch too large");
+    const void *kernel = batch == kWave ? reinterpret_cast<const void *>(pull2_kernel<true, true, true>)
+                                        : reinterpret_cast<const void *>(pull2_kernel<false, true, true>);
+    static bool asked[2][64];
+    if (dev >= 0 && dev < 64 && !asked[batch == kWave][dev]) {
+        const hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPull2LdsMax);
+        if (err != hipSuccess) {
+            set_error("csr_propagate_auto2: cannot reserve %zu bytes of LDS: %s", kPull2LdsMax, hipGetErrorString(err));
+            return BMTK_E_LAUNCH;
+        }
+        asked[batch == kWave][dev] = true;
+    }
+    // what the steps not pushed send to steps `step` and `step + 1`, into (or onto) those steps' ring slots
+    float *out_a = ring + (int64_t)(step % L) * GLIF3_NREC * ne, *out_b = ring + (int64_t)slot_now * GLIF3_NREC * ne;
+    const uint32_t *map_arg = (const uint32_t *)any_rel;
+    const int32_t *ctrl_arg = ctrl;
+    int64_t stride_arg = hist_stride;
+    int32_t L_arg = L, batch_arg = batch;
+    int n_map = n_16;
+    void *args[] = {&spike_hist, &stride_arg, &L_arg, &batch_arg, &tgt_indptr, &tgt_packed, &out_a, &out_b, &n_tgt, &ne,
+                    &slot_now, &map_arg, &n_map, &ctrl_arg};
+    const hipError_t err = hipLaunchKernel(kernel, grid, dim3(kPullBlock), args, lds, st);
+    if (err != hipSuccess) {
+        set_error("csr_propagate_auto2: launch failed: %s", hipGetErrorString(err));
+        return BMTK_E_LAUNCH;
+    }
+    BMTK_CHECK_LAUNCH("csr_propagate_auto2");
+    return BMTK_OK;
+}
+
 extern "C" int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist_stride, int32_t L, int64_t n_src,
                                         int32_t batch, const int32_t *indptr, const bmtk_synapse *packed, float *syn2,
                                         int64_t n_tgt, int64_t t_arrive, void *workspace, void *stream)
@@ -581,7 +699,7 @@ extern "C" int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist
     if (byte_map) {
         hipLaunchKernelGGL(pull_anyrel_kernel, dim3((unsigned)((n_src + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                            (hipStream_t)stream, spike_hist, hist_stride, L, batch, n_src, (int)(t_arrive % L),
-                           (uint8_t *)workspace);
+                           (uint8_t *)workspace, (const int32_t *)nullptr);
     } else {
         const int64_t map_threads = (int64_t)L * n_w32 * 32;
         hipLaunchKernelGGL(pull_anymap_kernel, dim3((unsigned)((map_threads + kBlock - 1) / kBlock)), dim3(kBlock), 0,
@@ -601,8 +719,8 @@ extern "C" int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist
     const dim3 grid(want < (unsigned)n_cu ? want : (unsigned)n_cu, (unsigned)((batch + kWave - 1) / kWave));
     BMTK_REQUIRE(grid.y <= 65535, "csr_propagate_pull2: batch too large");
     const void *const kernels[2][2] = {
-        {reinterpret_cast<const void *>(pull2_kernel<false, false>), reinterpret_cast<const void *>(pull2_kernel<false, true>)},
-        {reinterpret_cast<const void *>(pull2_kernel<true, false>), reinterpret_cast<const void *>(pull2_kernel<true, true>)}};
+        {reinterpret_cast<const void *>(pull2_kernel<false, false, false>), reinterpret_cast<const void *>(pull2_kernel<false, true, false>)},
+        {reinterpret_cast<const void *>(pull2_kernel<true, false, false>), reinterpret_cast<const void *>(pull2_kernel<true, true, false>)}};
     const void *kernel = kernels[batch == kWave][byte_map];
     static bool asked[2][2][64];
     if (dev >= 0 && dev < 64 && !asked[batch == kWave][byte_map][dev]) {
@@ -618,7 +736,10 @@ extern "C" int bmtk_csr_propagate_pull2(const uint64_t *spike_hist, int64_t hist
     const uint32_t *map_arg = any_map;
     int64_t stride_arg = hist_stride;
     int32_t L_arg = L, batch_arg = batch;
-    void *args[] = {&spike_hist, &stride_arg, &L_arg, &batch_arg, &indptr, &packed, &syn2, &n_tgt, &ne, &slot_now, &map_arg, &n_map};
+    float *out_a = syn2, *out_b = syn2 + GLIF3_NREC * ne;
+    const int32_t *no_ctrl = nullptr;
+    void *args[] = {&spike_hist, &stride_arg, &L_arg, &batch_arg, &indptr, &packed, &out_a, &out_b, &n_tgt, &ne, &slot_now,
+                    &map_arg, &n_map, &no_ctrl};
     const hipError_t err = hipLaunchKernel(kernel, grid, dim3(kPullBlock), args, lds, (hipStream_t)stream);
     if (err != hipSuccess) {
         set_error("csr_propagate_pull2: launch failed: %s", hipGetErrorString(err));

@@ -223,6 +223,52 @@ def test_two_step_pull_equals_two_pulls(batch, p, n_src, L):
         assert float(one[0].abs().max()) > 0 and not torch.equal(one[0], one[1])
 
 
+@pytest.mark.parametrize("batch,L", [(64, 6), (5, 6), (32, 8), (64, 2), (1, 3)])
+def test_two_step_auto_delivery_equals_the_oracle(batch, L):
+    """``ops.AutoPropagator2`` (bmtk_csr_propagate_auto2): called every second step, each of the two new steps goes
+    out as events or is left to a pull that sums two arrival steps in one pass.  The same run as for the one-step
+    switch -- activity from nothing to 20 % and back, so that pushed and pulled steps mix within and across calls
+    and arrival slots hold pushed weights when the pull adds its sums -- with quarter-pA weights: after every call
+    both arrival slots must equal the fp32 oracle's bit for bit, also with thresholds that force one form."""
+    rng = np.random.default_rng(34 + batch + L)
+    n, T = 500, 40
+    src, tgt, w, d, r = _edges(rng, n, n, 30000, max_delay=L - 1)
+    w = (np.round(w * 4) / 4 + np.sign(w) * 0.25).astype(np.float32)
+    by_src = net.coo_to_csr(src, tgt, w, d, r, n_rows=n, major="source")
+    by_tgt = net.csr_transpose(by_src, n)
+    t_src, t_tgt = ops.SynapseTable.from_numpy(by_src), ops.SynapseTable.from_numpy(by_tgt)
+    ne = n * batch
+    comp_a, comp_b = ops.SpikeCompactor(ne), ops.SpikeCompactor(ne)
+    rates = [0.0, 0.0, 0.002, 0.2, 0.002, 0.0, 0.2, 0.2, 0.01, 0.002, 0.2, 0.0, 0.002] * 4
+    zs = [(rng.random(ne) < rates[k]).astype(np.uint8) for k in range(T)]
+    counts = sorted(int(z.sum()) for z in zs)
+    mid = counts[len(counts) // 2]
+    for thr in (mid, 0, ne, counts[-1] - 1):
+        want = np.zeros((L, 4, ne), np.float32)
+        hist = torch.zeros(L, ops.n_words(ne) + 1, dtype=torch.int64, device="cuda")
+        ring = torch.zeros(L, 4, ne, device="cuda")
+        auto = ops.AutoPropagator2(t_src, t_tgt, hist, ring, n, n, batch, scatter_max_active=thr)
+        seen = set()
+        for k in range(1, T, 2):
+            lists = []
+            for step, comp in ((k - 1, comp_a), (k, comp_b)):
+                orc.gather_rows(zs[step], batch, by_tgt, want, n, step)
+                hist[step % L] = to_dev(bits_of(zs[step]))
+                lists += list(comp(to_dev(zs[step])))
+            auto.step2(k, *lists)
+            pulled = auto.pulled_steps()
+            seen |= {bool(pulled[(k - 1) % L]), bool(pulled[k % L])}
+            for slot in (k % L, (k + 1) % L):
+                np.testing.assert_array_equal(ring[slot].cpu().numpy(), want[slot],
+                                              err_msg="call %d slot %d threshold %d" % (k, slot, thr))
+                ring[slot].zero_()    # the consumer's part: both slots are read and cleared before the next call
+                want[slot] = 0.0
+        if thr == mid:
+            assert seen == {True, False}      # both forms ran
+        elif thr == ne:
+            assert seen == {False}
+
+
 def test_table_from_edges_on_the_device_equals_the_host_build():
     from bmtk_amd import network as net
     rng = np.random.default_rng(5)
