@@ -384,3 +384,37 @@ def test_device_side_switch_at_52k_neurons_batch_64():
         ring_g[slot].zero_()
     assert pulled == [r >= 5.0 for r in rates]
     assert float(ring_g.abs().max()) > 0
+
+def test_two_step_device_side_switch_at_52k_neurons_batch_64():
+    """``bmtk_csr_propagate_auto2`` at the same size and over the same activity as the one-step switch above,
+    called every second step: quiet steps pushed, busy ones pulled, both kinds within one call and across calls.
+    After every call both arrival slots == the slots the deterministic row-wise gather fills, bit for bit."""
+    n, batch, L, T = N52K, 64, 6, 14
+    t_tgt, t_src, _ = _network(n, 120, seed=21)
+    ne = n * batch
+    g = torch.Generator(device="cuda").manual_seed(5)
+    rates = [0.2, 0.2, 20.0, 0.2, 20.0, 20.0, 0.2, 0.2, 0.2, 5.0, 0.2, 20.0, 0.2, 0.2]
+    words = ops.n_words(ne)
+    hist = torch.zeros(L, words + 1, dtype=torch.int64, device="cuda")
+    ring_a = torch.zeros(L, 4, ne, device="cuda")
+    ring_g = torch.zeros(L, 4, ne, device="cuda")
+    comps = (ops.SpikeCompactor(ne), ops.SpikeCompactor(ne))
+    auto = ops.AutoPropagator2(t_src, t_tgt, hist, ring_a, n, n, batch)
+    pulled = {}
+    for k in range(1, T, 2):
+        lists = []
+        for step, comp in ((k - 1, comps[0]), (k, comps[1])):
+            z = (torch.rand(ne, device="cuda", generator=g) < rates[step] * 1e-3)
+            bits = torch.zeros(words + 1, dtype=torch.int64, device="cuda")
+            bits[:-1] = (z.view(-1, 64).to(torch.int64) << torch.arange(64, device="cuda")).sum(1)
+            hist[step % L] = bits
+            lists += list(comp(z.to(torch.uint8)))
+            ops.csr_propagate_gather(bits, n, t_tgt, ring_g, n, batch, step)
+        auto.step2(k, *lists)
+        now = auto.pulled_steps()
+        pulled[k - 1], pulled[k] = bool(now[(k - 1) % L]), bool(now[k % L])
+        for slot in (k % L, (k + 1) % L):
+            assert torch.equal(ring_a[slot], ring_g[slot]), (k, slot)
+            ring_a[slot].zero_()    # the consumer's part: both slots are read and cleared before the next call
+            ring_g[slot].zero_()
+    assert [pulled[k] for k in range(T)] == [r >= 5.0 for r in rates]
