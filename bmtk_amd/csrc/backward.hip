@@ -934,10 +934,7 @@ __global__ __launch_bounds__(kBlock) void bwd_rec_grad_kernel(bmtk_glif3_bwd a, 
 // Input weights.  The events of a step are ascending in source*batch+trial, so the trials in
 // which one source fired are adjacent: the wavefront that holds the first event of such a run
 // takes the whole run, which makes it the only writer of that source's row -- no atomics.
-#ifndef BWD_INP_GRID
-#define BWD_INP_GRID 1024
-#endif
-constexpr int kInpGradGrid = BWD_INP_GRID;
+constexpr int kInpGradGrid = 1024;  // workgroups of the input-gradient part of a launch
 // (a workgroup of any size: wavefront `wave` of `n_waves`)
 __device__ __forceinline__ void bwd_inp_grad_waves(const bmtk_glif3_bwd &a, const BwdStep &q, int wave, int n_waves);
 __device__ __forceinline__ void bwd_inp_grad_block(const bmtk_glif3_bwd &a, const BwdStep &q, int block, int n_blocks)
